@@ -1,0 +1,135 @@
+/*
+ * tinygemma_hip — C ABI of the MI355X (gfx950) implementation of tiny-gemma's int8 weight-only
+ * matrix-product path and of the single-GPU forward built around it.
+ *
+ * Plain pointers and sizes only; no C++ or torch types.  Every entry point returns TG_OK (0) or a
+ * negative TG_ERR_* code; tg_last_error() gives the message of the calling thread's last failure.
+ * The reference reports the same conditions by `assert` abort or std::runtime_error; the C++
+ * mirror in tiny-gemma_amd/host/ turns the codes back into those exceptions.
+ *
+ * One caller thread, one HIP stream (tg_stream()), the library owns all device memory of models
+ * and sessions.  Citations are file:line in the reference checkout.
+ */
+#ifndef TINYGEMMA_HIP_H
+#define TINYGEMMA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+	TG_OK = 0,
+	TG_ERR_UNSUPPORTED_SHAPE = -1, /* static_switch.hpp:28,56: "Unsupported ROW/COL dimension" */
+	TG_ERR_FILE_OPEN = -2,         /* transformer.hpp:163: "Could not open file." */
+	TG_ERR_FILE_SHORT = -3,        /* the reference ignores short reads (transformer.hpp:120-160); this library does not */
+	TG_ERR_BAD_ARG = -4,           /* the reference's assert()s on bs/seq/ndim (ops.hpp:622-646, decode.hpp:78-79) */
+	TG_ERR_HIP = -5,               /* a HIP runtime call failed */
+	TG_ERR_NO_DEVICE = -6,
+	TG_ERR_STATE = -7              /* e.g. a second prefill on a used session (decode.hpp:78-79), context overflow */
+};
+
+typedef struct tg_model tg_model;
+typedef struct tg_session tg_session;
+
+/* config::Config, config.hpp:7-44 */
+typedef struct {
+	int hidden_size;
+	int intermediate_size;
+	int n_layers;
+	int n_vocab;
+	int n_pos;
+	int n_pos_local;
+	int head_dim;
+	int n_head;
+	int n_kv;
+	float rope_theta;
+	float rope_theta_local;
+	int window_pattern;
+} tg_config;
+
+/* ---- library ---- */
+int tg_init(int device);              /* selects the device, creates the stream; idempotent */
+const char *tg_last_error(void);
+const char *tg_status_string(int code);
+void *tg_stream(void);                /* the hipStream_t every kernel of this library is launched on */
+int tg_synchronize(void);
+const char *tg_device_name(void);
+
+/* CONFIG_MAP.at(name), config.hpp:46-48: "270m" or "1B" */
+int tg_config_named(const char *name, tg_config *out);
+
+/* ---- kernel level: host pointers in the reference's layout -------------------------------- */
+/* gemv::launch_qgemv (linalg.hpp:176): C[outDim] must be zero on entry — like the reference it
+ * holds C += A.B, then C *= scales.  B is [inDim][outDim] row-major int8, scales [outDim].
+ * inDim/outDim outside ROW_SWITCH/COL_SWITCH (static_switch.hpp:7-58) -> TG_ERR_UNSUPPORTED_SHAPE. */
+int tg_qgemv(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim);
+/* gemv::launch_qgemv_logits (linalg.hpp:197) */
+int tg_qgemv_logits(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim);
+/* gemm::launch_qgemm (linalg.hpp:298): C[m][outDim] is overwritten. */
+int tg_qgemm(float *C, const float *A, const int8_t *B, const float *scales, int m, int inDim, int outDim);
+
+/* ---- kernel level: device-resident operands (what the forward uses; for timing) ----------- */
+typedef struct tg_qweight tg_qweight;
+/* uploads a reference-layout matrix once (re-tiled for the GPU, values unchanged) */
+int tg_qweight_create(const int8_t *B, const float *scales, int inDim, int outDim, tg_qweight **out);
+void tg_qweight_destroy(tg_qweight *w);
+int tg_dev_alloc(void **p, size_t bytes);
+int tg_dev_free(void *p);
+int tg_copy_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int tg_copy_d2h(void *dst_host, const void *src_dev, size_t bytes);
+/* y_dev[outDim] = scales * (x_dev . W); asynchronous on tg_stream(); overwrites y_dev */
+int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logits_variant);
+/* C_dev[m][outDim] = scales * (A_dev[m][inDim] . W); asynchronous */
+int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m);
+
+/* ---- model level --------------------------------------------------------------------------- */
+/* gemma::Transformer(Config), transformer.hpp:33 */
+int tg_model_create(const tg_config *cfg, tg_model **out);
+/* gemma::read_weights, transformer.hpp:99-165: flat little-endian file, no header */
+int tg_model_load_weights(tg_model *m, const char *path);
+/* same bytes from memory (n must equal tg_weight_file_bytes) */
+int tg_model_load_weights_mem(tg_model *m, const void *image, size_t n);
+size_t tg_weight_file_bytes(const tg_config *cfg);
+void tg_model_destroy(tg_model *m);
+
+/* What gemma::generate builds before the first forward (transformer.hpp:193-202): both RoPE
+ * tables, the GeLU table, the DecodeState (KV caches + counters) and the logits buffer.
+ * Like the reference's forward_* the tables are parameters: pass host arrays to use the caller's
+ * own (rope_*: [n_pos][head_dim] as decode::RoPE holds them, decode.hpp:107-127; gelu_table:
+ * [gelu_size], ops.hpp:22-39) or NULL to have the library compute them. */
+int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin, const float *rope_sw_cos,
+                      const float *rope_sw_sin, const float *gelu_table, float gelu_min, float gelu_max, int gelu_size,
+                      tg_session **out);
+int tg_session_reset(tg_session *s); /* empty KV caches, position 0 */
+void tg_session_destroy(tg_session *s);
+int tg_session_position(const tg_session *s);
+
+/* gemma::forward_prefill (transformer.hpp:49) + ops::argmax_logits (ops.hpp:744).
+ * logits (host, [n_vocab]) and argmax may each be NULL.  Needs an empty session. */
+int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, int32_t *argmax);
+/* gemma::forward_decode (transformer.hpp:75) + argmax */
+int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax);
+/* greedy branch of gemma::generate (transformer.hpp:204-250) without tokenizer/EOS stop:
+ * out_ids gets n_decode+1 ids (the first from the prefill logits); seconds are wall clock around
+ * forward_prefill+argmax and around the decode loop (the tok/s definitions of gemma.cpp:53-58). */
+int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, int32_t *out_ids,
+                       double *s_prefill, double *s_decode);
+/* Enqueues n_steps decode steps without host synchronisation (each step feeds the device-side
+ * argmax of the previous one).  Ids are read back with tg_session_read_ids after tg_synchronize. */
+int tg_decode_enqueue(tg_session *s, int n_steps);
+int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
+
+/* Debug taps: the residual stream of the most recent forward after block b
+ * (b = 0: embedding; 2l+1: after attention of layer l; 2l+2: after the MLP of layer l).
+ * After a prefill `rows` = prompt length, after a decode 1. out is [rows][hidden]. */
+int tg_session_tap(tg_session *s, int b, float *out, int rows);
+/* layer's KV cache as the reference holds it (decode.hpp:14-24): keys/values [max_pos][head_dim] */
+int tg_session_kv(tg_session *s, int layer, float *keys, float *values, int *position_ptr, int *buffer_ptr, int *max_pos);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

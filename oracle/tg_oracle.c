@@ -491,6 +491,7 @@ struct tgo_session {
 	float gmin, gmax;
 	int gsize;
 	kv_cache *kv;
+	int n_layers;
 	float *logits;
 };
 
@@ -535,6 +536,7 @@ tgo_session *tgo_session_create(tgo_model *m, float gmin, float gmax, int gsize)
 	s->gmin = gmin; s->gmax = gmax; s->gsize = gsize;
 	s->table = (float *)malloc(4 * (size_t)gsize);
 	tgo_gelu_table(gmin, gmax, gsize, s->table);
+	s->n_layers = c->n_layers;
 	s->kv = (kv_cache *)calloc((size_t)c->n_layers, sizeof(kv_cache));
 	for (int l = 0; l < c->n_layers; l++) {
 		kv_cache *kv = &s->kv[l];
@@ -549,7 +551,7 @@ tgo_session *tgo_session_create(tgo_model *m, float gmin, float gmax, int gsize)
 
 void tgo_session_destroy(tgo_session *s) {
 	if (!s) return;
-	for (int l = 0; l < s->m->cfg.n_layers; l++) { free(s->kv[l].k); free(s->kv[l].v); }
+	for (int l = 0; l < s->n_layers; l++) { free(s->kv[l].k); free(s->kv[l].v); }
 	free(s->kv); free(s->cos_g); free(s->sin_g); free(s->cos_l); free(s->sin_l); free(s->table); free(s->logits); free(s);
 }
 

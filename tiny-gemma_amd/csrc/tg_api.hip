@@ -1,0 +1,1006 @@
+// C ABI of libtinygemma_hip.so (declared in include/tinygemma_hip.h): library state, weight
+// upload / re-tiling, sessions, and the kernel sequences of forward_prefill / forward_decode.
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <chrono>
+
+#include "tg_internal.h"
+
+// ---------------------------------------------------------------------------------------------
+// library state and errors
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+thread_local std::string g_err;
+bool g_inited = false;
+int g_device = -1;
+hipStream_t g_stream = nullptr;
+char g_devname[256] = "";
+
+// workspace shared by every GEMV launch (launches are serialised on the one stream)
+float *g_ws_partial = nullptr;
+size_t g_ws_partial_floats = 0;
+unsigned *g_ws_counters = nullptr;
+size_t g_ws_counters_n = 0;
+
+bool legal_in(int d) { return d == 640 || d == 2048 || d == 1024 || d == 256 || d == 1152 || d == 6912; }            // static_switch.hpp:7-30
+bool legal_out(int d) { return d == 640 || d == 262144 || d == 2048 || d == 256 || d == 1024 || d == 1152 || d == 6912; }  // :32-58
+
+int ensure_init() {
+	if (g_inited) return TG_OK;
+	return tg_init(0);
+}
+
+int ensure_workspace(size_t partial_floats, size_t counters) {
+	if (partial_floats > g_ws_partial_floats) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		if (g_ws_partial) TG_HIP(hipFree(g_ws_partial));
+		g_ws_partial = nullptr;
+		TG_HIP(hipMalloc((void **)&g_ws_partial, partial_floats * sizeof(float)));
+		g_ws_partial_floats = partial_floats;
+	}
+	if (counters > g_ws_counters_n) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		if (g_ws_counters) TG_HIP(hipFree(g_ws_counters));
+		g_ws_counters = nullptr;
+		TG_HIP(hipMalloc((void **)&g_ws_counters, counters * sizeof(unsigned)));
+		TG_HIP(hipMemset(g_ws_counters, 0, counters * sizeof(unsigned)));
+		g_ws_counters_n = counters;
+	}
+	return TG_OK;
+}
+
+// A matrix on the device in the packed tile layout, with its launch geometry.
+struct PackedMat {
+	int8_t *W = nullptr;
+	float *scales = nullptr;
+	int K = 0, N = 0;   // N = number of (virtual) columns = ntiles * 128
+	int ntiles = 0, tpc = 1, KS = 1, ppb = 0;
+};
+
+void choose_split(PackedMat *p) {
+	const int pairs = p->K / 8;
+	int best = 1;
+	for (int ks = 1; ks <= pairs; ks++) {
+		if (pairs % ks) continue;
+		if (pairs / ks < 4) break;
+		best = ks;
+		if (p->ntiles * ks >= 256) break;
+	}
+	p->KS = best;
+	p->ppb = pairs / best;
+}
+
+// host: [K][N] row-major (leading dimension ld, column order given by colmap or identity) -> packed tiles
+void pack_host(int8_t *dst, const int8_t *src, int K, int N, size_t ld) {
+	const int kgs = K / 4;
+	for (int t = 0; t < N / TG_CT; t++) {
+		for (int kg = 0; kg < kgs; kg++) {
+			const int8_t *r0 = src + (size_t)(4 * kg) * ld + (size_t)t * TG_CT;
+			const int8_t *r1 = r0 + ld, *r2 = r1 + ld, *r3 = r2 + ld;
+			int8_t *d = dst + ((size_t)t * kgs + kg) * TG_CT * 4;
+			for (int c = 0; c < TG_CT; c++) {
+				d[4 * c + 0] = r0[c];
+				d[4 * c + 1] = r1[c];
+				d[4 * c + 2] = r2[c];
+				d[4 * c + 3] = r3[c];
+			}
+		}
+	}
+}
+
+int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_scales, int K, int N, int tpc) {
+	p->K = K;
+	p->N = N;
+	p->ntiles = N / TG_CT;
+	p->tpc = tpc;
+	choose_split(p);
+	std::vector<int8_t> tmp((size_t)K * N);
+	pack_host(tmp.data(), host_rowmajor, K, N, (size_t)N);
+	TG_HIP(hipMalloc((void **)&p->W, (size_t)K * N));
+	TG_HIP(hipMalloc((void **)&p->scales, (size_t)N * sizeof(float)));
+	TG_HIP(hipMemcpy(p->W, tmp.data(), (size_t)K * N, hipMemcpyHostToDevice));
+	TG_HIP(hipMemcpy(p->scales, host_scales, (size_t)N * sizeof(float), hipMemcpyHostToDevice));
+	return ensure_workspace((size_t)p->ntiles * p->KS * TG_CT, (size_t)p->ntiles);
+}
+
+void free_packed(PackedMat *p) {
+	if (p->W) (void)hipFree(p->W);
+	if (p->scales) (void)hipFree(p->scales);
+	p->W = nullptr;
+	p->scales = nullptr;
+}
+
+TgGemv gemv_base(const PackedMat &p) {
+	TgGemv g;
+	memset(&g, 0, sizeof(g));
+	g.W = p.W;
+	g.scales = p.scales;
+	g.K = p.K;
+	g.ntiles = p.ntiles;
+	g.KS = p.KS;
+	g.pairs_per_block = p.ppb;
+	g.tpc = p.tpc;
+	g.partial = g_ws_partial;
+	g.counters = g_ws_counters;
+	return g;
+}
+
+int upload_floats(float **dst, const float *src, size_t n) {
+	TG_HIP(hipMalloc((void **)dst, n * sizeof(float)));
+	TG_HIP(hipMemcpy(*dst, src, n * sizeof(float), hipMemcpyHostToDevice));
+	return TG_OK;
+}
+
+}  // namespace
+
+int tg_fail(int code, const std::string &msg) {
+	g_err = msg;
+	return code;
+}
+
+struct tg_qweight {
+	PackedMat p;
+};
+
+struct LayerDev {
+	PackedMat qkv, o, ug, d;
+	float *rms_q = nullptr, *rms_k = nullptr, *apre = nullptr, *apost = nullptr, *mpre = nullptr, *mpost = nullptr;
+	bool is_sw = false;
+};
+
+struct tg_model {
+	tg_config cfg;
+	bool loaded = false;
+	int8_t *wte = nullptr;  // [vocab][hidden], reference layout (rows are gathered, never streamed)
+	float *wte_scales = nullptr;
+	float *rmsw = nullptr;
+	PackedMat lm;
+	std::vector<LayerDev> L;
+};
+
+struct tg_session {
+	tg_model *m = nullptr;
+	float *cos_g = nullptr, *sin_g = nullptr, *cos_l = nullptr, *sin_l = nullptr;  // [n_pos][head_dim/2]
+	float *lut = nullptr;
+	float gmin = 0, geps = 0;
+	int lut_size = 0;
+	std::vector<float *> kc, vc;
+	std::vector<int> max_pos;
+	float *xr = nullptr;      // [(2L+1)][hidden] residual stream after every block of the last decode
+	float *qkv = nullptr, *attn_out = nullptr, *o_out = nullptr, *hbuf = nullptr, *d_out = nullptr, *logits = nullptr;
+	float *part_acc = nullptr, *part_ml = nullptr;
+	unsigned *attn_counter = nullptr, *argmax_counter = nullptr;
+	float *blk_val = nullptr;
+	int *blk_idx = nullptr;
+	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token
+	int *tok_log = nullptr;
+	int tok_log_cap = 0;
+	int pos = 0, bp_local = 0, bp_global = 0, steps = 0;  // host mirrors
+	float *taps = nullptr;    // prefill taps [(2L+1)][rows][hidden] (kept only for short prompts)
+	int tap_rows = 0;
+};
+
+namespace {
+constexpr int ATTN_MAX_BLOCKS = 256;
+constexpr int PREFILL_TAP_MAX_ROWS = 1024;
+
+bool layer_is_local(const tg_config &c, int l) { return (l % c.window_pattern) != (c.window_pattern - 1); }  // transformer.hpp:43
+
+int check_config(const tg_config *c) {
+	if (!c) return tg_fail(TG_ERR_BAD_ARG, "null config");
+	if (c->head_dim != 256 || c->n_head != 4 || c->n_kv != 1)
+		return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "attention kernels are built for 4 query heads, 1 KV head, head_dim 256 (config.hpp:47-48)");
+	if (!legal_in(c->hidden_size) || !legal_out(c->hidden_size))
+		return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported ROW dimension: " + std::to_string(c->hidden_size));
+	if (!legal_in(c->intermediate_size) || !legal_out(c->intermediate_size))
+		return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported COL dimension: " + std::to_string(c->intermediate_size));
+	if (!legal_out(c->n_vocab)) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported COL dimension: " + std::to_string(c->n_vocab));
+	if (c->hidden_size > 1152) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "hidden_size above 1152");
+	if (c->n_layers < 1 || c->n_pos < 1 || c->n_pos_local < 1 || c->window_pattern < 1) return tg_fail(TG_ERR_BAD_ARG, "bad config");
+	return TG_OK;
+}
+}  // namespace
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------
+// library
+// ---------------------------------------------------------------------------------------------
+int tg_init(int device) {
+	if (g_inited) {
+		if (device != g_device) return tg_fail(TG_ERR_BAD_ARG, "already initialised on another device");
+		return TG_OK;
+	}
+	int n = 0;
+	if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return tg_fail(TG_ERR_NO_DEVICE, "no HIP device");
+	if (device < 0 || device >= n) return tg_fail(TG_ERR_NO_DEVICE, "no such device");
+	TG_HIP(hipSetDevice(device));
+	hipDeviceProp_t prop;
+	TG_HIP(hipGetDeviceProperties(&prop, device));
+	snprintf(g_devname, sizeof(g_devname), "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+	TG_HIP(hipStreamCreate(&g_stream));
+	g_device = device;
+	g_inited = true;
+	return TG_OK;
+}
+
+const char *tg_last_error(void) { return g_err.c_str(); }
+
+const char *tg_status_string(int code) {
+	switch (code) {
+		case TG_OK: return "ok";
+		case TG_ERR_UNSUPPORTED_SHAPE: return "unsupported dimension";
+		case TG_ERR_FILE_OPEN: return "Could not open file.";
+		case TG_ERR_FILE_SHORT: return "weight file shorter than the configuration requires";
+		case TG_ERR_BAD_ARG: return "bad argument";
+		case TG_ERR_HIP: return "HIP runtime error";
+		case TG_ERR_NO_DEVICE: return "no HIP device";
+		case TG_ERR_STATE: return "session state does not allow this call";
+		default: return "unknown";
+	}
+}
+
+void *tg_stream(void) { return (void *)g_stream; }
+
+int tg_synchronize(void) {
+	if (ensure_init() != TG_OK) return TG_ERR_NO_DEVICE;
+	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+
+const char *tg_device_name(void) {
+	if (ensure_init() != TG_OK) return "";
+	return g_devname;
+}
+
+int tg_config_named(const char *name, tg_config *out) {
+	if (!name || !out) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	tg_config c = {0, 0, 0, 262144, 32768, 512, 256, 4, 1, 1000000.0f, 10000.0f, 6};  // config.hpp:46-48
+	if (strcmp(name, "270m") == 0) {
+		c.hidden_size = 640; c.intermediate_size = 2048; c.n_layers = 18;
+	} else if (strcmp(name, "1B") == 0) {
+		c.hidden_size = 1152; c.intermediate_size = 6912; c.n_layers = 26;
+	} else {
+		return tg_fail(TG_ERR_BAD_ARG, std::string("unknown model size: ") + name);
+	}
+	*out = c;
+	return TG_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------------------------
+int tg_dev_alloc(void **p, size_t bytes) {
+	if (int rc = ensure_init()) return rc;
+	TG_HIP(hipMalloc(p, bytes));
+	return TG_OK;
+}
+int tg_dev_free(void *p) {
+	TG_HIP(hipFree(p));
+	return TG_OK;
+}
+int tg_copy_h2d(void *dst, const void *src, size_t bytes) {
+	TG_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+int tg_copy_d2h(void *dst, const void *src, size_t bytes) {
+	TG_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// kernel level
+// ---------------------------------------------------------------------------------------------
+int tg_qweight_create(const int8_t *B, const float *scales, int inDim, int outDim, tg_qweight **out) {
+	if (int rc = ensure_init()) return rc;
+	if (!B || !scales || !out) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (!legal_in(inDim)) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported ROW dimension: " + std::to_string(inDim));
+	if (!legal_out(outDim)) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported COL dimension: " + std::to_string(outDim));
+	tg_qweight *w = new tg_qweight();
+	int rc = upload_packed(&w->p, B, scales, inDim, outDim, 1);
+	if (rc != TG_OK) {
+		free_packed(&w->p);
+		delete w;
+		return rc;
+	}
+	*out = w;
+	return TG_OK;
+}
+
+void tg_qweight_destroy(tg_qweight *w) {
+	if (!w) return;
+	(void)hipStreamSynchronize(g_stream);
+	free_packed(&w->p);
+	delete w;
+}
+
+int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logits_variant) {
+	(void)logits_variant;  // one kernel serves both reference variants (they differ only in rounding order)
+	if (!y_dev || !x_dev || !w) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	TgGemv g = gemv_base(w->p);
+	g.pro = TG_PRO_PLAIN;
+	g.x = x_dev;
+	g.epi = TG_EPI_STORE;
+	g.y = y_dev;
+	tg_launch_gemv(g, g_stream);
+	TG_HIP(hipGetLastError());
+	return TG_OK;
+}
+
+int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
+	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	tg_launch_gemm(C_dev, A_dev, w->p.W, w->p.scales, m, w->p.K, w->p.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+	TG_HIP(hipGetLastError());
+	return TG_OK;
+}
+
+static int qgemv_host(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim, int variant) {
+	if (int rc = ensure_init()) return rc;
+	if (!C || !A || !B || !scales) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	tg_qweight *w = nullptr;
+	int rc = tg_qweight_create(B, scales, inDim, outDim, &w);
+	if (rc != TG_OK) return rc;
+	float *x = nullptr, *y = nullptr;
+	std::vector<float> yh((size_t)outDim);
+	rc = tg_dev_alloc((void **)&x, sizeof(float) * inDim);
+	if (rc == TG_OK) rc = tg_dev_alloc((void **)&y, sizeof(float) * outDim);
+	if (rc == TG_OK) rc = tg_copy_h2d(x, A, sizeof(float) * inDim);
+	if (rc == TG_OK) rc = tg_qgemv_dev(y, x, w, variant);
+	if (rc == TG_OK) rc = tg_copy_d2h(yh.data(), y, sizeof(float) * outDim);
+	if (x) (void)hipFree(x);
+	if (y) (void)hipFree(y);
+	tg_qweight_destroy(w);
+	if (rc != TG_OK) return rc;
+	// The reference accumulates into C and then scales C (linalg.hpp:52-107); with the required
+	// zero C this is the plain product.  A non-zero C is carried through the same way.
+	for (int c = 0; c < outDim; c++) C[c] = C[c] * scales[c] + yh[c];
+	return TG_OK;
+}
+
+int tg_qgemv(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim) {
+	return qgemv_host(C, A, B, scales, inDim, outDim, 0);
+}
+int tg_qgemv_logits(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim) {
+	return qgemv_host(C, A, B, scales, inDim, outDim, 1);
+}
+
+int tg_qgemm(float *C, const float *A, const int8_t *B, const float *scales, int m, int inDim, int outDim) {
+	if (int rc = ensure_init()) return rc;
+	if (!C || !A || !B || !scales || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	tg_qweight *w = nullptr;
+	int rc = tg_qweight_create(B, scales, inDim, outDim, &w);
+	if (rc != TG_OK) return rc;
+	float *a = nullptr, *c = nullptr;
+	rc = tg_dev_alloc((void **)&a, sizeof(float) * (size_t)m * inDim);
+	if (rc == TG_OK) rc = tg_dev_alloc((void **)&c, sizeof(float) * (size_t)m * outDim);
+	if (rc == TG_OK) rc = tg_copy_h2d(a, A, sizeof(float) * (size_t)m * inDim);
+	if (rc == TG_OK) rc = tg_qgemm_dev(c, a, w, m);
+	if (rc == TG_OK) rc = tg_copy_d2h(C, c, sizeof(float) * (size_t)m * outDim);
+	if (a) (void)hipFree(a);
+	if (c) (void)hipFree(c);
+	tg_qweight_destroy(w);
+	return rc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// model
+// ---------------------------------------------------------------------------------------------
+size_t tg_weight_file_bytes(const tg_config *c) {
+	if (!c) return 0;
+	const size_t h = c->hidden_size, f = c->intermediate_size, V = c->n_vocab, hd = c->head_dim;
+	const size_t qo = (size_t)c->n_head * hd, kv = (size_t)c->n_kv * hd;
+	size_t per_layer = h * qo + 4 * qo + 2 * (h * kv + 4 * kv) + qo * h + 4 * h + 2 * 4 * hd + 2 * 4 * h + 2 * (h * f + 4 * f) +
+	                   f * h + 4 * h + 2 * 4 * h;
+	return V * h + 4 * h + 4 * h + per_layer * (size_t)c->n_layers + h * V + 4 * V;
+}
+
+int tg_model_create(const tg_config *cfg, tg_model **out) {
+	if (int rc = ensure_init()) return rc;
+	if (!out) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (int rc = check_config(cfg)) return rc;
+	tg_model *m = new tg_model();
+	m->cfg = *cfg;
+	m->L.resize((size_t)cfg->n_layers);
+	for (int l = 0; l < cfg->n_layers; l++) m->L[(size_t)l].is_sw = layer_is_local(*cfg, l);
+	*out = m;
+	return TG_OK;
+}
+
+static void model_free_weights(tg_model *m) {
+	(void)hipStreamSynchronize(g_stream);
+	if (m->wte) (void)hipFree(m->wte);
+	if (m->wte_scales) (void)hipFree(m->wte_scales);
+	if (m->rmsw) (void)hipFree(m->rmsw);
+	m->wte = nullptr; m->wte_scales = nullptr; m->rmsw = nullptr;
+	free_packed(&m->lm);
+	for (auto &L : m->L) {
+		free_packed(&L.qkv); free_packed(&L.o); free_packed(&L.ug); free_packed(&L.d);
+		float **ps[] = {&L.rms_q, &L.rms_k, &L.apre, &L.apost, &L.mpre, &L.mpost};
+		for (float **p : ps) {
+			if (*p) (void)hipFree(*p);
+			*p = nullptr;
+		}
+	}
+	m->loaded = false;
+}
+
+void tg_model_destroy(tg_model *m) {
+	if (!m) return;
+	model_free_weights(m);
+	delete m;
+}
+
+}  // extern "C"
+
+// Walks the flat file in the order of transformer.hpp:122-160 through `rd`.
+template <typename Reader>
+static int load_weights_impl(tg_model *m, Reader rd) {
+	const tg_config &c = m->cfg;
+	const int h = c.hidden_size, f = c.intermediate_size, V = c.n_vocab, hd = c.head_dim;
+	const int qo = c.n_head * hd, kv = c.n_kv * hd;
+	model_free_weights(m);
+	std::vector<int8_t> buf, buf2, cat;
+	std::vector<float> sc, sc2, catsc, fl;
+	int rc;
+	auto read_i8 = [&](std::vector<int8_t> &v, size_t n) { v.resize(n); return rd(v.data(), n); };
+	auto read_f = [&](std::vector<float> &v, size_t n) { v.resize(n); return rd(v.data(), n * 4); };
+	auto read_dev_f = [&](float **dst, size_t n) -> int {
+		if (int r = read_f(fl, n)) return r;
+		return upload_floats(dst, fl.data(), n);
+	};
+	// wte + scales, final norm
+	if ((rc = read_i8(buf, (size_t)V * h))) return rc;
+	TG_HIP(hipMalloc((void **)&m->wte, (size_t)V * h));
+	TG_HIP(hipMemcpy(m->wte, buf.data(), (size_t)V * h, hipMemcpyHostToDevice));
+	if ((rc = read_dev_f(&m->wte_scales, (size_t)h))) return rc;
+	if ((rc = read_dev_f(&m->rmsw, (size_t)h))) return rc;
+	for (int l = 0; l < c.n_layers; l++) {
+		LayerDev &L = m->L[(size_t)l];
+		// Q | K | V fused along the output dimension: [h][qo + 2 kv]
+		const int nq = qo + 2 * kv;
+		cat.assign((size_t)h * nq, 0);
+		catsc.assign((size_t)nq, 0.0f);
+		int col = 0;
+		for (int part = 0; part < 3; part++) {
+			const int n = part == 0 ? qo : kv;
+			if ((rc = read_i8(buf, (size_t)h * n))) return rc;
+			if ((rc = read_f(sc, (size_t)n))) return rc;
+			for (int r = 0; r < h; r++) memcpy(&cat[(size_t)r * nq + col], &buf[(size_t)r * n], (size_t)n);
+			memcpy(&catsc[(size_t)col], sc.data(), sizeof(float) * (size_t)n);
+			col += n;
+		}
+		if ((rc = upload_packed(&L.qkv, cat.data(), catsc.data(), h, nq, 1))) return rc;
+		// O
+		if ((rc = read_i8(buf, (size_t)qo * h))) return rc;
+		if ((rc = read_f(sc, (size_t)h))) return rc;
+		if ((rc = upload_packed(&L.o, buf.data(), sc.data(), qo, h, 1))) return rc;
+		if ((rc = read_dev_f(&L.rms_q, (size_t)hd))) return rc;
+		if ((rc = read_dev_f(&L.rms_k, (size_t)hd))) return rc;
+		if ((rc = read_dev_f(&L.apre, (size_t)h))) return rc;
+		if ((rc = read_dev_f(&L.apost, (size_t)h))) return rc;
+		// up | gate fused tile by tile: virtual tile 2t = up columns [128t, 128t+128), 2t+1 = the same gate columns
+		if ((rc = read_i8(buf, (size_t)h * f))) return rc;
+		if ((rc = read_f(sc, (size_t)f))) return rc;
+		if ((rc = read_i8(buf2, (size_t)h * f))) return rc;
+		if ((rc = read_f(sc2, (size_t)f))) return rc;
+		cat.assign((size_t)h * 2 * f, 0);
+		catsc.assign((size_t)2 * f, 0.0f);
+		for (int t = 0; t < f / TG_CT; t++) {
+			for (int r = 0; r < h; r++) {
+				memcpy(&cat[(size_t)r * 2 * f + (size_t)(2 * t) * TG_CT], &buf[(size_t)r * f + (size_t)t * TG_CT], TG_CT);
+				memcpy(&cat[(size_t)r * 2 * f + (size_t)(2 * t + 1) * TG_CT], &buf2[(size_t)r * f + (size_t)t * TG_CT], TG_CT);
+			}
+			memcpy(&catsc[(size_t)(2 * t) * TG_CT], &sc[(size_t)t * TG_CT], sizeof(float) * TG_CT);
+			memcpy(&catsc[(size_t)(2 * t + 1) * TG_CT], &sc2[(size_t)t * TG_CT], sizeof(float) * TG_CT);
+		}
+		if ((rc = upload_packed(&L.ug, cat.data(), catsc.data(), h, 2 * f, 2))) return rc;
+		// down
+		if ((rc = read_i8(buf, (size_t)f * h))) return rc;
+		if ((rc = read_f(sc, (size_t)h))) return rc;
+		if ((rc = upload_packed(&L.d, buf.data(), sc.data(), f, h, 1))) return rc;
+		if ((rc = read_dev_f(&L.mpre, (size_t)h))) return rc;
+		if ((rc = read_dev_f(&L.mpost, (size_t)h))) return rc;
+	}
+	if ((rc = read_i8(buf, (size_t)h * V))) return rc;
+	if ((rc = read_f(sc, (size_t)V))) return rc;
+	if ((rc = upload_packed(&m->lm, buf.data(), sc.data(), h, V, 1))) return rc;
+	m->loaded = true;
+	return TG_OK;
+}
+
+extern "C" {
+
+int tg_model_load_weights(tg_model *m, const char *path) {
+	if (!m || !path) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	FILE *fp = fopen(path, "rb");
+	if (!fp) return tg_fail(TG_ERR_FILE_OPEN, "Could not open file.");  // transformer.hpp:163
+	int rc = load_weights_impl(m, [&](void *dst, size_t n) -> int {
+		if (fread(dst, 1, n, fp) != n) return tg_fail(TG_ERR_FILE_SHORT, "weight file is shorter than the configuration requires");
+		return TG_OK;
+	});
+	fclose(fp);
+	if (rc != TG_OK) model_free_weights(m);
+	return rc;
+}
+
+int tg_model_load_weights_mem(tg_model *m, const void *image, size_t n) {
+	if (!m || !image) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (n != tg_weight_file_bytes(&m->cfg)) return tg_fail(TG_ERR_FILE_SHORT, "image size does not match the configuration");
+	const uint8_t *p = (const uint8_t *)image;
+	size_t off = 0;
+	int rc = load_weights_impl(m, [&](void *dst, size_t k) -> int {
+		if (off + k > n) return tg_fail(TG_ERR_FILE_SHORT, "image too short");
+		memcpy(dst, p + off, k);
+		off += k;
+		return TG_OK;
+	});
+	if (rc != TG_OK) model_free_weights(m);
+	return rc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// session
+// ---------------------------------------------------------------------------------------------
+static int upload_rope(float **cos_d, float **sin_d, const float *cos_h, const float *sin_h, float theta, int n_pos, int hd) {
+	const int half = hd / 2;
+	std::vector<float> c((size_t)n_pos * half), s((size_t)n_pos * half);
+	if (cos_h && sin_h) {
+		// decode::RoPE keeps [n_pos][hd] with both halves equal (decode.hpp:190-200): keep one half
+		for (int p = 0; p < n_pos; p++)
+			for (int d = 0; d < half; d++) {
+				c[(size_t)p * half + d] = cos_h[(size_t)p * hd + d];
+				s[(size_t)p * half + d] = sin_h[(size_t)p * hd + d];
+			}
+	} else {
+		// decode.hpp:176-201: freq_i = 1/pow(theta, 2i/hd) and angle = p*freq in fp32;
+		// cos/sin of that fp32 angle, correctly rounded
+		std::vector<float> freqs((size_t)half);
+		for (int i = 0; i < half; i++) freqs[(size_t)i] = 1.0f / powf(theta, (float)(2 * i) / (float)hd);
+		for (int p = 0; p < n_pos; p++)
+			for (int d = 0; d < half; d++) {
+				const float ang = (float)p * freqs[(size_t)d];
+				c[(size_t)p * half + d] = (float)cos((double)ang);
+				s[(size_t)p * half + d] = (float)sin((double)ang);
+			}
+	}
+	if (int rc = upload_floats(cos_d, c.data(), c.size())) return rc;
+	return upload_floats(sin_d, s.data(), s.size());
+}
+
+void tg_session_destroy(tg_session *s) {
+	if (!s) return;
+	(void)hipStreamSynchronize(g_stream);
+	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
+	              s->logits, s->part_acc, s->part_ml, s->attn_counter, s->argmax_counter, s->blk_val, s->blk_idx, s->ctr,
+	              s->tok_log, s->taps};
+	for (void *p : ps)
+		if (p) (void)hipFree(p);
+	for (float *p : s->kc)
+		if (p) (void)hipFree(p);
+	for (float *p : s->vc)
+		if (p) (void)hipFree(p);
+	delete s;
+}
+
+int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin, const float *rope_sw_cos,
+                      const float *rope_sw_sin, const float *gelu_table, float gelu_min, float gelu_max, int gelu_size,
+                      tg_session **out) {
+	if (!m || !out) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (!m->loaded) return tg_fail(TG_ERR_STATE, "model has no weights");
+	if (gelu_size < 1 || !(gelu_max > gelu_min)) return tg_fail(TG_ERR_BAD_ARG, "bad GeLU table range");
+	const tg_config &c = m->cfg;
+	tg_session *s = new tg_session();
+	s->m = m;
+	int rc = TG_OK;
+	auto fail = [&](int code) {
+		tg_session_destroy(s);
+		return code;
+	};
+	if ((rc = upload_rope(&s->cos_g, &s->sin_g, rope_cos, rope_sin, c.rope_theta, c.n_pos, c.head_dim))) return fail(rc);
+	if ((rc = upload_rope(&s->cos_l, &s->sin_l, rope_sw_cos, rope_sw_sin, c.rope_theta_local, c.n_pos, c.head_dim))) return fail(rc);
+	// lut::GeLUTable, ops.hpp:29-39
+	s->gmin = gelu_min;
+	s->geps = (float)(gelu_max - gelu_min) / (float)gelu_size;
+	s->lut_size = gelu_size;
+	{
+		std::vector<float> t((size_t)gelu_size);
+		if (gelu_table) {
+			memcpy(t.data(), gelu_table, sizeof(float) * (size_t)gelu_size);
+		} else {
+			const float c0 = 0.7978845608f, c1 = 0.044715f;
+			for (int i = 0; i < gelu_size; i++) {
+				const float x = gelu_min + (float)i * s->geps;
+				const double a = (double)x;
+				t[(size_t)i] = (float)((0.5 * a) * (1.0 + tanh((double)c0 * (a + (double)c1 * (a * a * a)))));
+			}
+		}
+		if ((rc = upload_floats(&s->lut, t.data(), t.size()))) return fail(rc);
+	}
+	const int L = c.n_layers, h = c.hidden_size, hd = c.head_dim, qo = c.n_head * hd;
+	s->kc.assign((size_t)L, nullptr);
+	s->vc.assign((size_t)L, nullptr);
+	s->max_pos.assign((size_t)L, 0);
+	for (int l = 0; l < L; l++) {
+		const int mp = m->L[(size_t)l].is_sw ? c.n_pos_local : c.n_pos;  // decode.hpp:30
+		s->max_pos[(size_t)l] = mp;
+		const size_t bytes = sizeof(float) * (size_t)mp * hd;
+		if (hipMalloc((void **)&s->kc[(size_t)l], bytes) != hipSuccess || hipMalloc((void **)&s->vc[(size_t)l], bytes) != hipSuccess)
+			return fail(tg_fail(TG_ERR_HIP, "KV cache allocation failed"));
+	}
+	s->tok_log_cap = c.n_pos + 1;
+#define TG_ALLOC(ptr, bytes)                                                                         \
+	if (hipMalloc((void **)&(ptr), (bytes)) != hipSuccess) return fail(tg_fail(TG_ERR_HIP, "session allocation failed: " #ptr))
+	TG_ALLOC(s->xr, sizeof(float) * (size_t)(2 * L + 1) * h);
+	TG_ALLOC(s->qkv, sizeof(float) * (size_t)(qo + 2 * hd));
+	TG_ALLOC(s->attn_out, sizeof(float) * (size_t)qo);
+	TG_ALLOC(s->o_out, sizeof(float) * (size_t)h);
+	TG_ALLOC(s->hbuf, sizeof(float) * (size_t)c.intermediate_size);
+	TG_ALLOC(s->d_out, sizeof(float) * (size_t)h);
+	TG_ALLOC(s->logits, sizeof(float) * (size_t)c.n_vocab);
+	TG_ALLOC(s->part_acc, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * hd);
+	TG_ALLOC(s->part_ml, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * 2);
+	TG_ALLOC(s->attn_counter, sizeof(unsigned));
+	TG_ALLOC(s->argmax_counter, sizeof(unsigned));
+	TG_ALLOC(s->blk_val, sizeof(float) * (size_t)m->lm.ntiles);
+	TG_ALLOC(s->blk_idx, sizeof(int) * (size_t)m->lm.ntiles);
+	TG_ALLOC(s->ctr, sizeof(int) * 8);
+	TG_ALLOC(s->tok_log, sizeof(int) * (size_t)s->tok_log_cap);
+#undef TG_ALLOC
+	if ((rc = tg_session_reset(s))) return fail(rc);
+	*out = s;
+	return TG_OK;
+}
+
+int tg_session_reset(tg_session *s) {
+	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	const tg_config &c = s->m->cfg;
+	TG_HIP(hipStreamSynchronize(g_stream));
+	for (size_t l = 0; l < s->kc.size(); l++) {
+		const size_t bytes = sizeof(float) * (size_t)s->max_pos[l] * c.head_dim;
+		TG_HIP(hipMemset(s->kc[l], 0, bytes));
+		TG_HIP(hipMemset(s->vc[l], 0, bytes));
+	}
+	TG_HIP(hipMemset(s->ctr, 0, sizeof(int) * 8));
+	TG_HIP(hipMemset(s->attn_counter, 0, sizeof(unsigned)));
+	TG_HIP(hipMemset(s->argmax_counter, 0, sizeof(unsigned)));
+	TG_HIP(hipMemset(s->xr, 0, sizeof(float) * (size_t)(2 * c.n_layers + 1) * c.hidden_size));
+	TG_HIP(hipDeviceSynchronize());
+	s->pos = s->bp_local = s->bp_global = s->steps = 0;
+	if (s->taps) {
+		TG_HIP(hipFree(s->taps));
+		s->taps = nullptr;
+	}
+	s->tap_rows = 0;
+	return TG_OK;
+}
+
+int tg_session_position(const tg_session *s) { return s ? s->pos : -1; }
+
+// ---------------------------------------------------------------------------------------------
+// forward_decode: 5 launches per layer + 1 for the head
+// ---------------------------------------------------------------------------------------------
+static int attn_chunk_for(int valid) {
+	int c = 16;
+	while (c < 256 && (valid + c - 1) / c > 128) c *= 2;
+	return c;
+}
+
+static int enqueue_decode_step(tg_session *s, bool want_logits) {
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	const int L = c.n_layers, h = c.hidden_size, hd = c.head_dim;
+	if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
+	if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
+	for (int l = 0; l < L; l++) {
+		const LayerDev &Ld = m->L[(size_t)l];
+		// --- pre-norm + Q|K|V (modules.hpp:137-144); folds the previous block's post-norm + residual
+		TgGemv g = gemv_base(Ld.qkv);
+		g.hidden = h;
+		g.w_pre = Ld.apre;
+		g.xr_out = s->xr + (size_t)(2 * l) * h;
+		if (l == 0) {
+			g.pro = TG_PRO_EMBED;
+			g.wte = m->wte;
+			g.wte_scales = m->wte_scales;
+			g.tok = s->ctr + 4;
+			g.vocab = c.n_vocab;
+			g.emb_scale = (float)sqrt((double)h);  // ops.hpp:586
+		} else {
+			g.pro = TG_PRO_RESNORM;
+			g.pend = s->d_out;
+			g.w_post = m->L[(size_t)l - 1].mpost;
+			g.x = s->xr + (size_t)(2 * l - 1) * h;
+		}
+		g.epi = TG_EPI_STORE;
+		g.y = s->qkv;
+		tg_launch_gemv(g, g_stream);
+		// --- q/k norm, RoPE, KV write, attention (modules.hpp:146-161)
+		TgAttnDecode a;
+		memset(&a, 0, sizeof(a));
+		a.qkv = s->qkv;
+		a.rms_q = Ld.rms_q;
+		a.rms_k = Ld.rms_k;
+		a.cos_t = Ld.is_sw ? s->cos_l : s->cos_g;
+		a.sin_t = Ld.is_sw ? s->sin_l : s->sin_g;
+		a.kc = s->kc[(size_t)l];
+		a.vc = s->vc[(size_t)l];
+		a.max_pos = s->max_pos[(size_t)l];
+		a.pos = s->ctr;
+		a.bp_index = Ld.is_sw ? 1 : 2;
+		const int valid = std::min(s->pos + 1, a.max_pos);
+		a.chunk = attn_chunk_for(valid);
+		a.part_acc = s->part_acc;
+		a.part_ml = s->part_ml;
+		a.counter = s->attn_counter;
+		a.out = s->attn_out;
+		a.n_head = c.n_head;
+		tg_launch_attn_decode(a, (valid + a.chunk - 1) / a.chunk, g_stream);
+		// --- O projection (modules.hpp:163-164)
+		g = gemv_base(Ld.o);
+		g.pro = TG_PRO_PLAIN;
+		g.x = s->attn_out;
+		g.epi = TG_EPI_STORE;
+		g.y = s->o_out;
+		tg_launch_gemv(g, g_stream);
+		// --- post-norm + residual, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
+		g = gemv_base(Ld.ug);
+		g.pro = TG_PRO_RESNORM;
+		g.hidden = h;
+		g.pend = s->o_out;
+		g.w_post = Ld.apost;
+		g.x = s->xr + (size_t)(2 * l) * h;
+		g.xr_out = s->xr + (size_t)(2 * l + 1) * h;
+		g.w_pre = Ld.mpre;
+		g.epi = TG_EPI_GEGLU;
+		g.y = s->hbuf;
+		g.lut = s->lut;
+		g.gmin = s->gmin;
+		g.geps = s->geps;
+		g.lut_size = s->lut_size;
+		tg_launch_gemv(g, g_stream);
+		// --- down projection (modules.hpp:216-217)
+		g = gemv_base(Ld.d);
+		g.pro = TG_PRO_PLAIN;
+		g.x = s->hbuf;
+		g.epi = TG_EPI_STORE;
+		g.y = s->d_out;
+		tg_launch_gemv(g, g_stream);
+	}
+	// --- last post-norm + residual, final norm, LM head, argmax (modules.hpp:242-246, ops.hpp:744)
+	TgGemv g = gemv_base(m->lm);
+	g.pro = TG_PRO_RESNORM;
+	g.hidden = h;
+	g.pend = s->d_out;
+	g.w_post = m->L[(size_t)L - 1].mpost;
+	g.x = s->xr + (size_t)(2 * L - 1) * h;
+	g.xr_out = s->xr + (size_t)(2 * L) * h;
+	g.w_pre = m->rmsw;
+	g.epi = TG_EPI_LOGITS;
+	g.y = want_logits ? s->logits : nullptr;
+	g.blk_val = s->blk_val;
+	g.blk_idx = s->blk_idx;
+	g.argmax_counter = s->argmax_counter;
+	g.tok_out = s->ctr + 4;
+	g.tok_log = s->tok_log;
+	g.step = s->ctr + 3;
+	g.pos = s->ctr;
+	tg_launch_gemv(g, g_stream);
+	TG_HIP(hipGetLastError());
+	s->pos += 1;
+	s->bp_local += 1;
+	s->bp_global += 1;
+	s->steps += 1;
+	(void)hd;
+	return TG_OK;
+}
+
+int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax) {
+	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	TG_HIP(hipMemcpyAsync(s->ctr + 4, &id, sizeof(int), hipMemcpyHostToDevice, g_stream));
+	if (int rc = enqueue_decode_step(s, logits != nullptr)) return rc;
+	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)s->m->cfg.n_vocab, hipMemcpyDeviceToHost, g_stream));
+	int32_t tok = -1;
+	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
+	if (argmax) *argmax = tok;
+	if (s->taps) {  // taps now describe the decode step
+		(void)hipFree(s->taps);
+		s->taps = nullptr;
+		s->tap_rows = 0;
+	}
+	return TG_OK;
+}
+
+int tg_decode_enqueue(tg_session *s, int n_steps) {
+	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	for (int i = 0; i < n_steps; i++)
+		if (int rc = enqueue_decode_step(s, false)) return rc;
+	if (s->taps) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		(void)hipFree(s->taps);
+		s->taps = nullptr;
+		s->tap_rows = 0;
+	}
+	return TG_OK;
+}
+
+int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out) {
+	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	TG_HIP(hipStreamSynchronize(g_stream));
+	const int n = std::min(max_ids, s->steps);
+	if (n > 0) TG_HIP(hipMemcpy(ids, s->tok_log, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
+	if (n_out) *n_out = n;
+	return TG_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_prefill
+// ---------------------------------------------------------------------------------------------
+int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, int32_t *argmax) {
+	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	if (n < 1) return tg_fail(TG_ERR_BAD_ARG, "empty prompt");
+	if (s->pos != 0) return tg_fail(TG_ERR_STATE, "prefill needs an empty session (decode.hpp:78-79)");
+	if (n > c.n_pos) return tg_fail(TG_ERR_STATE, "prompt longer than n_pos");
+	const int L = c.n_layers, h = c.hidden_size, f = c.intermediate_size, hd = c.head_dim;
+	const int qo = c.n_head * hd, nq = qo + 2 * hd;
+	const size_t S = (size_t)n;
+	int *d_ids = nullptr;
+	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr;
+	auto cleanup = [&]() {
+		void *ps[] = {d_ids, x, xn, qkv, ao, t, hb};
+		for (void *p : ps)
+			if (p) (void)hipFree(p);
+	};
+#define TG_TRY(expr)                                                                             \
+	do {                                                                                         \
+		hipError_t e_ = (expr);                                                                  \
+		if (e_ != hipSuccess) {                                                                  \
+			cleanup();                                                                           \
+			return tg_fail(TG_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));       \
+		}                                                                                        \
+	} while (0)
+	TG_TRY(hipMalloc((void **)&d_ids, sizeof(int) * S));
+	TG_TRY(hipMalloc((void **)&x, sizeof(float) * S * h));
+	TG_TRY(hipMalloc((void **)&xn, sizeof(float) * S * h));
+	TG_TRY(hipMalloc((void **)&qkv, sizeof(float) * S * nq));
+	TG_TRY(hipMalloc((void **)&ao, sizeof(float) * S * qo));
+	TG_TRY(hipMalloc((void **)&t, sizeof(float) * S * h));
+	TG_TRY(hipMalloc((void **)&hb, sizeof(float) * S * f));
+	const bool keep_taps = n <= PREFILL_TAP_MAX_ROWS;
+	if (s->taps) {
+		(void)hipFree(s->taps);
+		s->taps = nullptr;
+		s->tap_rows = 0;
+	}
+	if (keep_taps) {
+		TG_TRY(hipMalloc((void **)&s->taps, sizeof(float) * (size_t)(2 * L + 1) * S * h));
+		s->tap_rows = n;
+	}
+	auto tap = [&](int b) -> hipError_t {
+		if (!keep_taps) return hipSuccess;
+		return hipMemcpyAsync(s->taps + (size_t)b * S * h, x, sizeof(float) * S * h, hipMemcpyDeviceToDevice, g_stream);
+	};
+	TG_TRY(hipMemcpyAsync(d_ids, ids, sizeof(int) * S, hipMemcpyHostToDevice, g_stream));
+	tg_launch_embed_rows(x, d_ids, n, m->wte, m->wte_scales, h, c.n_vocab, g_stream);
+	TG_TRY(tap(0));
+	// xn = rmsnorm(x, attn_pre of layer 0)
+	tg_launch_norm_rows(xn, x, m->L[0].apre, nullptr, nullptr, nullptr, n, h, g_stream);
+	for (int l = 0; l < L; l++) {
+		const LayerDev &Ld = m->L[(size_t)l];
+		const int mp = s->max_pos[(size_t)l];
+		// Q|K|V (modules.hpp:106-108)
+		tg_launch_gemm(qkv, xn, Ld.qkv.W, Ld.qkv.scales, n, h, Ld.qkv.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
+		tg_launch_qk_norm_rope_rows(qkv, qkv + qo, qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
+		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
+		                            g_stream);
+		// attention (modules.hpp:123): local layers use sw_context = max_pos
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, g_stream);
+		// O (modules.hpp:127-128)
+		tg_launch_gemm(t, ao, Ld.o.W, Ld.o.scales, n, qo, Ld.o.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
+		tg_launch_norm_rows(xn, t, Ld.mpre, Ld.apost, x, x, n, h, g_stream);
+		TG_TRY(tap(2 * l + 1));
+		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
+		tg_launch_gemm(hb, xn, Ld.ug.W, Ld.ug.scales, n, h, Ld.ug.ntiles, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, g_stream);
+		tg_launch_gemm(t, hb, Ld.d.W, Ld.d.scales, n, f, Ld.d.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
+		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
+		tg_launch_norm_rows(xn, t, next_pre, Ld.mpost, x, x, n, h, g_stream);
+		TG_TRY(tap(2 * l + 2));
+	}
+	// LM head on the last position only (modules.hpp:232-240): xn already holds rmsnorm(x, RMSw)
+	{
+		TgGemv g = gemv_base(m->lm);
+		g.pro = TG_PRO_PLAIN;
+		g.x = xn + (S - 1) * h;
+		g.epi = TG_EPI_LOGITS;
+		g.y = logits ? s->logits : nullptr;
+		g.blk_val = s->blk_val;
+		g.blk_idx = s->blk_idx;
+		g.argmax_counter = s->argmax_counter;
+		g.tok_out = s->ctr + 4;
+		g.tok_log = s->tok_log;
+		g.step = s->ctr + 3;
+		g.pos = nullptr;
+		tg_launch_gemv(g, g_stream);
+	}
+	TG_TRY(hipGetLastError());
+	// KVCache::update_prefill's counters (decode.hpp:99-104)
+	s->pos = n;
+	s->bp_local = (n >= c.n_pos_local) ? c.n_pos_local : n;
+	s->bp_global = (n >= c.n_pos) ? c.n_pos : n;
+	s->steps = 1;
+	int ctr[3] = {s->pos, s->bp_local, s->bp_global};
+	TG_TRY(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
+	if (logits) TG_TRY(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)c.n_vocab, hipMemcpyDeviceToHost, g_stream));
+	int32_t tok = -1;
+	TG_TRY(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
+	TG_TRY(hipStreamSynchronize(g_stream));
+	if (argmax) *argmax = tok;
+	cleanup();
+#undef TG_TRY
+	return TG_OK;
+}
+
+int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, int32_t *out_ids, double *s_prefill,
+                       double *s_decode) {
+	if (!s || !prompt || !out_ids || n_decode < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	using clk = std::chrono::steady_clock;
+	auto t0 = clk::now();
+	int32_t tok = -1;
+	if (int rc = tg_forward_prefill(s, prompt, n_prompt, nullptr, &tok)) return rc;
+	auto t1 = clk::now();
+	if (int rc = tg_decode_enqueue(s, n_decode)) return rc;
+	int got = 0;
+	if (int rc = tg_session_read_ids(s, out_ids, n_decode + 1, &got)) return rc;
+	auto t2 = clk::now();
+	if (s_prefill) *s_prefill = std::chrono::duration<double>(t1 - t0).count();
+	if (s_decode) *s_decode = std::chrono::duration<double>(t2 - t1).count();
+	return got == n_decode + 1 ? TG_OK : tg_fail(TG_ERR_STATE, "token log incomplete");
+}
+
+// ---------------------------------------------------------------------------------------------
+// debug taps
+// ---------------------------------------------------------------------------------------------
+int tg_session_tap(tg_session *s, int b, float *out, int rows) {
+	if (!s || !out) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	const tg_config &c = s->m->cfg;
+	if (b < 0 || b > 2 * c.n_layers) return tg_fail(TG_ERR_BAD_ARG, "no such block");
+	TG_HIP(hipStreamSynchronize(g_stream));
+	const size_t h = (size_t)c.hidden_size;
+	if (s->taps) {
+		if (rows != s->tap_rows) return tg_fail(TG_ERR_BAD_ARG, "rows must equal the prompt length");
+		TG_HIP(hipMemcpy(out, s->taps + (size_t)b * s->tap_rows * h, sizeof(float) * (size_t)rows * h, hipMemcpyDeviceToHost));
+	} else {
+		if (rows != 1) return tg_fail(TG_ERR_BAD_ARG, "decode taps have one row");
+		TG_HIP(hipMemcpy(out, s->xr + (size_t)b * h, sizeof(float) * h, hipMemcpyDeviceToHost));
+	}
+	return TG_OK;
+}
+
+int tg_session_kv(tg_session *s, int layer, float *keys, float *values, int *position_ptr, int *buffer_ptr, int *max_pos) {
+	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	const tg_config &c = s->m->cfg;
+	if (layer < 0 || layer >= c.n_layers) return tg_fail(TG_ERR_BAD_ARG, "no such layer");
+	TG_HIP(hipStreamSynchronize(g_stream));
+	const size_t bytes = sizeof(float) * (size_t)s->max_pos[(size_t)layer] * c.head_dim;
+	if (keys) TG_HIP(hipMemcpy(keys, s->kc[(size_t)layer], bytes, hipMemcpyDeviceToHost));
+	if (values) TG_HIP(hipMemcpy(values, s->vc[(size_t)layer], bytes, hipMemcpyDeviceToHost));
+	if (position_ptr) *position_ptr = s->pos;
+	if (buffer_ptr) *buffer_ptr = s->m->L[(size_t)layer].is_sw ? s->bp_local : s->bp_global;
+	if (max_pos) *max_pos = s->max_pos[(size_t)layer];
+	return TG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,323 @@
+// Attention over the fp32 KV cache, plus the per-token work the reference does between the
+// Q/K/V projections and the attention itself (modules.hpp:146-159): per-head RMSNorm of q and k,
+// half-rotation RoPE, and the KV-cache write.
+//
+//   decode : ops::attention_decode (ops.hpp:224-370) — one query token, 4 heads sharing 1 KV head,
+//            keys = the valid slots of a ring (local layers) or linear (global layers) cache.
+//            The reference walks the slots sequentially with a renormalising online softmax; here
+//            the slots are split across workgroups (flash-decoding), each computing an exact
+//            softmax partial (max, sum, unnormalised output) over its chunk, merged by the last
+//            workgroup to finish.  Softmax is order independent, so only fp32 rounding differs.
+//   prefill: ops::attention_prefill (ops.hpp:377-526) — causal; local layers see keys
+//            qs-window .. qs inclusive (window+1 keys, ops.hpp:437-443).
+
+#include "tg_internal.h"
+
+namespace {
+
+constexpr int HD = 256;        // head_dim (config.hpp:47-48); checked on the host
+constexpr int NH = 4;          // query heads sharing the single KV head
+constexpr int ANT = 256;       // threads per workgroup
+constexpr int MAXCHUNK = 256;  // keys per workgroup, upper bound
+
+__device__ __forceinline__ float wsum(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+	return v;
+}
+__device__ __forceinline__ float wmax(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+	return v;
+}
+__device__ __forceinline__ float sum16(float v) {  // over aligned groups of 16 lanes
+#pragma unroll
+	for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+	return v;
+}
+
+// One wave normalises and rotates one 256-wide head vector (ops.hpp:126-180, decode.hpp:136-211).
+// Lane l owns dims {l, l+64, l+128, l+192}: both members of every rotation pair (d, d+128).
+// cs/sn point at the [hd/2] table row of this token's position.
+__device__ __forceinline__ void norm_rope_head(const float *src, const float *w, const float *cs, const float *sn, float mul,
+                                               float out[4], int lane) {
+	float x[4];
+#pragma unroll
+	for (int i = 0; i < 4; i++) x[i] = src[lane + 64 * i];
+	float ss = 0.0f;
+#pragma unroll
+	for (int i = 0; i < 4; i++) ss = fmaf(x[i], x[i], ss);
+	ss = wsum(ss);
+	const float irms = 1.0f / sqrtf(ss / (float)HD + 1e-06f);
+#pragma unroll
+	for (int i = 0; i < 4; i++) x[i] = (x[i] * irms) * (w[lane + 64 * i] + 1.0f);
+	const float c0 = cs[lane], c1 = cs[lane + 64], s0 = sn[lane], s1 = sn[lane + 64];
+	out[0] = fmaf(c0, x[0], (-x[2]) * s0) * mul;
+	out[1] = fmaf(c1, x[1], (-x[3]) * s1) * mul;
+	out[2] = fmaf(c0, x[2], x[0] * s0) * mul;
+	out[3] = fmaf(c1, x[3], x[1] * s1) * mul;
+}
+
+// scores of keys [k0, k0+n) against the 4 query heads in qs (already scaled by 1/sqrt(hd)).
+// 16 lanes share one key row (coalesced 256-byte pieces); sc[h][j-k0] receives q_h . k_j.
+// Key rows are ldk floats apart.  Slot `cur` is taken from knew (the token being decoded is not
+// in the cache yet).
+__device__ __forceinline__ void chunk_scores(const float (*qs)[HD], const float *kc, int ldk, const float *knew, int cur, int k0,
+                                             int n, float (*sc)[MAXCHUNK], int tid) {
+	const int lane = tid & 63, w = tid >> 6, sub = lane >> 4, sl = lane & 15;
+	float4 q[NH][4];
+#pragma unroll
+	for (int h = 0; h < NH; h++)
+#pragma unroll
+		for (int i = 0; i < 4; i++) q[h][i] = *reinterpret_cast<const float4 *>(&qs[h][i * 64 + sl * 4]);
+	for (int base = 0; base < n; base += 16) {
+		const int jj = base + w * 4 + sub;
+		const bool ok = jj < n;
+		const int j = k0 + (ok ? jj : 0);
+		const float *kr = (j == cur) ? knew : kc + (size_t)j * ldk;
+		float4 kv[4];
+#pragma unroll
+		for (int i = 0; i < 4; i++) kv[i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
+#pragma unroll
+		for (int h = 0; h < NH; h++) {
+			float d = 0.0f;
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				d = fmaf(q[h][i].x, kv[i].x, d);
+				d = fmaf(q[h][i].y, kv[i].y, d);
+				d = fmaf(q[h][i].z, kv[i].z, d);
+				d = fmaf(q[h][i].w, kv[i].w, d);
+			}
+			d = sum16(d);
+			if (ok && sl == 0) sc[h][jj] = d;
+		}
+	}
+}
+
+__global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) {
+	__shared__ float qs[NH][HD];
+	__shared__ float knew[HD], vnew[HD];
+	__shared__ float sc[NH][MAXCHUNK];
+	__shared__ float s_m[NH], s_l[NH];
+	__shared__ unsigned s_ticket;
+
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int pos = a.pos[0];                      // position_ptr before this token (decode.hpp:154)
+	const int bp = a.pos[a.bp_index];           // buffer_ptr before this token (decode.hpp:59)
+	const int cur = bp % a.max_pos;
+	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;  // decode.hpp:45-47 after update_single
+	const int nb = (valid + a.chunk - 1) / a.chunk;
+	const int b = blockIdx.x;
+	if (b >= nb) return;
+
+	// q heads: one wave each; k: wave 0 again
+	{
+		const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
+		float o[4];
+		norm_rope_head(a.qkv + w * HD, a.rms_q, cs, sn, 0.0625f, o, lane);  // ops.hpp:257: q *= 1/sqrt(256)
+#pragma unroll
+		for (int i = 0; i < 4; i++) qs[w][lane + 64 * i] = o[i];
+		if (w == 0) {
+			norm_rope_head(a.qkv + NH * HD, a.rms_k, cs, sn, 1.0f, o, lane);
+#pragma unroll
+			for (int i = 0; i < 4; i++) knew[lane + 64 * i] = o[i];
+		}
+		vnew[tid] = a.qkv[NH * HD + HD + tid];
+	}
+	__syncthreads();
+	if (b == 0) {  // KVCache::update_single, decode.hpp:49-70
+		a.kc[(size_t)cur * HD + tid] = knew[tid];
+		a.vc[(size_t)cur * HD + tid] = vnew[tid];
+	}
+
+	const int k0 = b * a.chunk;
+	const int n = (valid - k0 < a.chunk) ? valid - k0 : a.chunk;
+	chunk_scores(qs, a.kc, HD, knew, cur, k0, n, sc, tid);
+	__syncthreads();
+
+	// softmax statistics of this chunk: wave h owns head h
+	{
+		float m = -INFINITY;
+		for (int j = lane; j < n; j += 64) m = fmaxf(m, sc[w][j]);
+		m = wmax(m);
+		float l = 0.0f;
+		for (int j = lane; j < n; j += 64) {
+			const float p = expf(sc[w][j] - m);
+			sc[w][j] = p;
+			l += p;
+		}
+		l = wsum(l);
+		if (lane == 0) { s_m[w] = m; s_l[w] = l; }
+	}
+	__syncthreads();
+
+	// P.V: thread = output dim, 4 heads
+	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
+	for (int j0 = 0; j0 < n; j0 += 8) {
+		float vv[8];
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			const int jj = j0 + u;
+			const int j = k0 + (jj < n ? jj : 0);
+			vv[u] = (j == cur) ? vnew[tid] : a.vc[(size_t)j * HD + tid];
+		}
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			if (j0 + u < n) {
+#pragma unroll
+				for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][j0 + u], vv[u], acc[h]);
+			}
+		}
+	}
+
+	if (nb == 1) {
+#pragma unroll
+		for (int h = 0; h < NH; h++) a.out[h * HD + tid] = acc[h] / s_l[h];
+		return;
+	}
+#pragma unroll
+	for (int h = 0; h < NH; h++) a.part_acc[((size_t)b * NH + h) * HD + tid] = acc[h];
+	if (tid < NH) {
+		a.part_ml[((size_t)b * NH + tid) * 2 + 0] = s_m[tid];
+		a.part_ml[((size_t)b * NH + tid) * 2 + 1] = s_l[tid];
+	}
+	__threadfence();
+	__syncthreads();
+	if (tid == 0) s_ticket = atomicAdd(a.counter, 1u);
+	__syncthreads();
+	if (s_ticket != (unsigned)(nb - 1)) return;
+	__threadfence();
+	// merge: O = sum_b acc_b * exp(m_b - M) / sum_b l_b * exp(m_b - M)
+#pragma unroll
+	for (int h = 0; h < NH; h++) {
+		float M = -INFINITY;
+		for (int i = 0; i < nb; i++) M = fmaxf(M, __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2));
+		float L = 0.0f, O = 0.0f;
+		for (int i = 0; i < nb; i++) {
+			const float mi = __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2);
+			const float li = __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2 + 1);
+			const float e = expf(mi - M);
+			L = fmaf(li, e, L);
+			O = fmaf(__builtin_nontemporal_load(a.part_acc + ((size_t)i * NH + h) * HD + tid), e, O);
+		}
+		a.out[h * HD + tid] = O / L;
+	}
+	if (tid == 0) *a.counter = 0u;
+}
+
+// ---------------------------------------------------------------------------------------------
+// prefill
+// ---------------------------------------------------------------------------------------------
+
+// One workgroup per prompt position: q heads and k normalised + rotated in place
+// (modules.hpp:115-119), k/v rows of the last min(S, max_pos) positions copied to cache slots
+// 0.. (KVCache::update_prefill, decode.hpp:72-105).
+__global__ __launch_bounds__(ANT) void qk_norm_rope_rows_kernel(float *q, float *k, const float *v, const float *rms_q,
+                                                                const float *rms_k, const float *cos_t, const float *sin_t,
+                                                                float *kc, float *vc, int max_pos, int S, int ldq, int ldkv) {
+	const int s = blockIdx.x, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const float *cs = cos_t + (size_t)s * (HD / 2), *sn = sin_t + (size_t)s * (HD / 2);
+	float o[4];
+	float *qrow = q + (size_t)s * ldq + w * HD;
+	norm_rope_head(qrow, rms_q, cs, sn, 1.0f, o, lane);
+#pragma unroll
+	for (int i = 0; i < 4; i++) qrow[lane + 64 * i] = o[i];
+	const int start = (S >= max_pos) ? S - max_pos : 0;
+	float *krow = k + (size_t)s * ldkv;
+	if (w == 0) {
+		norm_rope_head(krow, rms_k, cs, sn, 1.0f, o, lane);
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			krow[lane + 64 * i] = o[i];
+			if (s >= start) kc[(size_t)(s - start) * HD + lane + 64 * i] = o[i];
+		}
+	}
+	if (s >= start) vc[(size_t)(s - start) * HD + tid] = v[(size_t)s * ldkv + tid];
+}
+
+// One workgroup per query position, all 4 heads; keys streamed in chunks with a running
+// (max, sum, acc) per head.  q rows are [S][ldq] with head h at column h*256; k, v rows [S][ldkv].
+__global__ __launch_bounds__(ANT) void attn_prefill_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
+                                                           int ldkv, int ldo, int is_sw, int window) {
+	__shared__ float qs[NH][HD];
+	__shared__ float sc[NH][MAXCHUNK];
+	__shared__ float s_m[NH], s_l[NH], s_c[NH];
+
+	const int qi = blockIdx.x, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+#pragma unroll
+	for (int h = 0; h < NH; h++) qs[h][tid] = q[(size_t)qi * ldq + h * HD + tid] * 0.0625f;  // ops.hpp:406,463
+	if (tid < NH) { s_m[tid] = -INFINITY; s_l[tid] = 0.0f; }
+	__syncthreads();
+	int kbeg = 0;
+	if (is_sw) kbeg = (qi >= window) ? qi - window : 0;  // ops.hpp:437-441
+	const int kend = qi + 1;
+	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
+	for (int k0 = kbeg; k0 < kend; k0 += MAXCHUNK) {
+		const int n = (kend - k0 < MAXCHUNK) ? kend - k0 : MAXCHUNK;
+		chunk_scores(qs, k, ldkv, nullptr, -1, k0, n, sc, tid);
+		__syncthreads();
+		{
+			float m = -INFINITY;
+			for (int j = lane; j < n; j += 64) m = fmaxf(m, sc[w][j]);
+			m = wmax(m);
+			const float m_old = s_m[w];
+			const float m_new = fmaxf(m_old, m);
+			float l = 0.0f;
+			for (int j = lane; j < n; j += 64) {
+				const float p = expf(sc[w][j] - m_new);
+				sc[w][j] = p;
+				l += p;
+			}
+			l = wsum(l);
+			if (lane == 0) {
+				const float c = expf(m_old - m_new);  // 0 on the first chunk
+				s_c[w] = c;
+				s_l[w] = fmaf(s_l[w], c, l);
+				s_m[w] = m_new;
+			}
+		}
+		__syncthreads();
+#pragma unroll
+		for (int h = 0; h < NH; h++) acc[h] *= s_c[h];
+		for (int j0 = 0; j0 < n; j0 += 8) {
+			float vv[8];
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				const int jj = j0 + u;
+				vv[u] = v[(size_t)(k0 + (jj < n ? jj : 0)) * ldkv + tid];
+			}
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				if (j0 + u < n) {
+#pragma unroll
+					for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][j0 + u], vv[u], acc[h]);
+				}
+			}
+		}
+		__syncthreads();
+	}
+#pragma unroll
+	for (int h = 0; h < NH; h++) o[(size_t)qi * ldo + h * HD + tid] = acc[h] / s_l[h];
+}
+
+}  // namespace
+
+void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s) {
+	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)max_blocks), dim3(ANT), 0, s, a);
+}
+
+void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
+                                 const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
+                                 hipStream_t s) {
+	(void)n_head;
+	(void)hd;
+	hipLaunchKernelGGL(qk_norm_rope_rows_kernel, dim3((unsigned)S), dim3(ANT), 0, s, q, k, v, rms_q, rms_k, cos_t, sin_t, kc, vc,
+	                   max_pos, S, ldq, ldkv);
+}
+
+void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
+                            int ldo, int is_sw, int window, hipStream_t s) {
+	(void)n_head;
+	(void)hd;
+	hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)S), dim3(ANT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window);
+}

@@ -1,0 +1,172 @@
+// Row-wise prefill kernels (one workgroup per prompt position) and the prefill GEMM.
+//
+//   embed_rows : ops::embedding_prefill (ops.hpp:529-571)
+//   norm_rows  : ops::rmsnorm on [S][dim] (ops.hpp:126-222), optionally preceded by the
+//                "post-norm the block output, add the residual" step of modules.hpp:130-132, 199-201
+//   gemm       : gemm::launch_qgemm (linalg.hpp:210-308): C = (A . W) * scales, C overwritten.
+//                This version keeps the reference's arithmetic exactly — one fused multiply-add
+//                chain per output element over k = 0..K-1 in fp32 (linalg.hpp:215-235) — on the
+//                vector ALUs, reading the packed int8 tiles directly.
+
+#include "tg_internal.h"
+
+namespace {
+
+constexpr int RNT = 256;
+
+__device__ __forceinline__ float wsum(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+	return v;
+}
+
+__device__ __forceinline__ float bsum(float v, float *sred) {
+	v = wsum(v);
+	__syncthreads();
+	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
+	__syncthreads();
+	return (sred[0] + sred[1]) + (sred[2] + sred[3]);
+}
+
+__device__ __forceinline__ float b2f(int d, int j) { return (float)(int8_t)(d >> (8 * j)); }
+
+__device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin, float geps, int size) {
+	int idx = (int)((x - gmin) / geps);
+	if (idx < 0) return 0.0f;
+	if (idx >= size) return x;
+	return lut[idx];
+}
+
+__global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *ids, const int8_t *wte, const float *scales,
+                                                         int hidden, int vocab, float emb_scale) {
+	const int s = blockIdx.x;
+	int tok = ids[s];
+	tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+	const int8_t *row = wte + (size_t)tok * hidden;
+	for (int d = threadIdx.x; d < hidden; d += RNT) x[(size_t)s * hidden + d] = scales[d] * (emb_scale * (float)row[d]);
+}
+
+__global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *w_pre, const float *w_post,
+                                                        const float *resid, float *resid_out, int dim) {
+	__shared__ float xs[1152];
+	__shared__ float sred[4];
+	const int s = blockIdx.x, tid = threadIdx.x;
+	const float eps = 1e-06f;
+	const float *row = in + (size_t)s * dim;
+	float ss = 0.0f;
+	for (int d = tid; d < dim; d += RNT) {
+		float p = row[d];
+		xs[d] = p;
+		ss = fmaf(p, p, ss);
+	}
+	ss = bsum(ss, sred);
+	if (resid != nullptr) {
+		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
+		float s2 = 0.0f;
+		for (int d = tid; d < dim; d += RNT) {
+			float t = (xs[d] * irms) * (w_post[d] + 1.0f) + resid[(size_t)s * dim + d];
+			xs[d] = t;
+			resid_out[(size_t)s * dim + d] = t;
+			s2 = fmaf(t, t, s2);
+		}
+		ss = bsum(s2, sred);
+	}
+	if (out != nullptr) {
+		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
+		for (int d = tid; d < dim; d += RNT) out[(size_t)s * dim + d] = (xs[d] * irms) * (w_pre[d] + 1.0f);
+	}
+}
+
+// 64 rows x 128 columns per workgroup; thread (ty = tid/32, tx = tid%32) owns rows ty*8..+7 and
+// columns tx*4..+3 of the tile.  For the fused up|gate matrix (epi GEGLU) the workgroup walks the
+// tile pair (2t, 2t+1) and writes gelu(gate) * up.
+template <int EPI>
+__global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *A, const int8_t *Wp, const float *scales, int m,
+                                                         int K, int ntiles, const float *lut, float gmin, float geps, int lut_size) {
+	constexpr int NTILE = (EPI == TG_EPI_GEGLU) ? 2 : 1;
+	const int tid = threadIdx.x, tx = tid & 31, ty = tid >> 5;
+	const int row0 = blockIdx.y * 64 + ty * 8;
+	const int kgs = K >> 2;
+	float acc[NTILE][8][4];
+#pragma unroll
+	for (int t = 0; t < NTILE; t++)
+#pragma unroll
+		for (int r = 0; r < 8; r++)
+#pragma unroll
+			for (int c = 0; c < 4; c++) acc[t][r][c] = 0.0f;
+	const float *arow[8];
+#pragma unroll
+	for (int r = 0; r < 8; r++) arow[r] = A + (size_t)((row0 + r < m) ? row0 + r : m - 1) * K;
+
+	for (int kg = 0; kg < kgs; kg++) {
+		float4 av[8];
+#pragma unroll
+		for (int r = 0; r < 8; r++) av[r] = *reinterpret_cast<const float4 *>(arow[r] + 4 * kg);
+#pragma unroll
+		for (int t = 0; t < NTILE; t++) {
+			const int tile = blockIdx.x * NTILE + t;
+			const uint4 wv = *(reinterpret_cast<const uint4 *>(Wp) + ((size_t)tile * kgs + kg) * (TG_CT / 4) + tx);
+			const int d[4] = {(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
+#pragma unroll
+			for (int c = 0; c < 4; c++) {
+				const float w0 = b2f(d[c], 0), w1 = b2f(d[c], 1), w2 = b2f(d[c], 2), w3 = b2f(d[c], 3);
+#pragma unroll
+				for (int r = 0; r < 8; r++) {
+					float a = acc[t][r][c];
+					a = fmaf(av[r].x, w0, a);
+					a = fmaf(av[r].y, w1, a);
+					a = fmaf(av[r].z, w2, a);
+					a = fmaf(av[r].w, w3, a);
+					acc[t][r][c] = a;
+				}
+			}
+		}
+	}
+	const int N = ntiles * TG_CT;
+#pragma unroll
+	for (int r = 0; r < 8; r++) {
+		if (row0 + r >= m) continue;
+		if (EPI == TG_EPI_GEGLU) {
+			const int cu = (blockIdx.x * 2) * TG_CT + tx * 4, cg = cu + TG_CT;
+			float4 o;
+			float *op = &o.x;
+#pragma unroll
+			for (int c = 0; c < 4; c++) {
+				const float up = acc[0][r][c] * scales[cu + c];
+				const float gate = acc[NTILE - 1][r][c] * scales[cg + c];
+				op[c] = gelu_lut(gate, lut, gmin, geps, lut_size) * up;
+			}
+			*reinterpret_cast<float4 *>(C + (size_t)(row0 + r) * (N / 2) + blockIdx.x * TG_CT + tx * 4) = o;
+		} else {
+			const int c0 = blockIdx.x * TG_CT + tx * 4;
+			float4 o = make_float4(acc[0][r][0] * scales[c0], acc[0][r][1] * scales[c0 + 1], acc[0][r][2] * scales[c0 + 2],
+			                       acc[0][r][3] * scales[c0 + 3]);
+			*reinterpret_cast<float4 *>(C + (size_t)(row0 + r) * N + c0) = o;
+		}
+	}
+}
+
+}  // namespace
+
+void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,
+                          hipStream_t s) {
+	const float emb_scale = (float)sqrt((double)hidden);  // ops.hpp:537
+	hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, x, ids, wte, scales, hidden, vocab, emb_scale);
+}
+
+void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
+                         int S, int dim, hipStream_t s) {
+	hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, out, in, w_pre, w_post, resid, resid_out, dim);
+}
+
+void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int epi,
+                    const float *lut, float gmin, float geps, int lut_size, hipStream_t s) {
+	dim3 block(RNT);
+	if (epi == TG_EPI_GEGLU) {
+		dim3 grid((unsigned)(ntiles / 2), (unsigned)((m + 63) / 64));
+		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_GEGLU>, grid, block, 0, s, C, A, Wp, scales, m, K, ntiles, lut, gmin, geps, lut_size);
+	} else {
+		dim3 grid((unsigned)ntiles, (unsigned)((m + 63) / 64));
+		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_STORE>, grid, block, 0, s, C, A, Wp, scales, m, K, ntiles, lut, gmin, geps, lut_size);
+	}
+}
