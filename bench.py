@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the int8 weight-only path on one MI355X.
+
+A step is one greedy decode token (forward_decode + argmax) of a Gemma-3-1B-shaped model with
+random-init weights, after a 178-token random prompt has been prefilled: the workload the
+reference's README quotes its decode tok/s on (1024-token completions, mean prompt 178 tokens).
+Weights, KV cache and the prompt are resident in HBM before the timed region; nothing crosses
+PCIe inside it (each step feeds the device-side argmax of the previous one).
+
+Prints one JSON line.  `roofline` is for the dominant kernel of a step, the LM-head GEMV
+(tg_gemv_lmhead_argmax: 1152 x 262144 int8 + scales + x + logits = 304,091,648 algorithmic
+bytes per launch), timed with HIP events on the library's stream during real decode steps.
+`cpu_baseline` times the reference's single-threaded AVX2 path (oracle/_ref, built from the
+reference's own sources) — or, where that library is absent, the scalar C restatement — on
+this machine's host cores over a bounded sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as ge  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+
+MODELS = {
+    # name: (prompt tokens, decode bytes of weights+scales per token, LM-head GEMV algorithmic bytes)
+    "1B": (178, 1_002_637_312, 304_091_648),
+    "270m": (64, 269_588_480, 169_871_872),
+}
+
+
+class HipEvents:
+    """hipEvent timing on a given stream through libamdhip64 (torch's events only see torch's stream)."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+
+    def create(self):
+        e = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.hip.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, e0, e1):
+        assert self.hip.hipEventSynchronize(e1) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), e0, e1) == 0
+        return float(ms.value)
+
+
+def cpu_baseline(image_path, cfg_name, prompt, n_decode):
+    """Decode tok/s of the CPU path on one core: prefill the same prompt, then n_decode greedy steps."""
+    orc = ge.load_oracle()
+    cfg = orc.named_config(cfg_name)
+    if orc.Ref.available():
+        kind, sess_model = "reference", orc.Ref().model(cfg, image_path)
+    else:
+        kind, sess_model = "port", orc.Oracle().model(cfg, path=image_path)
+    sess = sess_model.session()
+    t0 = time.perf_counter()
+    tok, _, _ = sess.prefill(prompt, want_logits=False)
+    t1 = time.perf_counter()
+    for _ in range(n_decode):
+        tok, _, _ = sess.decode(tok, want_logits=False)
+    t2 = time.perf_counter()
+    return {
+        "value": n_decode / (t2 - t1),
+        "unit": "tok/s",
+        "cores": 1,
+        "kind": kind,
+        "sample": f"{n_decode} greedy decode steps after the same {len(prompt)}-token prompt "
+                  f"(prefill on the same core: {len(prompt) / (t1 - t0):.2f} tok/s)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--model", default="1B", choices=sorted(MODELS))
+    ap.add_argument("--seed", type=int, default=20251)
+    ap.add_argument("--cpu-steps", type=int, default=128, help="decode steps of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--profile-steps", type=int, default=32)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is single-GPU (batch-1 decode has no data parallelism to spread); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    tg = ge.load_package()
+    from tiny_gemma_amd import weights as tgw
+
+    dev = tg.init(0)
+    n_prompt, step_bytes, lm_bytes = MODELS[args.model]
+    cfg = tg.named_config(args.model)
+    if n_prompt + args.warmup + args.steps + args.profile_steps + 1 > cfg.n_pos:
+        print("bench.py: steps exceed the model's context (n_pos)", file=sys.stderr)
+        sys.exit(2)
+
+    t0 = time.perf_counter()
+    image = tgw.random_weight_image(cfg, args.seed)
+    t_gen = time.perf_counter() - t0
+    model = tg.Transformer(cfg)
+    t0 = time.perf_counter()
+    model.read_weights_mem(image)
+    t_load = time.perf_counter() - t0
+    sess = model.session()
+    rng = np.random.default_rng(args.seed)
+    prompt = rng.integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+
+    # prefill (untimed part of the warm-up; reported separately)
+    tg.synchronize()
+    t0 = time.perf_counter()
+    sess.prefill(prompt, want_logits=False)
+    t_prefill = time.perf_counter() - t0
+
+    ev = HipEvents()
+    stream = tg.lib().tg_stream()
+    e0, e1 = ev.create(), ev.create()
+    sess.decode_enqueue(args.warmup)
+    tg.synchronize()
+    # ---- timed region: exactly `steps` decode steps ----
+    ev.record(e0, stream)
+    t0 = time.perf_counter()
+    sess.decode_enqueue(args.steps)
+    ev.record(e1, stream)
+    tg.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = ev.elapsed_ms(e0, e1)
+    ids = sess.read_ids(1 + args.warmup + args.steps)
+    assert ids.size == 1 + args.warmup + args.steps and ids.min() >= 0
+
+    # ---- per-kernel-class event timing over further real decode steps ----
+    ms_sum = (C.c_double * 7)()
+    launches = (C.c_int * 7)()
+    tg.check(tg.lib().tg_decode_profile(sess.h, args.profile_steps, ms_sum, launches))
+    names = ["qkv", "attention", "oproj", "upgate_geglu", "down", "lmhead_argmax", "argmax_finish"]
+    per_kernel_us = {n: 1e3 * ms_sum[i] / max(1, launches[i]) for i, n in enumerate(names)}
+    lm_s = 1e-6 * per_kernel_us["lmhead_argmax"]
+    achieved = lm_bytes / lm_s / 1e9
+
+    tok_s = args.steps / wall
+    out = {
+        "metric": "decode_tokens_per_s",
+        "value": tok_s,
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": 1e3 * wall / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"gemma-3-{args.model} shape, int8 weight-only, random-init N(0,0.02); {n_prompt}-token random prompt "
+                        f"prefilled, then greedy decode, batch 1, GeLU LUT(-4,4,1024)",
+            "prompt_tokens": n_prompt,
+            "decode_position_start": n_prompt + args.warmup,
+            "seed": args.seed,
+        },
+        "roofline": {
+            "kernel": "tg_gemv_lmhead_argmax",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": lm_bytes,
+            "avg_launch_us": per_kernel_us["lmhead_argmax"],
+        },
+        "decode_step": {
+            "gpu_ms_per_step_events": gpu_ms / args.steps,
+            "weight_bytes_per_token": step_bytes,
+            "weight_stream_GBps": step_bytes * tok_s / 1e9,
+            "frac_of_hbm_roofline": step_bytes * tok_s / 1e9 / HBM_PEAK_GBS,
+            "avg_kernel_us": per_kernel_us,
+        },
+        "prefill": {"tokens": n_prompt, "tok_s_forward_only": n_prompt / t_prefill},
+        "setup_s": {"generate_weights": t_gen, "upload_and_retile": t_load},
+        "device": dev,
+    }
+    if args.cpu_steps > 0:
+        path = f"/tmp/tg_bench_{args.model}_{args.seed}.bin"
+        image.tofile(path)
+        try:
+            out["cpu_baseline"] = cpu_baseline(path, args.model, prompt, args.cpu_steps)
+            out["cpu_baseline"]["host_cpus"] = os.cpu_count()
+        finally:
+            os.remove(path)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -122,6 +122,12 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 int tg_decode_enqueue(tg_session *s, int n_steps);
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
 
+/* Kernel classes of one decode step, in launch order per layer; the head runs once per step. */
+enum { TG_KC_QKV = 0, TG_KC_ATTN, TG_KC_OPROJ, TG_KC_UPGATE, TG_KC_DOWN, TG_KC_LMHEAD, TG_KC_ARGMAX, TG_KC_COUNT };
+/* Runs n_steps decode steps like tg_decode_enqueue, with a HIP event recorded on tg_stream()
+ * before every launch: ms_sum[k] / launches[k] is the average event-to-event time of class k. */
+int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches);
+
 /* Debug taps: the residual stream of the most recent forward after block b
  * (b = 0: embedding; 2l+1: after attention of layer l; 2l+2: after the MLP of layer l).
  * After a prefill `rows` = prompt length, after a decode 1. out is [rows][hidden]. */

@@ -22,12 +22,6 @@ int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
 
-// workspace shared by every GEMV launch (launches are serialised on the one stream)
-float *g_ws_partial = nullptr;
-size_t g_ws_partial_floats = 0;
-unsigned *g_ws_counters = nullptr;
-size_t g_ws_counters_n = 0;
-
 bool legal_in(int d) { return d == 640 || d == 2048 || d == 1024 || d == 256 || d == 1152 || d == 6912; }            // static_switch.hpp:7-30
 bool legal_out(int d) { return d == 640 || d == 262144 || d == 2048 || d == 256 || d == 1024 || d == 1152 || d == 6912; }  // :32-58
 
@@ -36,55 +30,36 @@ int ensure_init() {
 	return tg_init(0);
 }
 
-int ensure_workspace(size_t partial_floats, size_t counters) {
-	if (partial_floats > g_ws_partial_floats) {
-		TG_HIP(hipStreamSynchronize(g_stream));
-		if (g_ws_partial) TG_HIP(hipFree(g_ws_partial));
-		g_ws_partial = nullptr;
-		TG_HIP(hipMalloc((void **)&g_ws_partial, partial_floats * sizeof(float)));
-		g_ws_partial_floats = partial_floats;
-	}
-	if (counters > g_ws_counters_n) {
-		TG_HIP(hipStreamSynchronize(g_stream));
-		if (g_ws_counters) TG_HIP(hipFree(g_ws_counters));
-		g_ws_counters = nullptr;
-		TG_HIP(hipMalloc((void **)&g_ws_counters, counters * sizeof(unsigned)));
-		TG_HIP(hipMemset(g_ws_counters, 0, counters * sizeof(unsigned)));
-		g_ws_counters_n = counters;
-	}
-	return TG_OK;
-}
-
-// A matrix on the device in the packed tile layout, with its launch geometry.
+// A matrix on the device.  `W` is the GEMV layout: ntiles tiles of C columns, each a contiguous
+// [K/4][C][4] slab (C chosen per matrix so that narrow matrices still give hundreds of
+// workgroups).  `Wg` (optional) is the same matrix in 128-column tiles for the prefill GEMM.
 struct PackedMat {
 	int8_t *W = nullptr;
-	float *scales = nullptr;
-	int K = 0, N = 0;   // N = number of (virtual) columns = ntiles * 128
-	int ntiles = 0, tpc = 1, KS = 1, ppb = 0;
+	float *scales = nullptr;   // per virtual column, GEMV tile order
+	int8_t *Wg = nullptr;
+	float *scales_g = nullptr; // per virtual column, GEMM tile order
+	int K = 0, N = 0;          // N = number of (virtual) columns
+	int ntiles = 0, C = 0, lc_shift = 0;
+	int ntiles_g = 0;
 };
 
-void choose_split(PackedMat *p) {
-	const int pairs = p->K / 8;
-	int best = 1;
-	for (int ks = 1; ks <= pairs; ks++) {
-		if (pairs % ks) continue;
-		if (pairs / ks < 4) break;
-		best = ks;
-		if (p->ntiles * ks >= 256) break;
-	}
-	p->KS = best;
-	p->ppb = pairs / best;
+// Largest tile width that still yields >= 256 workgroups (at least 4 columns; 8 for the fused
+// up|gate matrix, whose tile holds C/2 up and C/2 gate columns).
+int choose_tile_cols(int N, int min_c) {
+	int C = TG_CT;
+	while (C > min_c && (N % C != 0 || N / C < 256)) C >>= 1;
+	return C;
 }
 
-// host: [K][N] row-major (leading dimension ld, column order given by colmap or identity) -> packed tiles
-void pack_host(int8_t *dst, const int8_t *src, int K, int N, size_t ld) {
+// host: [K][N] row-major -> tiles of C columns, each [K/4][C][4]
+void pack_host(int8_t *dst, const int8_t *src, int K, int N, int C) {
 	const int kgs = K / 4;
-	for (int t = 0; t < N / TG_CT; t++) {
+	for (int t = 0; t < N / C; t++) {
 		for (int kg = 0; kg < kgs; kg++) {
-			const int8_t *r0 = src + (size_t)(4 * kg) * ld + (size_t)t * TG_CT;
-			const int8_t *r1 = r0 + ld, *r2 = r1 + ld, *r3 = r2 + ld;
-			int8_t *d = dst + ((size_t)t * kgs + kg) * TG_CT * 4;
-			for (int c = 0; c < TG_CT; c++) {
+			const int8_t *r0 = src + (size_t)(4 * kg) * N + (size_t)t * C;
+			const int8_t *r1 = r0 + N, *r2 = r1 + N, *r3 = r2 + N;
+			int8_t *d = dst + ((size_t)t * kgs + kg) * C * 4;
+			for (int c = 0; c < C; c++) {
 				d[4 * c + 0] = r0[c];
 				d[4 * c + 1] = r1[c];
 				d[4 * c + 2] = r2[c];
@@ -94,26 +69,72 @@ void pack_host(int8_t *dst, const int8_t *src, int K, int N, size_t ld) {
 	}
 }
 
-int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_scales, int K, int N, int tpc) {
+int upload_tiles(int8_t **Wd, float **sd, const int8_t *host_rowmajor, const float *host_scales, int K, int N, int C) {
+	std::vector<int8_t> tmp((size_t)K * N);
+	pack_host(tmp.data(), host_rowmajor, K, N, C);
+	TG_HIP(hipMalloc((void **)Wd, (size_t)K * N));
+	TG_HIP(hipMalloc((void **)sd, (size_t)N * sizeof(float)));
+	TG_HIP(hipMemcpy(*Wd, tmp.data(), (size_t)K * N, hipMemcpyHostToDevice));
+	TG_HIP(hipMemcpy(*sd, host_scales, (size_t)N * sizeof(float), hipMemcpyHostToDevice));
+	return TG_OK;
+}
+
+// Plain matrix [K][N] (reference layout) -> GEMV tiles, and GEMM tiles if with_gemm.
+int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_scales, int K, int N, bool with_gemm) {
 	p->K = K;
 	p->N = N;
-	p->ntiles = N / TG_CT;
-	p->tpc = tpc;
-	choose_split(p);
-	std::vector<int8_t> tmp((size_t)K * N);
-	pack_host(tmp.data(), host_rowmajor, K, N, (size_t)N);
-	TG_HIP(hipMalloc((void **)&p->W, (size_t)K * N));
-	TG_HIP(hipMalloc((void **)&p->scales, (size_t)N * sizeof(float)));
-	TG_HIP(hipMemcpy(p->W, tmp.data(), (size_t)K * N, hipMemcpyHostToDevice));
-	TG_HIP(hipMemcpy(p->scales, host_scales, (size_t)N * sizeof(float), hipMemcpyHostToDevice));
-	return ensure_workspace((size_t)p->ntiles * p->KS * TG_CT, (size_t)p->ntiles);
+	p->C = choose_tile_cols(N, 4);
+	p->lc_shift = 0;
+	while ((4 << p->lc_shift) < p->C) p->lc_shift++;
+	p->ntiles = N / p->C;
+	if (int rc = upload_tiles(&p->W, &p->scales, host_rowmajor, host_scales, K, N, p->C)) return rc;
+	if (with_gemm) {
+		p->ntiles_g = N / TG_CT;
+		if (int rc = upload_tiles(&p->Wg, &p->scales_g, host_rowmajor, host_scales, K, N, TG_CT)) return rc;
+	}
+	return TG_OK;
+}
+
+// up [K][f] and gate [K][f] -> one matrix of 2f virtual columns whose tiles of C columns hold
+// C/2 up columns followed by the same C/2 gate columns (so gelu(gate)*up never leaves a workgroup).
+void fuse_up_gate(std::vector<int8_t> &cat, std::vector<float> &catsc, const int8_t *up, const float *ups, const int8_t *gate,
+                  const float *gates, int K, int f, int C) {
+	const int C2 = C / 2;
+	cat.assign((size_t)K * 2 * f, 0);
+	catsc.assign((size_t)2 * f, 0.0f);
+	for (int t = 0; t < f / C2; t++) {
+		for (int r = 0; r < K; r++) {
+			memcpy(&cat[(size_t)r * 2 * f + (size_t)t * C], &up[(size_t)r * f + (size_t)t * C2], (size_t)C2);
+			memcpy(&cat[(size_t)r * 2 * f + (size_t)t * C + C2], &gate[(size_t)r * f + (size_t)t * C2], (size_t)C2);
+		}
+		memcpy(&catsc[(size_t)t * C], &ups[(size_t)t * C2], sizeof(float) * (size_t)C2);
+		memcpy(&catsc[(size_t)t * C + C2], &gates[(size_t)t * C2], sizeof(float) * (size_t)C2);
+	}
+}
+
+int upload_up_gate(PackedMat *p, const int8_t *up, const float *ups, const int8_t *gate, const float *gates, int K, int f) {
+	std::vector<int8_t> cat;
+	std::vector<float> catsc;
+	p->K = K;
+	p->N = 2 * f;
+	p->C = choose_tile_cols(2 * f, 8);
+	p->lc_shift = 0;
+	while ((4 << p->lc_shift) < p->C) p->lc_shift++;
+	p->ntiles = p->N / p->C;
+	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, p->C);
+	if (int rc = upload_tiles(&p->W, &p->scales, cat.data(), catsc.data(), K, 2 * f, p->C)) return rc;
+	// GEMM layout: 128-column tiles, tile 2t = up columns [128t, 128t+128), tile 2t+1 = the same gate columns
+	p->ntiles_g = p->N / TG_CT;
+	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, 2 * TG_CT);
+	return upload_tiles(&p->Wg, &p->scales_g, cat.data(), catsc.data(), K, 2 * f, TG_CT);
 }
 
 void free_packed(PackedMat *p) {
-	if (p->W) (void)hipFree(p->W);
-	if (p->scales) (void)hipFree(p->scales);
-	p->W = nullptr;
-	p->scales = nullptr;
+	void *ps[] = {p->W, p->scales, p->Wg, p->scales_g};
+	for (void *q : ps)
+		if (q) (void)hipFree(q);
+	p->W = p->Wg = nullptr;
+	p->scales = p->scales_g = nullptr;
 }
 
 TgGemv gemv_base(const PackedMat &p) {
@@ -123,11 +144,8 @@ TgGemv gemv_base(const PackedMat &p) {
 	g.scales = p.scales;
 	g.K = p.K;
 	g.ntiles = p.ntiles;
-	g.KS = p.KS;
-	g.pairs_per_block = p.ppb;
-	g.tpc = p.tpc;
-	g.partial = g_ws_partial;
-	g.counters = g_ws_counters;
+	g.C = p.C;
+	g.lc_shift = p.lc_shift;
 	return g;
 }
 
@@ -174,8 +192,8 @@ struct tg_session {
 	std::vector<int> max_pos;
 	float *xr = nullptr;      // [(2L+1)][hidden] residual stream after every block of the last decode
 	float *qkv = nullptr, *attn_out = nullptr, *o_out = nullptr, *hbuf = nullptr, *d_out = nullptr, *logits = nullptr;
-	float *part_acc = nullptr, *part_ml = nullptr;
-	unsigned *attn_counter = nullptr, *argmax_counter = nullptr;
+	float *part_acc = nullptr, *part_ml = nullptr;      // attention partials [nb][4][256], [nb][4][2]
+	float *merged_acc = nullptr, *merged_ml = nullptr;  // long contexts: partials folded into one
 	float *blk_val = nullptr;
 	int *blk_idx = nullptr;
 	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token
@@ -187,7 +205,7 @@ struct tg_session {
 };
 
 namespace {
-constexpr int ATTN_MAX_BLOCKS = 256;
+constexpr int ATTN_MAX_BLOCKS = TG_ATTN_MAX_BLOCKS;
 constexpr int PREFILL_TAP_MAX_ROWS = 1024;
 
 bool layer_is_local(const tg_config &c, int l) { return (l % c.window_pattern) != (c.window_pattern - 1); }  // transformer.hpp:43
@@ -305,7 +323,7 @@ int tg_qweight_create(const int8_t *B, const float *scales, int inDim, int outDi
 	if (!legal_in(inDim)) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported ROW dimension: " + std::to_string(inDim));
 	if (!legal_out(outDim)) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported COL dimension: " + std::to_string(outDim));
 	tg_qweight *w = new tg_qweight();
-	int rc = upload_packed(&w->p, B, scales, inDim, outDim, 1);
+	int rc = upload_packed(&w->p, B, scales, inDim, outDim, outDim <= 16384);
 	if (rc != TG_OK) {
 		free_packed(&w->p);
 		delete w;
@@ -326,18 +344,17 @@ int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logi
 	(void)logits_variant;  // one kernel serves both reference variants (they differ only in rounding order)
 	if (!y_dev || !x_dev || !w) return tg_fail(TG_ERR_BAD_ARG, "null argument");
 	TgGemv g = gemv_base(w->p);
-	g.pro = TG_PRO_PLAIN;
 	g.x = x_dev;
-	g.epi = TG_EPI_STORE;
 	g.y = y_dev;
-	tg_launch_gemv(g, g_stream);
+	tg_launch_gemv(g, TG_ROLE_PLAIN, g_stream);
 	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
 
 int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
-	tg_launch_gemm(C_dev, A_dev, w->p.W, w->p.scales, m, w->p.K, w->p.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+	if (!w->p.Wg) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "no GEMM tiling was built for this matrix (outDim too large)");
+	tg_launch_gemm(C_dev, A_dev, w->p.Wg, w->p.scales_g, m, w->p.K, w->p.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
 	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
@@ -477,41 +494,31 @@ static int load_weights_impl(tg_model *m, Reader rd) {
 			memcpy(&catsc[(size_t)col], sc.data(), sizeof(float) * (size_t)n);
 			col += n;
 		}
-		if ((rc = upload_packed(&L.qkv, cat.data(), catsc.data(), h, nq, 1))) return rc;
+		if ((rc = upload_packed(&L.qkv, cat.data(), catsc.data(), h, nq, true))) return rc;
 		// O
 		if ((rc = read_i8(buf, (size_t)qo * h))) return rc;
 		if ((rc = read_f(sc, (size_t)h))) return rc;
-		if ((rc = upload_packed(&L.o, buf.data(), sc.data(), qo, h, 1))) return rc;
+		if ((rc = upload_packed(&L.o, buf.data(), sc.data(), qo, h, true))) return rc;
 		if ((rc = read_dev_f(&L.rms_q, (size_t)hd))) return rc;
 		if ((rc = read_dev_f(&L.rms_k, (size_t)hd))) return rc;
 		if ((rc = read_dev_f(&L.apre, (size_t)h))) return rc;
 		if ((rc = read_dev_f(&L.apost, (size_t)h))) return rc;
-		// up | gate fused tile by tile: virtual tile 2t = up columns [128t, 128t+128), 2t+1 = the same gate columns
+		// up | gate fused tile by tile
 		if ((rc = read_i8(buf, (size_t)h * f))) return rc;
 		if ((rc = read_f(sc, (size_t)f))) return rc;
 		if ((rc = read_i8(buf2, (size_t)h * f))) return rc;
 		if ((rc = read_f(sc2, (size_t)f))) return rc;
-		cat.assign((size_t)h * 2 * f, 0);
-		catsc.assign((size_t)2 * f, 0.0f);
-		for (int t = 0; t < f / TG_CT; t++) {
-			for (int r = 0; r < h; r++) {
-				memcpy(&cat[(size_t)r * 2 * f + (size_t)(2 * t) * TG_CT], &buf[(size_t)r * f + (size_t)t * TG_CT], TG_CT);
-				memcpy(&cat[(size_t)r * 2 * f + (size_t)(2 * t + 1) * TG_CT], &buf2[(size_t)r * f + (size_t)t * TG_CT], TG_CT);
-			}
-			memcpy(&catsc[(size_t)(2 * t) * TG_CT], &sc[(size_t)t * TG_CT], sizeof(float) * TG_CT);
-			memcpy(&catsc[(size_t)(2 * t + 1) * TG_CT], &sc2[(size_t)t * TG_CT], sizeof(float) * TG_CT);
-		}
-		if ((rc = upload_packed(&L.ug, cat.data(), catsc.data(), h, 2 * f, 2))) return rc;
+		if ((rc = upload_up_gate(&L.ug, buf.data(), sc.data(), buf2.data(), sc2.data(), h, f))) return rc;
 		// down
 		if ((rc = read_i8(buf, (size_t)f * h))) return rc;
 		if ((rc = read_f(sc, (size_t)h))) return rc;
-		if ((rc = upload_packed(&L.d, buf.data(), sc.data(), f, h, 1))) return rc;
+		if ((rc = upload_packed(&L.d, buf.data(), sc.data(), f, h, true))) return rc;
 		if ((rc = read_dev_f(&L.mpre, (size_t)h))) return rc;
 		if ((rc = read_dev_f(&L.mpost, (size_t)h))) return rc;
 	}
 	if ((rc = read_i8(buf, (size_t)h * V))) return rc;
 	if ((rc = read_f(sc, (size_t)V))) return rc;
-	if ((rc = upload_packed(&m->lm, buf.data(), sc.data(), h, V, 1))) return rc;
+	if ((rc = upload_packed(&m->lm, buf.data(), sc.data(), h, V, false))) return rc;
 	m->loaded = true;
 	return TG_OK;
 }
@@ -579,7 +586,7 @@ void tg_session_destroy(tg_session *s) {
 	if (!s) return;
 	(void)hipStreamSynchronize(g_stream);
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
-	              s->logits, s->part_acc, s->part_ml, s->attn_counter, s->argmax_counter, s->blk_val, s->blk_idx, s->ctr,
+	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
 	              s->tok_log, s->taps};
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
@@ -647,8 +654,8 @@ int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin,
 	TG_ALLOC(s->logits, sizeof(float) * (size_t)c.n_vocab);
 	TG_ALLOC(s->part_acc, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * hd);
 	TG_ALLOC(s->part_ml, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * 2);
-	TG_ALLOC(s->attn_counter, sizeof(unsigned));
-	TG_ALLOC(s->argmax_counter, sizeof(unsigned));
+	TG_ALLOC(s->merged_acc, sizeof(float) * (size_t)c.n_head * hd);
+	TG_ALLOC(s->merged_ml, sizeof(float) * (size_t)c.n_head * 2);
 	TG_ALLOC(s->blk_val, sizeof(float) * (size_t)m->lm.ntiles);
 	TG_ALLOC(s->blk_idx, sizeof(int) * (size_t)m->lm.ntiles);
 	TG_ALLOC(s->ctr, sizeof(int) * 8);
@@ -669,8 +676,6 @@ int tg_session_reset(tg_session *s) {
 		TG_HIP(hipMemset(s->vc[l], 0, bytes));
 	}
 	TG_HIP(hipMemset(s->ctr, 0, sizeof(int) * 8));
-	TG_HIP(hipMemset(s->attn_counter, 0, sizeof(unsigned)));
-	TG_HIP(hipMemset(s->argmax_counter, 0, sizeof(unsigned)));
 	TG_HIP(hipMemset(s->xr, 0, sizeof(float) * (size_t)(2 * c.n_layers + 1) * c.hidden_size));
 	TG_HIP(hipDeviceSynchronize());
 	s->pos = s->bp_local = s->bp_global = s->steps = 0;
@@ -687,18 +692,43 @@ int tg_session_position(const tg_session *s) { return s ? s->pos : -1; }
 // ---------------------------------------------------------------------------------------------
 // forward_decode: 5 launches per layer + 1 for the head
 // ---------------------------------------------------------------------------------------------
-static int attn_chunk_for(int valid) {
-	int c = 16;
-	while (c < 256 && (valid + c - 1) / c > 128) c *= 2;
-	return c;
+// Keys per attention workgroup.  Up to 4096 keys the chunk is sized so that at most
+// TG_ATTN_MERGE_MAX partials result, which the output projection merges in its prologue;
+// beyond that 128-key chunks are used and a merge launch folds the partials first.
+static int attn_chunk_for(int valid, bool *needs_merge) {
+	int c = ((valid + TG_ATTN_MERGE_MAX - 1) / TG_ATTN_MERGE_MAX + 15) / 16 * 16;
+	*needs_merge = c > 256;
+	return *needs_merge ? 128 : c;
 }
 
-static int enqueue_decode_step(tg_session *s, bool want_logits) {
+// Event pool for tg_decode_profile: one event before every launch of a step plus one at the end.
+struct StepProfile {
+	std::vector<hipEvent_t> ev;
+	std::vector<int> cls;
+	size_t used = 0;
+	hipError_t mark(int kernel_class) {
+		if (used == ev.size()) {
+			hipEvent_t e;
+			hipError_t rc = hipEventCreate(&e);
+			if (rc != hipSuccess) return rc;
+			ev.push_back(e);
+			cls.push_back(0);
+		}
+		cls[used] = kernel_class;
+		return hipEventRecord(ev[used++], g_stream);
+	}
+};
+
+static int enqueue_decode_step(tg_session *s, StepProfile *prof) {
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
-	const int L = c.n_layers, h = c.hidden_size, hd = c.head_dim;
+	const int L = c.n_layers, h = c.hidden_size;
 	if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
 	if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
+#define TG_MARK(k)                                 \
+	if (prof) {                                    \
+		TG_HIP(prof->mark(k));                     \
+	}
 	for (int l = 0; l < L; l++) {
 		const LayerDev &Ld = m->L[(size_t)l];
 		// --- pre-norm + Q|K|V (modules.hpp:137-144); folds the previous block's post-norm + residual
@@ -706,22 +736,21 @@ static int enqueue_decode_step(tg_session *s, bool want_logits) {
 		g.hidden = h;
 		g.w_pre = Ld.apre;
 		g.xr_out = s->xr + (size_t)(2 * l) * h;
+		g.y = s->qkv;
+		TG_MARK(TG_KC_QKV);
 		if (l == 0) {
-			g.pro = TG_PRO_EMBED;
 			g.wte = m->wte;
 			g.wte_scales = m->wte_scales;
 			g.tok = s->ctr + 4;
 			g.vocab = c.n_vocab;
 			g.emb_scale = (float)sqrt((double)h);  // ops.hpp:586
+			tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream);
 		} else {
-			g.pro = TG_PRO_RESNORM;
 			g.pend = s->d_out;
 			g.w_post = m->L[(size_t)l - 1].mpost;
 			g.x = s->xr + (size_t)(2 * l - 1) * h;
+			tg_launch_gemv(g, TG_ROLE_QKV, g_stream);
 		}
-		g.epi = TG_EPI_STORE;
-		g.y = s->qkv;
-		tg_launch_gemv(g, g_stream);
 		// --- q/k norm, RoPE, KV write, attention (modules.hpp:146-161)
 		TgAttnDecode a;
 		memset(&a, 0, sizeof(a));
@@ -736,76 +765,75 @@ static int enqueue_decode_step(tg_session *s, bool want_logits) {
 		a.pos = s->ctr;
 		a.bp_index = Ld.is_sw ? 1 : 2;
 		const int valid = std::min(s->pos + 1, a.max_pos);
-		a.chunk = attn_chunk_for(valid);
+		bool needs_merge = false;
+		a.chunk = attn_chunk_for(valid, &needs_merge);
 		a.part_acc = s->part_acc;
 		a.part_ml = s->part_ml;
-		a.counter = s->attn_counter;
-		a.out = s->attn_out;
 		a.n_head = c.n_head;
+		TG_MARK(TG_KC_ATTN);
 		tg_launch_attn_decode(a, (valid + a.chunk - 1) / a.chunk, g_stream);
-		// --- O projection (modules.hpp:163-164)
+		if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream);
+		// --- merge of the attention partials + O projection (modules.hpp:161-164)
 		g = gemv_base(Ld.o);
-		g.pro = TG_PRO_PLAIN;
-		g.x = s->attn_out;
-		g.epi = TG_EPI_STORE;
+		g.pos = s->ctr;
+		g.attn_max_pos = a.max_pos;
+		g.attn_chunk = needs_merge ? a.max_pos : a.chunk;  // merged: a single partial
+		g.part_acc = needs_merge ? s->merged_acc : s->part_acc;
+		g.part_ml = needs_merge ? s->merged_ml : s->part_ml;
 		g.y = s->o_out;
-		tg_launch_gemv(g, g_stream);
+		TG_MARK(TG_KC_OPROJ);
+		tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream);
 		// --- post-norm + residual, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
 		g = gemv_base(Ld.ug);
-		g.pro = TG_PRO_RESNORM;
 		g.hidden = h;
 		g.pend = s->o_out;
 		g.w_post = Ld.apost;
 		g.x = s->xr + (size_t)(2 * l) * h;
 		g.xr_out = s->xr + (size_t)(2 * l + 1) * h;
 		g.w_pre = Ld.mpre;
-		g.epi = TG_EPI_GEGLU;
 		g.y = s->hbuf;
 		g.lut = s->lut;
 		g.gmin = s->gmin;
 		g.geps = s->geps;
 		g.lut_size = s->lut_size;
-		tg_launch_gemv(g, g_stream);
+		TG_MARK(TG_KC_UPGATE);
+		tg_launch_gemv(g, TG_ROLE_UPGATE, g_stream);
 		// --- down projection (modules.hpp:216-217)
 		g = gemv_base(Ld.d);
-		g.pro = TG_PRO_PLAIN;
 		g.x = s->hbuf;
-		g.epi = TG_EPI_STORE;
 		g.y = s->d_out;
-		tg_launch_gemv(g, g_stream);
+		TG_MARK(TG_KC_DOWN);
+		tg_launch_gemv(g, TG_ROLE_DOWN, g_stream);
 	}
 	// --- last post-norm + residual, final norm, LM head, argmax (modules.hpp:242-246, ops.hpp:744)
 	TgGemv g = gemv_base(m->lm);
-	g.pro = TG_PRO_RESNORM;
 	g.hidden = h;
 	g.pend = s->d_out;
 	g.w_post = m->L[(size_t)L - 1].mpost;
 	g.x = s->xr + (size_t)(2 * L - 1) * h;
 	g.xr_out = s->xr + (size_t)(2 * L) * h;
 	g.w_pre = m->rmsw;
-	g.epi = TG_EPI_LOGITS;
-	g.y = want_logits ? s->logits : nullptr;
+	g.y = s->logits;
 	g.blk_val = s->blk_val;
 	g.blk_idx = s->blk_idx;
-	g.argmax_counter = s->argmax_counter;
-	g.tok_out = s->ctr + 4;
-	g.tok_log = s->tok_log;
-	g.step = s->ctr + 3;
-	g.pos = s->ctr;
-	tg_launch_gemv(g, g_stream);
+	TG_MARK(TG_KC_LMHEAD);
+	tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream);
+	TG_MARK(TG_KC_ARGMAX);
+	tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
+	TG_MARK(-1);
+#undef TG_MARK
 	TG_HIP(hipGetLastError());
 	s->pos += 1;
 	s->bp_local += 1;
 	s->bp_global += 1;
 	s->steps += 1;
-	(void)hd;
 	return TG_OK;
 }
 
 int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax) {
 	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
 	TG_HIP(hipMemcpyAsync(s->ctr + 4, &id, sizeof(int), hipMemcpyHostToDevice, g_stream));
-	if (int rc = enqueue_decode_step(s, logits != nullptr)) return rc;
+	if (int rc = enqueue_decode_step(s, nullptr)) return rc;
 	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)s->m->cfg.n_vocab, hipMemcpyDeviceToHost, g_stream));
 	int32_t tok = -1;
 	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
@@ -822,7 +850,7 @@ int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax)
 int tg_decode_enqueue(tg_session *s, int n_steps) {
 	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	for (int i = 0; i < n_steps; i++)
-		if (int rc = enqueue_decode_step(s, false)) return rc;
+		if (int rc = enqueue_decode_step(s, nullptr)) return rc;
 	if (s->taps) {
 		TG_HIP(hipStreamSynchronize(g_stream));
 		(void)hipFree(s->taps);
@@ -830,6 +858,36 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 		s->tap_rows = 0;
 	}
 	return TG_OK;
+}
+
+int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches) {
+	if (!s || n_steps < 1 || !ms_sum || !launches) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	for (int k = 0; k < TG_KC_COUNT; k++) {
+		ms_sum[k] = 0.0;
+		launches[k] = 0;
+	}
+	StepProfile prof;
+	int rc = TG_OK;
+	for (int i = 0; i < n_steps && rc == TG_OK; i++) {
+		prof.used = 0;
+		rc = enqueue_decode_step(s, &prof);
+		if (rc != TG_OK) break;
+		if (hipStreamSynchronize(g_stream) != hipSuccess) {
+			rc = tg_fail(TG_ERR_HIP, "hipStreamSynchronize failed");
+			break;
+		}
+		for (size_t e = 0; e + 1 < prof.used; e++) {
+			float ms = 0.0f;
+			if (hipEventElapsedTime(&ms, prof.ev[e], prof.ev[e + 1]) != hipSuccess) {
+				rc = tg_fail(TG_ERR_HIP, "hipEventElapsedTime failed");
+				break;
+			}
+			ms_sum[prof.cls[e]] += (double)ms;
+			launches[prof.cls[e]] += 1;
+		}
+	}
+	for (hipEvent_t e : prof.ev) (void)hipEventDestroy(e);
+	return rc;
 }
 
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out) {
@@ -899,7 +957,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		const LayerDev &Ld = m->L[(size_t)l];
 		const int mp = s->max_pos[(size_t)l];
 		// Q|K|V (modules.hpp:106-108)
-		tg_launch_gemm(qkv, xn, Ld.qkv.W, Ld.qkv.scales, n, h, Ld.qkv.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		tg_launch_gemm(qkv, xn, Ld.qkv.Wg, Ld.qkv.scales_g, n, h, Ld.qkv.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
 		// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
 		tg_launch_qk_norm_rope_rows(qkv, qkv + qo, qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
@@ -907,13 +965,13 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
 		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, g_stream);
 		// O (modules.hpp:127-128)
-		tg_launch_gemm(t, ao, Ld.o.W, Ld.o.scales, n, qo, Ld.o.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		tg_launch_gemm(t, ao, Ld.o.Wg, Ld.o.scales_g, n, qo, Ld.o.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
 		tg_launch_norm_rows(xn, t, Ld.mpre, Ld.apost, x, x, n, h, g_stream);
 		TG_TRY(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
-		tg_launch_gemm(hb, xn, Ld.ug.W, Ld.ug.scales, n, h, Ld.ug.ntiles, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, g_stream);
-		tg_launch_gemm(t, hb, Ld.d.W, Ld.d.scales, n, f, Ld.d.ntiles, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		tg_launch_gemm(hb, xn, Ld.ug.Wg, Ld.ug.scales_g, n, h, Ld.ug.ntiles_g, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, g_stream);
+		tg_launch_gemm(t, hb, Ld.d.Wg, Ld.d.scales_g, n, f, Ld.d.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
 		tg_launch_norm_rows(xn, t, next_pre, Ld.mpost, x, x, n, h, g_stream);
@@ -922,18 +980,12 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	// LM head on the last position only (modules.hpp:232-240): xn already holds rmsnorm(x, RMSw)
 	{
 		TgGemv g = gemv_base(m->lm);
-		g.pro = TG_PRO_PLAIN;
 		g.x = xn + (S - 1) * h;
-		g.epi = TG_EPI_LOGITS;
-		g.y = logits ? s->logits : nullptr;
+		g.y = s->logits;
 		g.blk_val = s->blk_val;
 		g.blk_idx = s->blk_idx;
-		g.argmax_counter = s->argmax_counter;
-		g.tok_out = s->ctr + 4;
-		g.tok_log = s->tok_log;
-		g.step = s->ctr + 3;
-		g.pos = nullptr;
-		tg_launch_gemv(g, g_stream);
+		tg_launch_gemv(g, TG_ROLE_LMHEAD_PLAIN, g_stream);
+		tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 0, g_stream);
 	}
 	TG_TRY(hipGetLastError());
 	// KVCache::update_prefill's counters (decode.hpp:99-104)

@@ -5,9 +5,10 @@
 //   decode : ops::attention_decode (ops.hpp:224-370) — one query token, 4 heads sharing 1 KV head,
 //            keys = the valid slots of a ring (local layers) or linear (global layers) cache.
 //            The reference walks the slots sequentially with a renormalising online softmax; here
-//            the slots are split across workgroups (flash-decoding), each computing an exact
-//            softmax partial (max, sum, unnormalised output) over its chunk, merged by the last
-//            workgroup to finish.  Softmax is order independent, so only fp32 rounding differs.
+//            the slots are split across workgroups (flash-decoding), each writing an exact softmax
+//            partial (max, sum, unnormalised output) of its chunk; the partials are merged in the
+//            prologue of the output projection (tg_gemv.hip) — via attn_merge_kernel first when
+//            there are many.  Softmax is order independent, so only fp32 rounding differs.
 //   prefill: ops::attention_prefill (ops.hpp:377-526) — causal; local layers see keys
 //            qs-window .. qs inclusive (window+1 keys, ops.hpp:437-443).
 
@@ -99,7 +100,6 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	__shared__ float knew[HD], vnew[HD];
 	__shared__ float sc[NH][MAXCHUNK];
 	__shared__ float s_m[NH], s_l[NH];
-	__shared__ unsigned s_ticket;
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int pos = a.pos[0];                      // position_ptr before this token (decode.hpp:154)
@@ -170,39 +170,52 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 		}
 	}
 
-	if (nb == 1) {
-#pragma unroll
-		for (int h = 0; h < NH; h++) a.out[h * HD + tid] = acc[h] / s_l[h];
-		return;
-	}
+	// partial (max, sum, unnormalised output) of this chunk; merged by the consumer
 #pragma unroll
 	for (int h = 0; h < NH; h++) a.part_acc[((size_t)b * NH + h) * HD + tid] = acc[h];
 	if (tid < NH) {
 		a.part_ml[((size_t)b * NH + tid) * 2 + 0] = s_m[tid];
 		a.part_ml[((size_t)b * NH + tid) * 2 + 1] = s_l[tid];
 	}
-	__threadfence();
+}
+
+// Long contexts only: folds more than TG_ATTN_MERGE_MAX partials into one (max 0, sum 1, normalised
+// output) so that the consumer's merge stays small.  One workgroup per head.
+__global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, float *merged_acc, float *merged_ml) {
+	__shared__ float wg[TG_ATTN_MAX_BLOCKS];
+	__shared__ float sred[4];
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x;
+	const int pos = a.pos[0];
+	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;
+	const int nb = (valid + a.chunk - 1) / a.chunk;
+	const bool ok = tid < nb;
+	const float m = ok ? a.part_ml[((size_t)tid * NH + h) * 2] : -INFINITY;
+	const float l = ok ? a.part_ml[((size_t)tid * NH + h) * 2 + 1] : 0.0f;
+	float M = wmax(m);
+	if (lane == 0) sred[w] = M;
 	__syncthreads();
-	if (tid == 0) s_ticket = atomicAdd(a.counter, 1u);
+	M = fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
 	__syncthreads();
-	if (s_ticket != (unsigned)(nb - 1)) return;
-	__threadfence();
-	// merge: O = sum_b acc_b * exp(m_b - M) / sum_b l_b * exp(m_b - M)
+	const float e = ok ? expf(m - M) : 0.0f;
+	float L = wsum(l * e);
+	if (lane == 0) sred[w] = L;
+	__syncthreads();
+	L = (sred[0] + sred[1]) + (sred[2] + sred[3]);
+	wg[tid] = e / L;
+	__syncthreads();
+	float o = 0.0f;
+	for (int b0 = 0; b0 < nb; b0 += 8) {
+		float v[8];
 #pragma unroll
-	for (int h = 0; h < NH; h++) {
-		float M = -INFINITY;
-		for (int i = 0; i < nb; i++) M = fmaxf(M, __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2));
-		float L = 0.0f, O = 0.0f;
-		for (int i = 0; i < nb; i++) {
-			const float mi = __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2);
-			const float li = __builtin_nontemporal_load(a.part_ml + ((size_t)i * NH + h) * 2 + 1);
-			const float e = expf(mi - M);
-			L = fmaf(li, e, L);
-			O = fmaf(__builtin_nontemporal_load(a.part_acc + ((size_t)i * NH + h) * HD + tid), e, O);
-		}
-		a.out[h * HD + tid] = O / L;
+		for (int u = 0; u < 8; u++) v[u] = (b0 + u < nb) ? a.part_acc[((size_t)(b0 + u) * NH + h) * HD + tid] : 0.0f;
+#pragma unroll
+		for (int u = 0; u < 8; u++) o = fmaf(v[u], wg[(b0 + u < nb) ? b0 + u : 0], o);
 	}
-	if (tid == 0) *a.counter = 0u;
+	merged_acc[h * HD + tid] = o;
+	if (tid == 0) {
+		merged_ml[h * 2 + 0] = 0.0f;
+		merged_ml[h * 2 + 1] = 1.0f;
+	}
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -304,6 +317,10 @@ __global__ __launch_bounds__(ANT) void attn_prefill_kernel(float *o, const float
 
 void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s) {
 	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)max_blocks), dim3(ANT), 0, s, a);
+}
+
+void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s) {
+	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH), dim3(ANT), 0, s, a, merged_acc, merged_ml);
 }
 
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,

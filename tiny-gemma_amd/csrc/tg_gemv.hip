@@ -4,26 +4,29 @@
 //     y[c] = scales[c] * sum_r x[r] * float(W[r][c])
 // with the scale applied once after the whole fp32 reduction (linalg.hpp:83-107).
 //
-// Work decomposition: grid = (128-column tiles) x (K splits).  Inside a workgroup every lane
-// streams 16-byte pieces of the packed tile (4 columns x 4 input rows, see tg_internal.h),
-// converts each byte with one sign-extending convert, and keeps one fp32 accumulator per column;
-// lanes 0-31 and 32-63 of a wave take alternating row groups.  The lane/wave partials are summed
-// through LDS in a fixed order; when the reduction is split over several workgroups the partial
-// sums go through a small HBM workspace and the last workgroup to finish (ticket counter) adds
-// them in a fixed order and runs the epilogue, so results are run-to-run deterministic.
+// Work decomposition: one workgroup per tile of C output columns, over the WHOLE reduction
+// length, so no partial sums ever leave the workgroup: no atomics, no device-scope fences (on
+// this multi-XCD part a fence is an L2 write-back + invalidate, tens of microseconds when
+// hundreds of workgroups issue one).  C is chosen per matrix (4 ... 128) so that every matrix,
+// however narrow, yields a few hundred workgroups.  The tile is stored as one contiguous slab
+// [K/4][C][4] (tg_internal.h): the 256 lanes read consecutive 16-byte pieces (4 columns x 4 rows),
+// C/4 lanes across the columns and 1024/C lanes along K; each byte is converted with one
+// sign-extending convert and fed to an fp32 FMA; lanes that share columns are combined with
+// cross-lane shuffles and one small LDS exchange between the 4 waves, in a fixed order, so
+// results are run-to-run deterministic.
 //
 // Prologues fold the work that precedes a projection in modules::attention / modules::mlp
 // (modules.hpp:135-220) into the same launch: embedding gather, post-norm + residual add of the
-// previous block, pre-norm.  Epilogues fold what follows it: LUT-GeLU(gate) * up, or logits
-// write-out plus greedy argmax.
+// previous block, pre-norm, or the merge of the attention partials.  Epilogues fold what follows:
+// LUT-GeLU(gate) * up, or logits write-out plus the per-workgroup stage of the greedy argmax.
 
 #include "tg_internal.h"
 
 namespace {
 
-constexpr int NW = 4;          // waves per workgroup
-constexpr int NT = NW * 64;    // threads per workgroup
-constexpr int UNROLL = 4;      // 16-byte loads in flight per lane
+constexpr int NT = 256;     // threads per workgroup (4 waves)
+constexpr int NWAVE = 4;
+constexpr int UNROLL = 4;   // 16-byte weight loads per lane per batch (two batches in flight)
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
@@ -39,10 +42,7 @@ __device__ __forceinline__ float block_sum(float v, float *sred) {
 	__syncthreads();
 	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
 	__syncthreads();
-	float t = 0.0f;
-#pragma unroll
-	for (int i = 0; i < NW; i++) t += sred[i];
-	return t;
+	return (sred[0] + sred[1]) + (sred[2] + sred[3]);
 }
 
 __device__ __forceinline__ float b2f(int d, int j) {  // signed byte j of d -> float (exact)
@@ -57,31 +57,88 @@ __device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin,
 	return lut[idx];
 }
 
-__global__ __launch_bounds__(NT) void gemv_kernel(const TgGemv g) {
-	__shared__ float xs[TG_MAX_K];
-	__shared__ float red[NW * 2 * TG_CT];
-	__shared__ float sred[NW];
-	__shared__ unsigned s_ticket;
-	__shared__ float s_bv[NW];
-	__shared__ int s_bi[NW];
+__device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const float4 xv) {
+	const int d0 = v.x, d1 = v.y, d2 = v.z, d3 = v.w;
+	acc[0] = fmaf(xv.x, b2f(d0, 0), acc[0]); acc[0] = fmaf(xv.y, b2f(d0, 1), acc[0]);
+	acc[0] = fmaf(xv.z, b2f(d0, 2), acc[0]); acc[0] = fmaf(xv.w, b2f(d0, 3), acc[0]);
+	acc[1] = fmaf(xv.x, b2f(d1, 0), acc[1]); acc[1] = fmaf(xv.y, b2f(d1, 1), acc[1]);
+	acc[1] = fmaf(xv.z, b2f(d1, 2), acc[1]); acc[1] = fmaf(xv.w, b2f(d1, 3), acc[1]);
+	acc[2] = fmaf(xv.x, b2f(d2, 0), acc[2]); acc[2] = fmaf(xv.y, b2f(d2, 1), acc[2]);
+	acc[2] = fmaf(xv.z, b2f(d2, 2), acc[2]); acc[2] = fmaf(xv.w, b2f(d2, 3), acc[2]);
+	acc[3] = fmaf(xv.x, b2f(d3, 0), acc[3]); acc[3] = fmaf(xv.y, b2f(d3, 1), acc[3]);
+	acc[3] = fmaf(xv.z, b2f(d3, 2), acc[3]); acc[3] = fmaf(xv.w, b2f(d3, 3), acc[3]);
+}
+
+template <int PRO, int EPI>
+__device__ __forceinline__ void gemv_body(const TgGemv &g) {
+	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
+	__shared__ __attribute__((aligned(16))) float red[NWAVE][TG_CT];
+	__shared__ float sred[NWAVE];
+	__shared__ float wgt[4][TG_ATTN_MERGE_MAX];
+	__shared__ float s_bv[NWAVE];
+	__shared__ int s_bi[NWAVE];
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-	const int tile = blockIdx.x, ks = blockIdx.y;
+	const int tile = blockIdx.x;
+	const int C = g.C, LC = C >> 2, lcs = g.lc_shift;  // LC = 1 << lcs lanes across the tile's columns
+	const int KL = NT >> lcs;                          // lanes along K
+	const int cl = tid & (LC - 1), kpos = tid >> lcs;
+	const int kgs = g.K >> 2;
+	const i32x4 *Wt = reinterpret_cast<const i32x4 *>(g.W) + (size_t)tile * kgs * LC + cl;
+	const int nit = (kgs + KL - 1) / KL;  // uniform trip count; lanes past the end are predicated off
 
-	// ---------------- prologue: input vector into LDS ----------------
-	if (g.pro == TG_PRO_PLAIN) {
-		const int r0 = ks * g.pairs_per_block * 8, n = g.pairs_per_block * 8;
-		for (int i = tid; i < n; i += NT) xs[r0 + i] = g.x[r0 + i];
-	} else {
+	// first batch of weight loads is issued before the prologue: it does not depend on x
+	i32x4 v[UNROLL];
+#pragma unroll
+	for (int u = 0; u < UNROLL; u++) {
+		const int kg = kpos + u * KL;
+		v[u] = (u < nit && kg < kgs) ? __builtin_nontemporal_load(Wt + (size_t)kg * LC) : i32x4{0, 0, 0, 0};
+	}
+
+	// ---------------- prologue: input vector ----------------
+	if (PRO == TG_PRO_ATTN_MERGE) {
+		// merge of the flash-decoding partials of the attention launch that precedes this projection:
+		//   out_h = sum_b acc_{b,h} * exp(m_{b,h} - M_h) / sum_b l_{b,h} * exp(m_{b,h} - M_h)
+		const int pos = g.pos[0];
+		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
+		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
+		if (tid < 4 * TG_ATTN_MERGE_MAX) {
+			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
+			const bool ok = b < nb;
+			const float m = ok ? g.part_ml[((size_t)b * 4 + h) * 2] : -INFINITY;
+			const float l = ok ? g.part_ml[((size_t)b * 4 + h) * 2 + 1] : 0.0f;
+			float M = m;
+#pragma unroll
+			for (int o = TG_ATTN_MERGE_MAX / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+			const float e = ok ? expf(m - M) : 0.0f;
+			float L = l * e;
+#pragma unroll
+			for (int o = TG_ATTN_MERGE_MAX / 2; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+			wgt[h][b] = e / L;
+		}
+		__syncthreads();
+#pragma unroll
+		for (int h = 0; h < 4; h++) {
+			float a[TG_ATTN_MERGE_MAX];
+#pragma unroll
+			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
+				a[b] = (b < nb) ? g.part_acc[((size_t)b * 4 + h) * 256 + tid] : 0.0f;
+			float o = 0.0f;
+#pragma unroll
+			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) o = fmaf(a[b], wgt[h][b], o);
+			xs[h * 256 + tid] = o;
+		}
+		__syncthreads();
+	} else if (PRO != TG_PRO_PLAIN) {
 		const int h = g.hidden;
 		const float eps = 1e-06f;
-		if (g.pro == TG_PRO_EMBED) {
+		if (PRO == TG_PRO_EMBED) {
 			// ops.hpp:537-568: s[d] * (sqrt(hidden) * q)
 			int tok = *g.tok;
 			tok = tok < 0 ? 0 : (tok >= g.vocab ? g.vocab - 1 : tok);
 			const int8_t *row = g.wte + (size_t)tok * h;
 			for (int d = tid; d < h; d += NT) xs[d] = g.wte_scales[d] * (g.emb_scale * (float)row[d]);
-		} else if (g.pro == TG_PRO_NORM) {
+		} else if (PRO == TG_PRO_NORM) {
 			for (int d = tid; d < h; d += NT) xs[d] = g.x[d];
 		} else {
 			// modules.hpp:166-168 / 218-219: x = rmsnorm(block_out, post) + residual
@@ -95,7 +152,7 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const TgGemv g) {
 			const float irms = 1.0f / sqrtf(ss / (float)h + eps);
 			for (int d = tid; d < h; d += NT) xs[d] = (xs[d] * irms) * (g.w_post[d] + 1.0f) + g.x[d];
 		}
-		if (g.xr_out != nullptr && tile == 0 && ks == 0)
+		if (g.xr_out != nullptr && tile == 0)
 			for (int d = tid; d < h; d += NT) g.xr_out[d] = xs[d];
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
 		float ss = 0.0f;
@@ -103,99 +160,71 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const TgGemv g) {
 		ss = block_sum(ss, sred);
 		const float irms = 1.0f / sqrtf(ss / (float)h + eps);
 		for (int d = tid; d < h; d += NT) xs[d] = (xs[d] * irms) * (g.w_pre[d] + 1.0f);
+		__syncthreads();
 	}
-	__syncthreads();
 
-	// ---------------- main loop: stream the packed tile ----------------
-	const int half = lane >> 5, cl = lane & 31;
-	const int kgs = g.K >> 2;
-	const i32x4 *Wt = reinterpret_cast<const i32x4 *>(g.W) + (size_t)tile * kgs * (TG_CT / 4);
-	const int p0 = ks * g.pairs_per_block;
-	const int np = (g.pairs_per_block - w + NW - 1) / NW;  // pairs p0 + w, p0 + w + NW, ...
-	float acc0 = 0.0f, acc1 = 0.0f, acc2 = 0.0f, acc3 = 0.0f;
-	for (int i = 0; i < np; i += UNROLL) {
-		i32x4 v[UNROLL];
-		int kg[UNROLL];
+	// ---------------- main loop: stream the tile, next batch in flight while this one is consumed ----------------
+	float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+	for (int i0 = 0; i0 < nit; i0 += UNROLL) {
+		i32x4 vn[UNROLL];
 #pragma unroll
 		for (int u = 0; u < UNROLL; u++) {
-			const bool ok = (i + u) < np;
-			kg[u] = ok ? 2 * (p0 + w + (i + u) * NW) + half : 2 * p0;
-			v[u] = ok ? __builtin_nontemporal_load(Wt + (size_t)kg[u] * (TG_CT / 4) + cl) : i32x4{0, 0, 0, 0};
+			const int kg = kpos + (i0 + UNROLL + u) * KL;
+			vn[u] = (i0 + UNROLL + u < nit && kg < kgs) ? __builtin_nontemporal_load(Wt + (size_t)kg * LC) : i32x4{0, 0, 0, 0};
 		}
+		float4 xv[UNROLL];
 #pragma unroll
 		for (int u = 0; u < UNROLL; u++) {
-			const float4 xv = *reinterpret_cast<const float4 *>(&xs[4 * kg[u]]);
-			const int d0 = v[u].x, d1 = v[u].y, d2 = v[u].z, d3 = v[u].w;
-			acc0 = fmaf(xv.x, b2f(d0, 0), acc0); acc0 = fmaf(xv.y, b2f(d0, 1), acc0);
-			acc0 = fmaf(xv.z, b2f(d0, 2), acc0); acc0 = fmaf(xv.w, b2f(d0, 3), acc0);
-			acc1 = fmaf(xv.x, b2f(d1, 0), acc1); acc1 = fmaf(xv.y, b2f(d1, 1), acc1);
-			acc1 = fmaf(xv.z, b2f(d1, 2), acc1); acc1 = fmaf(xv.w, b2f(d1, 3), acc1);
-			acc2 = fmaf(xv.x, b2f(d2, 0), acc2); acc2 = fmaf(xv.y, b2f(d2, 1), acc2);
-			acc2 = fmaf(xv.z, b2f(d2, 2), acc2); acc2 = fmaf(xv.w, b2f(d2, 3), acc2);
-			acc3 = fmaf(xv.x, b2f(d3, 0), acc3); acc3 = fmaf(xv.y, b2f(d3, 1), acc3);
-			acc3 = fmaf(xv.z, b2f(d3, 2), acc3); acc3 = fmaf(xv.w, b2f(d3, 3), acc3);
+			int kg = kpos + (i0 + u) * KL;
+			kg = (kg < kgs) ? kg : 0;  // weights of a predicated-off piece are zero; any finite x will do
+			xv[u] = (PRO == TG_PRO_PLAIN) ? *reinterpret_cast<const float4 *>(g.x + 4 * kg)
+			                              : *reinterpret_cast<const float4 *>(&xs[4 * kg]);
 		}
-	}
-
-	// ---------------- workgroup reduction (fixed order) ----------------
-	*reinterpret_cast<float4 *>(&red[(w * 2 + half) * TG_CT + cl * 4]) = make_float4(acc0, acc1, acc2, acc3);
-	__syncthreads();
-	float sum = 0.0f;
-	if (tid < TG_CT) {
 #pragma unroll
-		for (int i = 0; i < NW * 2; i++) sum += red[i * TG_CT + tid];
+		for (int u = 0; u < UNROLL; u++) fma16(acc, v[u], xv[u]);
+#pragma unroll
+		for (int u = 0; u < UNROLL; u++) v[u] = vn[u];
 	}
 
-	// ---------------- cross-workgroup reduction ----------------
-	const int group_n = g.KS * g.tpc;
-	int t_first = tile, t_count = 1;
-	float val[2] = {sum, 0.0f};
-	if (group_n > 1) {
-		if (tid < TG_CT) g.partial[((size_t)tile * g.KS + ks) * TG_CT + tid] = sum;
-		__threadfence();
-		__syncthreads();
-		if (tid == 0) s_ticket = atomicAdd(&g.counters[tile / g.tpc], 1u);
-		__syncthreads();
-		if (s_ticket != (unsigned)(group_n - 1)) return;
-		__threadfence();
-		t_first = (tile / g.tpc) * g.tpc;
-		t_count = g.tpc;
-		if (tid < TG_CT) {
-			for (int t = 0; t < t_count; t++) {
-				float s = 0.0f;
-				const float *pp = g.partial + (size_t)(t_first + t) * g.KS * TG_CT + tid;
-				for (int k = 0; k < g.KS; k++) s += __builtin_nontemporal_load(pp + (size_t)k * TG_CT);
-				val[t] = s;
-			}
-		}
-		if (tid == 0) g.counters[tile / g.tpc] = 0u;
+	// ---------------- reduction over the lanes along K (fixed order) ----------------
+	for (int o = 32; o >= LC; o >>= 1) {
+#pragma unroll
+		for (int j = 0; j < 4; j++) acc[j] += __shfl_xor(acc[j], o, 64);
 	}
+	if (lane < LC) *reinterpret_cast<float4 *>(&red[w][lane * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+	__syncthreads();
 
 	// ---------------- epilogue ----------------
-	if (g.epi == TG_EPI_STORE) {
-		if (tid < TG_CT) {
-			const int col = t_first * TG_CT + tid;
-			g.y[col] = val[0] * g.scales[col];
+	if (EPI == TG_EPI_STORE) {
+		if (tid < C) {
+			const int col = tile * C + tid;
+			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+			g.y[col] = sum * g.scales[col];
 		}
 		return;
 	}
-	if (g.epi == TG_EPI_GEGLU) {
-		// modules.hpp:211-215: gelu(gate) * up ; tiles (2t, 2t+1) hold up | gate columns of block t
-		if (tid < TG_CT) {
-			const float up = val[0] * g.scales[t_first * TG_CT + tid];
-			const float gate = val[1] * g.scales[(t_first + 1) * TG_CT + tid];
-			g.y[(t_first / 2) * TG_CT + tid] = gelu_lut(gate, g.lut, g.gmin, g.geps, g.lut_size) * up;
+	if (EPI == TG_EPI_GEGLU) {
+		// modules.hpp:211-215: gelu(gate) * up; the tile holds C/2 up columns, then the same C/2 gate columns
+		const int C2 = C >> 1;
+		if (tid < C2) {
+			const float su = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+			const float sg = (red[0][tid + C2] + red[1][tid + C2]) + (red[2][tid + C2] + red[3][tid + C2]);
+			const float up = su * g.scales[tile * C + tid];
+			const float gate = sg * g.scales[tile * C + C2 + tid];
+			g.y[tile * C2 + tid] = gelu_lut(gate, g.lut, g.gmin, g.geps, g.lut_size) * up;
 		}
 		return;
 	}
-	// TG_EPI_LOGITS: logits + greedy argmax (ops.hpp:749-757: strict '>' from index 0 => lowest index wins)
+	// TG_EPI_LOGITS: logits + first stage of the greedy argmax
+	// (ops.hpp:749-757: strict '>' scan from index 0, so the lowest index wins ties)
 	float bv = -INFINITY;
 	int bi = 0x7fffffff;
-	if (tid < TG_CT) {
-		const int col = t_first * TG_CT + tid;
-		const float v = val[0] * g.scales[col];
-		if (g.y != nullptr) g.y[col] = v;
-		if (v > bv) { bv = v; bi = col; }
+	if (tid < C) {
+		const int col = tile * C + tid;
+		const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+		const float val = sum * g.scales[col];
+		if (g.y != nullptr) g.y[col] = val;
+		if (val > bv) { bv = val; bi = col; }
 	}
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) {
@@ -206,22 +235,38 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const TgGemv g) {
 	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
 	__syncthreads();
 	if (tid == 0) {
-		for (int i = 1; i < NW; i++)
+		for (int i = 1; i < NWAVE; i++)
 			if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
 		g.blk_val[tile] = bv;
 		g.blk_idx[tile] = bi;
 	}
-	__threadfence();
-	__syncthreads();
-	if (tid == 0) s_ticket = atomicAdd(g.argmax_counter, 1u);
-	__syncthreads();
-	if (s_ticket != (unsigned)(g.ntiles * g.KS / group_n - 1)) return;
-	__threadfence();
-	bv = -INFINITY;
-	bi = 0x7fffffff;
-	for (int i = tid; i < g.ntiles; i += NT) {
-		const float ov = __builtin_nontemporal_load(g.blk_val + i);
-		const int oi = __builtin_nontemporal_load(g.blk_idx + i);
+}
+
+// One named entry point per role, so that profiles separate the projections.
+#define TG_GEMV_KERNEL(NAME, PRO, EPI) \
+	__global__ __launch_bounds__(NT) void NAME(const TgGemv g) { gemv_body<PRO, EPI>(g); }
+TG_GEMV_KERNEL(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE)        // layer 0: embedding + pre-norm + Q|K|V
+TG_GEMV_KERNEL(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE)            // post-norm + residual + pre-norm + Q|K|V
+TG_GEMV_KERNEL(tg_gemv_oproj, TG_PRO_ATTN_MERGE, TG_EPI_STORE)       // attention merge + output projection
+TG_GEMV_KERNEL(tg_gemv_upgate_geglu, TG_PRO_RESNORM, TG_EPI_GEGLU)   // post-norm + residual + pre-norm + up|gate + gelu*up
+TG_GEMV_KERNEL(tg_gemv_down, TG_PRO_PLAIN, TG_EPI_STORE)             // down projection
+TG_GEMV_KERNEL(tg_gemv_lmhead_argmax, TG_PRO_RESNORM, TG_EPI_LOGITS) // last post-norm + final norm + LM head + argmax stage 1
+TG_GEMV_KERNEL(tg_gemv_lmhead_plain, TG_PRO_PLAIN, TG_EPI_LOGITS)    // LM head on an already normalised vector (prefill)
+TG_GEMV_KERNEL(tg_gemv_plain, TG_PRO_PLAIN, TG_EPI_STORE)            // stand-alone y = s * (x . W)
+
+// Second stage of the greedy argmax, and the per-token bookkeeping: the winning id becomes the
+// next step's input token, is appended to the id log, and KVCache::update_single's counters
+// (decode.hpp:68-69) advance once per token.
+__global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log,
+                                                       int advance) {
+	__shared__ float s_bv[NWAVE];
+	__shared__ int s_bi[NWAVE];
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	float bv = -INFINITY;
+	int bi = 0x7fffffff;
+	for (int i = tid; i < n; i += NT) {
+		const float ov = blk_val[i];
+		const int oi = blk_idx[i];
 		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 	}
 #pragma unroll
@@ -230,31 +275,40 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const TgGemv g) {
 		const int oi = __shfl_xor(bi, o, 64);
 		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 	}
-	__syncthreads();
 	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
 	__syncthreads();
 	if (tid == 0) {
-		for (int i = 1; i < NW; i++)
+		for (int i = 1; i < NWAVE; i++)
 			if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
 		if (bi == 0x7fffffff) bi = -1;  // all NaN: the reference's scan leaves -1 (ops.hpp:750)
-		*g.argmax_counter = 0u;
-		*g.tok_out = bi;
-		if (g.step != nullptr) {
-			const int st = *g.step;
-			if (g.tok_log != nullptr) g.tok_log[st] = bi;
-			*g.step = st + 1;
-		}
-		if (g.pos != nullptr) {  // KVCache::update_single's counters (decode.hpp:68-69), once per token
-			g.pos[0] += 1;
-			g.pos[1] += 1;
-			g.pos[2] += 1;
+		ctr[4] = bi;
+		const int st = ctr[3];
+		tok_log[st] = bi;
+		ctr[3] = st + 1;
+		if (advance) {
+			ctr[0] += 1;
+			ctr[1] += 1;
+			ctr[2] += 1;
 		}
 	}
 }
 
 }  // namespace
 
-void tg_launch_gemv(const TgGemv &g, hipStream_t s) {
-	dim3 grid((unsigned)g.ntiles, (unsigned)g.KS);
-	hipLaunchKernelGGL(gemv_kernel, grid, dim3(NT), 0, s, g);
+void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s) {
+	dim3 grid((unsigned)g.ntiles), block(NT);
+	switch (role) {
+		case TG_ROLE_QKV_EMBED: hipLaunchKernelGGL(tg_gemv_qkv_embed, grid, block, 0, s, g); break;
+		case TG_ROLE_QKV: hipLaunchKernelGGL(tg_gemv_qkv, grid, block, 0, s, g); break;
+		case TG_ROLE_OPROJ: hipLaunchKernelGGL(tg_gemv_oproj, grid, block, 0, s, g); break;
+		case TG_ROLE_UPGATE: hipLaunchKernelGGL(tg_gemv_upgate_geglu, grid, block, 0, s, g); break;
+		case TG_ROLE_DOWN: hipLaunchKernelGGL(tg_gemv_down, grid, block, 0, s, g); break;
+		case TG_ROLE_LMHEAD: hipLaunchKernelGGL(tg_gemv_lmhead_argmax, grid, block, 0, s, g); break;
+		case TG_ROLE_LMHEAD_PLAIN: hipLaunchKernelGGL(tg_gemv_lmhead_plain, grid, block, 0, s, g); break;
+		default: hipLaunchKernelGGL(tg_gemv_plain, grid, block, 0, s, g); break;
+	}
+}
+
+void tg_launch_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log, int advance, hipStream_t s) {
+	hipLaunchKernelGGL(tg_argmax_finish, dim3(1), dim3(NT), 0, s, blk_val, blk_idx, n, ctr, tok_log, advance);
 }

@@ -15,66 +15,60 @@
 //
 // The reference keeps W as [in][out] row-major int8 (csrc/include/tensor.hpp:144-192): bytes run
 // along the output dimension and the reduction runs across rows.  On the device every matrix is
-// re-tiled once at upload into
+// re-tiled once at upload into tiles of C output columns,
 //
-//        P[tile][kg][c][j]      tile = col / 128, kg = row / 4, c = col % 128, j = row % 4
+//        P[tile][kg][c][j]      tile = col / C, kg = row / 4, c = col % C, j = row % 4
 //
 // so that (1) one 16-byte lane load holds 4 output columns x 4 consecutive input rows, with the
 // 4 rows of one column packed in one dword (the k-contiguous operand shape MFMA wants, and four
-// sign-extending byte->float converts for the GEMV), (2) a wave's 64 lane loads are one
-// contiguous 1 KiB segment covering two kg rows of a 128-column tile, and (3) everything a
-// workgroup streams for its tile is one contiguous slab of K*128 bytes.  The values are the
-// reference's bytes, only their addresses change.
+// sign-extending byte->float converts for the GEMV), (2) consecutive lanes read consecutive
+// 16-byte pieces, and (3) everything a workgroup streams for its tile is one contiguous slab of
+// K*C bytes.  The GEMV uses C = 4 ... 128 per matrix (a tile per workgroup over the whole K, so
+// narrow matrices still give hundreds of workgroups); the prefill GEMM uses C = 128.  The values
+// are the reference's bytes, only their addresses change.
 // ---------------------------------------------------------------------------------------------
-#define TG_CT 128            // output columns per packed tile
+#define TG_CT 128            // widest tile (and the GEMM tile width)
 #define TG_MAX_K 6912        // largest reduction length (1B down projection)
-
-inline size_t tg_packed_index(int K, int r, int c) {
-	return (((size_t)(c / TG_CT) * (size_t)(K / 4) + (size_t)(r / 4)) * TG_CT + (size_t)(c % TG_CT)) * 4 + (size_t)(r % 4);
-}
+#define TG_MAX_HIDDEN 1152   // largest residual-stream width
+#define TG_ATTN_MERGE_MAX 16 // attention partials the output projection merges in its prologue
+#define TG_ATTN_MAX_BLOCKS 256  // attention workgroups per launch, upper bound
 
 // ---- GEMV launch description --------------------------------------------------------------
-enum { TG_PRO_PLAIN = 0, TG_PRO_NORM = 1, TG_PRO_RESNORM = 2, TG_PRO_EMBED = 3 };
+enum { TG_PRO_PLAIN = 0, TG_PRO_NORM = 1, TG_PRO_RESNORM = 2, TG_PRO_EMBED = 3, TG_PRO_ATTN_MERGE = 4 };
 enum { TG_EPI_STORE = 0, TG_EPI_GEGLU = 1, TG_EPI_LOGITS = 2 };
 
 struct TgGemv {
-	// matrix
-	const int8_t *W;       // packed, ntiles tiles of 128 columns
+	// matrix: ntiles tiles of C columns, each a contiguous [K/4][C][4] slab
+	const int8_t *W;
 	const float *scales;   // one per (virtual) column, tile order
 	int K;                 // reduction length (rows of the reference matrix)
-	int ntiles;            // 128-column tiles (grid.x)
-	int KS;                // K splits (grid.y)
-	int pairs_per_block;   // (K/8)/KS: one "pair" = 8 input rows x 128 columns = 1 KiB
-	int tpc;               // tiles per completion group: 1, or 2 for the fused up|gate matrix
-	// workspace for the cross-workgroup reduction (unused when KS*tpc == 1)
-	float *partial;        // [ntiles][KS][128]
-	unsigned *counters;    // [ntiles/tpc], zero between launches
-	// prologue: how the input vector is produced
-	int pro;
-	int hidden;            // length of the residual stream (PRO_NORM/RESNORM/EMBED)
+	int ntiles;            // grid.x
+	int C;                 // columns per tile: 4, 8, ..., 128
+	int lc_shift;          // log2(C/4)
+	// prologue (the TG_PRO_* mode is fixed by the kernel role)
+	int hidden;            // length of the residual stream (NORM/RESNORM/EMBED); equals K there
 	const float *x;        // PLAIN: the input [K]; NORM: vector to normalise; RESNORM: residual
 	const float *pend;     // RESNORM: block output still to be post-normalised and added
 	const float *w_post;   // RESNORM: post-norm weights
 	const float *w_pre;    // NORM/RESNORM/EMBED: pre-norm weights
-	float *xr_out;         // NORM/RESNORM/EMBED: residual stream written by workgroup (0,0); may be null
+	float *xr_out;         // NORM/RESNORM/EMBED: residual stream written by workgroup 0; may be null
 	const int8_t *wte;     // EMBED: [vocab][hidden] row-major int8 (reference layout)
 	const float *wte_scales;
 	const int *tok;        // EMBED: device token id (clamped to [0, vocab))
 	int vocab;
 	float emb_scale;       // EMBED: float(sqrt(hidden))
-	// epilogue
-	int epi;
+	const int *pos;        // ATTN_MERGE: device counters (pos[0] = position of this token)
+	int attn_max_pos;      // ATTN_MERGE: cache slots of this layer
+	int attn_chunk;        // ATTN_MERGE: keys per attention workgroup
+	const float *part_acc; // ATTN_MERGE: [nb][4][256]
+	const float *part_ml;  // ATTN_MERGE: [nb][4][2]
+	// epilogue (the TG_EPI_* mode is fixed by the kernel role)
 	float *y;              // STORE: [N]; GEGLU: [N/2]; LOGITS: [N] or null
 	const float *lut;      // GEGLU
 	float gmin, geps;
 	int lut_size;
-	float *blk_val;        // LOGITS: per-workgroup maxima [ntiles]
+	float *blk_val;        // LOGITS: per-workgroup maximum and its index, [ntiles]
 	int *blk_idx;
-	unsigned *argmax_counter;
-	int *tok_out;          // LOGITS: winning index (lowest index on ties)
-	int *tok_log;          // LOGITS: optional history, tok_log[*step] = winner
-	int *step;             // LOGITS: device step counter, incremented by the last workgroup
-	int *pos;              // LOGITS: device position counter, incremented by the last workgroup
 };
 
 struct TgAttnDecode {
@@ -88,13 +82,15 @@ struct TgAttnDecode {
 	int chunk;               // keys per workgroup
 	float *part_acc;         // [nblocks][n_head][hd]
 	float *part_ml;          // [nblocks][n_head][2]
-	unsigned *counter;
-	float *out;              // [n_head*hd]
 	int n_head;
 };
 
-void tg_launch_gemv(const TgGemv &g, hipStream_t s);
+enum { TG_ROLE_PLAIN = 0, TG_ROLE_QKV_EMBED, TG_ROLE_QKV, TG_ROLE_OPROJ, TG_ROLE_UPGATE, TG_ROLE_DOWN, TG_ROLE_LMHEAD,
+       TG_ROLE_LMHEAD_PLAIN };
+void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s);
 void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s);
+void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s);
+void tg_launch_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log, int advance, hipStream_t s);
 
 // ---- prefill kernels (rows = prompt positions) -----------------------------------------------
 void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,
