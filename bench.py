@@ -95,6 +95,7 @@ def main():
     ap.add_argument("--seed", type=int, default=20251)
     ap.add_argument("--cpu-steps", type=int, default=128, help="decode steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=32)
+    ap.add_argument("--no-graphs", action="store_true", help="plain stream launches instead of HIP graph replay")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is single-GPU (batch-1 decode has no data parallelism to spread); run with --gpus 1",
@@ -105,6 +106,7 @@ def main():
     from tiny_gemma_amd import weights as tgw
 
     dev = tg.init(0)
+    tg.lib().tg_set_graphs(0 if args.no_graphs else 1)
     n_prompt, step_bytes, lm_bytes = MODELS[args.model]
     cfg = tg.named_config(args.model)
     if n_prompt + args.warmup + args.steps + args.profile_steps + 1 > cfg.n_pos:
@@ -173,6 +175,7 @@ def main():
             "prompt_tokens": n_prompt,
             "decode_position_start": n_prompt + args.warmup,
             "seed": args.seed,
+            "launch": "stream" if args.no_graphs else "hipGraph replay",
         },
         "roofline": {
             "kernel": "tg_gemv_lmhead_argmax",

@@ -120,6 +120,8 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 /* Enqueues n_steps decode steps without host synchronisation (each step feeds the device-side
  * argmax of the previous one).  Ids are read back with tg_session_read_ids after tg_synchronize. */
 int tg_decode_enqueue(tg_session *s, int n_steps);
+/* tg_decode_enqueue replays captured HIP graphs of a decode step by default; 0 = plain stream launches */
+int tg_set_graphs(int enable);
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
 
 /* Kernel classes of one decode step, in launch order per layer; the head runs once per step. */

@@ -1,0 +1,130 @@
+"""Seeded inputs shared by tests/golden/make_golden.py (which records the reference's outputs) and
+the tests (which regenerate the same inputs).  Only numpy; nothing here touches the reference."""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# name: (inDim, outDim, logits variant, seed).  cfg1 is the bare matvec of the benchmark
+# configuration list: x ~ N(0,1), W uniform in [-127,127] stored [640][2048], scales ~ U(0.001,0.02).
+GEMV_CASES = {
+    "cfg1_640x2048": (640, 2048, False, 101),
+    "q_1152x1024": (1152, 1024, False, 102),
+    "kv_640x256": (640, 256, False, 103),
+    "o_1024x1152": (1024, 1152, False, 104),
+    "up_1152x6912": (1152, 6912, False, 105),       # row tile 8 in the reference
+    "down_6912x1152": (6912, 1152, False, 106),
+    "down_2048x640": (2048, 640, False, 107),
+    "sq_256x256": (256, 256, False, 108),
+    "lmhead_640x262144": (640, 262144, True, 109),  # row tile 4
+    "lmhead_1152x262144": (1152, 262144, True, 110),
+}
+
+# name: (m, inDim, outDim, seed): ragged m around the reference's 6-row / 256-row blocking
+GEMM_CASES = {
+    "m1_640x256": (1, 640, 256, 201),
+    "m7_640x1024": (7, 640, 1024, 202),
+    "m64_640x2048": (64, 640, 2048, 203),
+    "m178_1152x1024": (178, 1152, 1024, 204),
+    "m257_2048x640": (257, 2048, 640, 205),
+    "m13_6912x1152": (13, 6912, 1152, 206),
+    "m70_1152x6912": (70, 1152, 6912, 207),
+}
+
+RMSNORM_CASES = {"h640": (5, 640, 301), "h1152": (3, 1152, 302), "hd256": (8, 256, 303)}
+ROPE_ROWS = np.array([0, 1, 2, 17, 511, 512, 1000, 4095, 16384, 32767])
+# name: (S, is_sw, sw_context, seed)
+ATTN_PREFILL_CASES = {"causal_40": (40, False, 512, 401), "window_700": (700, True, 512, 402), "window16_50": (50, True, 16, 403)}
+# name: (max_pos, valid, seed)
+ATTN_DECODE_CASES = {"one_key": (512, 1, 501), "partial_37": (512, 37, 502), "full_ring": (512, 512, 503), "global_1300": (2048, 1300, 504)}
+
+# name: (shape, n_layers, seed, prompt tokens, decode steps, decode steps with taps, GeLU table size)
+MODEL_CASES = {
+    "small6": ("270m", 6, 11, 70, 12, 4, 1024),           # one global layer (l = 5), short prompt
+    "small6_window": ("270m", 6, 12, 600, 6, 3, 1024),    # prompt longer than the 512-slot ring
+    "small6_finelut": ("270m", 6, 11, 70, 12, 4, 1 << 20),  # near-continuous GeLU table: tight end-to-end check
+    "full270m": ("270m", 18, 1, 64, 256, 2, 1024),        # 64-token prompt + 256 greedy steps
+    "full1B": ("1B", 26, 1, 178, 1024, 2, 1024),          # 178-token prompt + 1024 greedy steps
+}
+
+
+def gemv_inputs(i, n, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(i).astype(np.float32)
+    W = rng.integers(-127, 128, (i, n), dtype=np.int8)
+    s = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    return x, W, s
+
+
+def gemm_inputs(m, i, n, seed):
+    rng = np.random.default_rng(seed)
+    A = rng.standard_normal((m, i)).astype(np.float32)
+    W = rng.integers(-127, 128, (i, n), dtype=np.int8)
+    s = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    return A, W, s
+
+
+def rmsnorm_inputs(rows, dim, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((rows, dim)) * 3).astype(np.float32), (rng.standard_normal(dim) * 0.1).astype(np.float32)
+
+
+def rope_apply_input(seed):
+    return np.random.default_rng(seed).standard_normal((4, 9, 256)).astype(np.float32)
+
+
+def gelu_input(seed):
+    x = (np.random.default_rng(seed).standard_normal(4096) * 2.5).astype(np.float32)
+    x[:8] = [-4.0, 4.0, -4.00001, 3.99999, 0.0, -0.0, 10.0, -10.0]
+    return x
+
+
+def embedding_inputs(seed):
+    rng = np.random.default_rng(seed)
+    wte = rng.integers(-127, 128, (1000, 640), dtype=np.int8)
+    sc = rng.uniform(0.001, 0.02, 640).astype(np.float32)
+    ids = rng.integers(0, 1000, 17).astype(np.int32)
+    return ids, wte, sc
+
+
+def attn_prefill_inputs(S, seed):
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((4, S, 256)).astype(np.float32)
+    k = rng.standard_normal((S, 256)).astype(np.float32)
+    v = rng.standard_normal((S, 256)).astype(np.float32)
+    return q, k, v
+
+
+def attn_decode_inputs(max_pos, seed):
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((4, 256)).astype(np.float32)
+    kc = rng.standard_normal((max_pos, 256)).astype(np.float32)
+    vc = rng.standard_normal((max_pos, 256)).astype(np.float32)
+    return q, kc, vc
+
+
+def attn_rows(S):
+    """Query rows of an attention output kept in the fixture."""
+    return np.unique(np.concatenate([np.arange(0, S, 37), np.arange(max(0, S - 6), S)]))
+
+
+def tap_rows(S):
+    """Prompt positions of the residual-stream taps kept in the fixture."""
+    return np.unique(np.concatenate([np.arange(0, S, 11), [S - 1]]))
+
+
+def argmax_input(seed):
+    return np.random.default_rng(seed).standard_normal(262144).astype(np.float32)
+
+
+def prompt_ids(seed, n):
+    return np.random.default_rng(1000 + seed).integers(0, 262144, n).astype(np.int32)
+
+
+def oracle_config(shape, n_layers):
+    from oracle.oracle import named_config
+    return named_config(shape, n_layers)

@@ -1,0 +1,130 @@
+"""GPU: the int8 GEMV / GEMM through the C ABI against the CPU checker on the same seeded inputs.
+
+Tolerance: the GEMV sums each column in fp32 in a different (parallel) order than the reference's
+row-by-row walk, so it agrees to fp32 rounding: norm-relative error <= 3e-6 here (the bound of
+the task is 1e-3).  On integer-valued inputs with power-of-two scales every order gives the same
+bits, so those must match exactly.  The prefill GEMM keeps the reference's per-element order
+(one fused chain over k) and must be bit-exact.
+"""
+import numpy as np
+import pytest
+
+import golden_inputs as gi
+from conftest import normrel
+
+pytestmark = pytest.mark.gpu
+GEMV_TOL = 3e-6
+
+
+@pytest.mark.parametrize("name", list(gi.GEMV_CASES))
+def test_qgemv_vs_checker(tg, oracle, golden, name):
+    i, n, logits, seed = gi.GEMV_CASES[name]
+    x, W, s = gi.gemv_inputs(i, n, seed)
+    y = np.zeros(n, np.float32)
+    tg.launch_qgemv(y, x, W, s, i, n, logits=logits)
+    ref = oracle.qgemv(x, W, s, logits)
+    assert normrel(y, ref) < GEMV_TOL
+    assert np.abs(y - ref).max() <= 2e-5 * np.abs(ref).max()
+    assert normrel(y[:2048], golden[f"gemv/{name}/head"]) < GEMV_TOL  # the compiled reference's own output
+
+
+@pytest.mark.parametrize("i,n,logits", [(256, 256, False), (640, 2048, False), (1152, 6912, False), (6912, 1152, False),
+                                        (2048, 640, False), (1152, 262144, True)])
+def test_qgemv_integer_inputs_bit_exact(tg, i, n, logits):
+    rng = np.random.default_rng(i * 7 + n)
+    x = rng.integers(-8, 9, i).astype(np.float32)
+    W = rng.integers(-127, 128, (i, n), dtype=np.int8)
+    s = np.full(n, 2.0 ** -10, np.float32)
+    y = np.zeros(n, np.float32)
+    tg.launch_qgemv(y, x, W, s, i, n, logits=logits)
+    exact = (x.astype(np.int64) @ W.astype(np.int64)).astype(np.float64) * 2.0 ** -10
+    assert np.array_equal(y.astype(np.float64), exact)
+
+
+def test_qgemv_extreme_weights(tg, oracle):
+    """All weights at +-127 and at 0; a zero input; a one-hot input picks out one row of W."""
+    i, n = 640, 2048
+    s = np.linspace(0.001, 0.02, n).astype(np.float32)
+    x = np.random.default_rng(1).standard_normal(i).astype(np.float32)
+    for fill in (127, -127, 0):
+        W = np.full((i, n), fill, np.int8)
+        y = np.zeros(n, np.float32)
+        tg.launch_qgemv(y, x, W, s, i, n)
+        assert normrel(y, oracle.qgemv(x, W, s)) < GEMV_TOL if fill else not y.any()
+    W = np.random.default_rng(2).integers(-127, 128, (i, n), dtype=np.int8)
+    y = np.zeros(n, np.float32)
+    tg.launch_qgemv(y, np.zeros(i, np.float32), W, s, i, n)
+    assert not y.any()
+    e = np.zeros(i, np.float32)
+    e[333] = 1.0
+    tg.launch_qgemv(y, e, W, s, i, n)
+    assert np.array_equal(y, W[333].astype(np.float32) * s)
+
+
+def test_qgemv_accumulates_into_c_like_the_reference(tg, oracle):
+    """linalg.hpp:52-107: C += A.B, then C *= scales: a non-zero C is carried through the scale."""
+    x, W, s = gi.gemv_inputs(640, 256, 5)
+    c0 = np.random.default_rng(6).standard_normal(256).astype(np.float32)
+    y = c0.copy()
+    tg.launch_qgemv(y, x, W, s, 640, 256)
+    ref = (c0.astype(np.float64) + x.astype(np.float64) @ W.astype(np.float64)) * s
+    assert normrel(y, ref) < GEMV_TOL
+
+
+def test_unsupported_shapes_raise(tg):
+    """Same legal set and same failure as ROW_SWITCH / COL_SWITCH (static_switch.hpp:7-58)."""
+    for i, n in [(512, 256), (256, 512), (262144, 256), (100, 100)]:
+        x = np.zeros(i, np.float32)
+        W = np.zeros((i, n), np.int8)
+        s = np.ones(n, np.float32)
+        with pytest.raises(tg.TgError) as e:
+            tg.launch_qgemv(np.zeros(n, np.float32), x, W, s, i, n)
+        assert e.value.code == -1 and "Unsupported" in str(e.value)
+        with pytest.raises(tg.TgError):
+            tg.launch_qgemm(np.zeros((2, n), np.float32), np.zeros((2, i), np.float32), W, s, 2, i, n)
+
+
+@pytest.mark.parametrize("name", list(gi.GEMM_CASES))
+def test_qgemm_bit_exact(tg, oracle, golden, name):
+    m, i, n, seed = gi.GEMM_CASES[name]
+    A, W, s = gi.gemm_inputs(m, i, n, seed)
+    Cm = np.full((m, n), np.nan, np.float32)  # launch_qgemm overwrites C (linalg.hpp:244)
+    tg.launch_qgemm(Cm, A, W, s, m, i, n)
+    assert np.array_equal(Cm, oracle.qgemm(A, W, s))
+    assert np.array_equal(Cm.reshape(-1)[:2048], golden[f"gemm/{name}/head"])
+
+
+def test_device_resident_gemv_matches_host_entry(tg, oracle):
+    x, W, s = gi.gemv_inputs(1152, 6912, 9)
+    w = tg.QWeight(W, s)
+    xd = tg.DeviceBuffer.from_numpy(x)
+    yd = tg.DeviceBuffer(4 * 6912)
+    for _ in range(3):
+        w.gemv(yd, xd)
+    tg.synchronize()
+    y = yd.to_numpy(np.float32, 6912)
+    y2 = np.zeros(6912, np.float32)
+    tg.launch_qgemv(y2, x, W, s, 1152, 6912)
+    assert np.array_equal(y, y2)  # deterministic: same bits every launch
+    assert normrel(y, oracle.qgemv(x, W, s)) < GEMV_TOL
+
+
+def test_full_size_properties(tg):
+    """LM-head size (302 MB of weights): linearity and a checksum of checksums, no CPU checker needed."""
+    i, n = 1152, 262144
+    rng = np.random.default_rng(3)
+    W = rng.integers(-127, 128, (i, n), dtype=np.int8)
+    s = np.full(n, 2.0 ** -9, np.float32)
+    w = tg.QWeight(W, s)
+    xa = rng.integers(-4, 5, i).astype(np.float32)
+    xb = rng.integers(-4, 5, i).astype(np.float32)
+    outs = []
+    for x in (xa, xb, xa + xb):
+        xd = tg.DeviceBuffer.from_numpy(x)
+        yd = tg.DeviceBuffer(4 * n)
+        w.gemv(yd, xd, logits=True)
+        tg.synchronize()
+        outs.append(yd.to_numpy(np.float32, n))
+    assert np.array_equal(outs[0] + outs[1], outs[2])  # exact on integer data
+    colsum = W.astype(np.int64).sum(axis=1)            # sum_c y[c] = s * sum_r x[r] * rowsum(W)[r]
+    assert float(outs[0].astype(np.float64).sum()) == float((xa.astype(np.int64) * colsum).sum()) * 2.0 ** -9

@@ -1,0 +1,239 @@
+"""GPU: forward_prefill / forward_decode / greedy generation through the C ABI against the CPU
+checker on the same weights, prompts and tables, and against the compiled reference's recorded
+token ids (tests/golden/golden.npz).
+
+Tolerances.  All arithmetic is fp32 on both sides; summation orders differ.  With a near-continuous
+GeLU table (2^20 entries) the two agree to fp32 rounding end to end (<= 5e-5 norm-relative after
+6 layers).  With the reference CLI's 1024-entry step-function table (csrc/include/ops.hpp:22-52)
+an ULP upstream can move a gate activation to the next table entry, which is worth ~1e-4 of a
+layer's output; the compiled reference and the strict-IEEE checker differ from each other by the
+same mechanism.  Those cases are held to 5e-3 per tap, and greedy token ids must be identical.
+"""
+import numpy as np
+import pytest
+
+import golden_inputs as gi
+from conftest import normrel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tables(oracle):
+    cg, sg = oracle.rope_tables(1000000.0, 32768)
+    cl, sl = oracle.rope_tables(10000.0, 32768)
+    return (cg, sg), (cl, sl)
+
+
+def build(tg, oracle, weight_images, tables, name, own_tables=False):
+    shape, n_layers, seed, n_prompt, nd, nt, gsize = gi.MODEL_CASES[name]
+    image = weight_images(shape, n_layers, seed)
+    model = tg.Transformer(tg.named_config(shape, n_layers))
+    model.read_weights_mem(image)
+    if own_tables:
+        sess = model.session(gsize=gsize)
+    else:
+        sess = model.session(rope=tables[0], rope_sw=tables[1], gelu_table=oracle.gelu_table(-4.0, 4.0, gsize))
+    osess = oracle.model(gi.oracle_config(shape, n_layers), image=image).session(-4.0, 4.0, gsize)
+    return model, sess, osess, gi.prompt_ids(seed, n_prompt)
+
+
+def compare_run(sess, osess, prompt, n_decode, tol, tol_first):
+    tok, logits = sess.prefill(prompt)
+    otok, ologits, otaps = osess.prefill(prompt, taps=True)
+    taps = sess.taps(rows=prompt.size)
+    assert taps.shape[0] == otaps.shape[0] + 1
+    assert normrel(taps[1], otaps[0]) < tol_first      # attention block of layer 0: nothing discontinuous upstream
+    worst = max(normrel(taps[b + 1], otaps[b]) for b in range(otaps.shape[0]))
+    assert worst < tol, worst
+    assert normrel(logits, ologits) < tol
+    assert tok == otok
+    toks = [tok]
+    for _ in range(n_decode):
+        tok, logits = sess.decode(toks[-1])
+        otok, ologits, otp = osess.decode(toks[-1], taps=True)
+        dt = sess.taps(rows=1)[:, 0, :]
+        worst = max(worst, max(normrel(dt[b + 1], otp[b]) for b in range(otp.shape[0])))
+        assert normrel(logits, ologits) < tol
+        assert tok == otok
+        toks.append(tok)
+    assert worst < tol, worst
+    return np.array(toks, np.int32), worst
+
+
+def test_embedding_tap_is_exact(tg, oracle, weight_images, tables):
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
+    sess.prefill(prompt, want_logits=False)
+    image = weight_images("270m", 6, 11)
+    wte = image[:262144 * 640].view(np.int8).reshape(262144, 640)
+    sc = image[262144 * 640:262144 * 640 + 4 * 640].view(np.float32)
+    assert np.array_equal(sess.tap(0, rows=prompt.size), oracle.embedding(prompt, wte, sc))
+
+
+def test_small_model_fine_table(tg, oracle, golden, weight_images, tables):
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut")
+    toks, worst = compare_run(sess, osess, prompt, 12, tol=5e-5, tol_first=3e-6)
+    assert np.array_equal(toks, golden["model/small6_finelut/tokens"])
+    # and against the compiled reference's own activations (its rope tables differ in the last bits)
+    sess.reset()
+    sess.prefill(prompt)
+    taps = sess.taps(rows=prompt.size)[1:]
+    assert normrel(taps[:, gi.tap_rows(prompt.size), :], golden["model/small6_finelut/prefill_taps"]) < 2e-4
+
+
+def test_small_model_cli_table(tg, oracle, golden, weight_images, tables):
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
+    toks, worst = compare_run(sess, osess, prompt, 12, tol=5e-3, tol_first=3e-6)
+    assert np.array_equal(toks, golden["model/small6/tokens"])
+
+
+def test_library_built_tables(tg, oracle, golden, weight_images, tables):
+    """NULL tables: the library computes RoPE and GeLU tables itself (decode.hpp:176-201, ops.hpp:29-39)."""
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut", own_tables=True)
+    toks, worst = compare_run(sess, osess, prompt, 4, tol=5e-5, tol_first=3e-6)
+
+
+def test_prompt_longer_than_window(tg, oracle, golden, weight_images, tables):
+    """600-token prompt on a model with 512-slot ring caches: 513-key window in prefill
+    (ops.hpp:437-443), ring of 512 in decode, tail of the prompt in slots 0..511 (decode.hpp:84-104)."""
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_window")
+    nd = gi.MODEL_CASES["small6_window"][4]
+    tok, logits = sess.prefill(prompt)
+    otok, ologits, otaps = osess.prefill(prompt, taps=True)
+    taps = sess.taps(rows=prompt.size)
+    assert normrel(taps[1], otaps[0]) < 3e-6
+    assert normrel(taps[1:], otaps) < 5e-3 and normrel(logits, ologits) < 5e-3 and tok == otok
+    k0, v0, pp, bp = sess.kv(0)
+    ok0, ov0, opp, obp = osess.kv(0)
+    assert (pp, bp) == (opp, obp) == (600, 512)
+    assert normrel(k0, ok0) < 3e-6 and normrel(v0, ov0) < 3e-6  # layer 0: rows 88..599 of the prompt in slots 0..511
+    toks = [tok]
+    for _ in range(nd):
+        tok, logits = sess.decode(toks[-1])
+        otok, ologits, _ = osess.decode(toks[-1])
+        assert tok == otok and normrel(logits, ologits) < 5e-3
+        toks.append(tok)
+    assert np.array_equal(np.array(toks, np.int32), golden["model/small6_window/tokens"])
+    for layer in (0, 5):
+        k, v, pp, bp = sess.kv(layer)
+        ok, ov, opp, obp = osess.kv(layer)
+        assert (pp, bp) == (opp, obp)
+        n = 512 if layer == 0 else 600 + nd
+        assert normrel(k[:n], ok[:n]) < 5e-3 and normrel(v[:n], ov[:n]) < 5e-3
+    assert (sess.kv(0)[2], sess.kv(0)[3]) == (600 + nd, 512 + nd)
+
+
+def test_decode_from_empty_session(tg, oracle, weight_images, tables):
+    """forward_decode without a prefill: position 0, a single key."""
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut")
+    tok = int(prompt[0])
+    for _ in range(3):
+        t, lg = sess.decode(tok)
+        ot, olg, _ = osess.decode(tok)
+        assert t == ot and normrel(lg, olg) < 5e-5
+        tok = t
+    assert sess.position == 3
+
+
+def greedy_vs_golden(sess, golden, name, prompt, n_decode):
+    toks, s_prefill, s_decode = sess.greedy(prompt, n_decode)
+    ref = golden[f"model/{name}/tokens"]
+    gaps = golden[f"model/{name}/top2_gaps"]
+    mism = np.nonzero(toks != ref)[0]
+    if mism.size:
+        # only a genuine near-tie of the reference's own logits may flip
+        assert gaps[mism[0]] < 2e-3, f"first mismatch at step {mism[0]}, reference top-2 gap {gaps[mism[0]]}"
+        pytest.fail(f"greedy ids diverge from the reference at step {mism[0]} (a near-tie: top-2 gap {gaps[mism[0]]:.2e})")
+    return s_prefill, s_decode
+
+
+def test_full_270m_greedy_ids(tg, oracle, golden, weight_images, tables):
+    """64-token prompt + 256 greedy steps, 18 layers: ids identical to the compiled reference."""
+    import hashlib
+    image = weight_images("270m", 18, 1)
+    assert hashlib.sha256(image.tobytes()).hexdigest() == str(golden["model/full270m/weights_sha"])
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full270m")
+    greedy_vs_golden(sess, golden, "full270m", prompt, 256)
+
+
+def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
+    """178-token prompt + 1024 greedy steps, 26 layers (the benchmark workload)."""
+    if "model/full1B/tokens" not in golden:
+        pytest.skip("fixture was written without the 1B case")
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full1B")
+    greedy_vs_golden(sess, golden, "full1B", prompt, 1024)
+    # last-position activations of the prefill against the reference's
+    sess.reset()
+    tok, logits = sess.prefill(prompt)
+    assert normrel(logits[:4096], golden["model/full1B/prefill_logits_head"]) < 2e-2
+    last = sess.taps(rows=prompt.size)[1:, -1, :]
+    assert normrel(last, golden["model/full1B/prefill_taps_last"]) < 2e-2
+
+
+def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
+    """HIP-graph replay must give the same bits as plain launches, on every replay."""
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
+    results = []
+    for graphs in (0, 1, 1):
+        tg.lib().tg_set_graphs(graphs)
+        sess.reset()
+        sess.prefill(prompt, want_logits=False)
+        chunks = []
+        for n in (1, 5, 9):  # several enqueue calls with host work and synchronisation between replays
+            sess.decode_enqueue(n)
+            tg.synchronize()
+            chunks.append(sess.taps(rows=1).copy())
+        results.append((sess.read_ids(16).copy(), chunks))
+    tg.lib().tg_set_graphs(1)
+    for ids, chunks in results[1:]:
+        assert np.array_equal(ids, results[0][0])
+        for a, b in zip(chunks, results[0][1]):
+            assert np.array_equal(a, b)
+
+
+def test_long_context_merge_path(tg, oracle, weight_images, tables):
+    """More than 4096 keys on a global layer: 128-key chunks plus the merge launch."""
+    cfg_o = gi.oracle_config("270m", 2)
+    cfg_o.pattern = 2  # layer 0 local, layer 1 global
+    image = oracle.generate_weights(cfg_o, 21)
+    cfg = tg.named_config("270m", 2)
+    cfg.window_pattern = 2
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(image)
+    table = oracle.gelu_table(-4.0, 4.0, 1 << 20)
+    sess = model.session(rope=tables[0], rope_sw=tables[1], gelu_table=table)
+    osess = oracle.model(cfg_o, image=image).session(-4.0, 4.0, 1 << 20)
+    prompt = gi.prompt_ids(21, 4100)
+    tok, logits = sess.prefill(prompt)
+    otok, ologits, _ = osess.prefill(prompt)
+    assert tok == otok and normrel(logits, ologits) < 5e-5
+    for _ in range(3):
+        t, lg = sess.decode(tok)
+        ot, olg, _ = osess.decode(tok)
+        assert t == ot and normrel(lg, olg) < 5e-5
+        tok = t
+
+
+def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
+    sess.prefill(prompt[:8], want_logits=False)
+    with pytest.raises(tg.TgError) as e:       # one prefill per DecodeState (decode.hpp:78-79)
+        sess.prefill(prompt[:8], want_logits=False)
+    assert e.value.code == -7
+    m2 = tg.Transformer(tg.named_config("270m", 6))
+    with pytest.raises(tg.TgError) as e:       # transformer.hpp:163
+        m2.read_weights(str(tmp_path / "missing.bin"))
+    assert e.value.code == -2 and "Could not open file." in str(e.value)
+    short = tmp_path / "short.bin"
+    weight_images("270m", 6, 11)[:10_000_000].tofile(short)
+    with pytest.raises(tg.TgError) as e:
+        m2.read_weights(str(short))
+    assert e.value.code == -3
+    with pytest.raises(tg.TgError) as e:       # no weights yet
+        m2.session()
+    assert e.value.code == -7
+    bad = tg.named_config("270m", 2)
+    bad.hidden_size = 512
+    with pytest.raises(tg.TgError) as e:
+        tg.Transformer(bad)
+    assert e.value.code == -1

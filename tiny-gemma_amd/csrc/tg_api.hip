@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <map>
 
 #include "tg_internal.h"
 
@@ -18,6 +19,7 @@ namespace {
 
 thread_local std::string g_err;
 bool g_inited = false;
+bool g_use_graphs = true;
 int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
@@ -202,6 +204,7 @@ struct tg_session {
 	int pos = 0, bp_local = 0, bp_global = 0, steps = 0;  // host mirrors
 	float *taps = nullptr;    // prefill taps [(2L+1)][rows][hidden] (kept only for short prompts)
 	int tap_rows = 0;
+	std::map<uint64_t, hipGraphExec_t> graphs;  // captured decode steps, keyed by the attention launch geometry
 };
 
 namespace {
@@ -585,6 +588,8 @@ static int upload_rope(float **cos_d, float **sin_d, const float *cos_h, const f
 void tg_session_destroy(tg_session *s) {
 	if (!s) return;
 	(void)hipStreamSynchronize(g_stream);
+	for (auto &kv : s->graphs) (void)hipGraphExecDestroy(kv.second);
+	s->graphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
 	              s->tok_log, s->taps};
@@ -719,7 +724,7 @@ struct StepProfile {
 	}
 };
 
-static int enqueue_decode_step(tg_session *s, StepProfile *prof) {
+static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid) {
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
 	const int L = c.n_layers, h = c.hidden_size;
@@ -771,7 +776,11 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof) {
 		a.part_ml = s->part_ml;
 		a.n_head = c.n_head;
 		TG_MARK(TG_KC_ATTN);
-		tg_launch_attn_decode(a, (valid + a.chunk - 1) / a.chunk, g_stream);
+		// a captured step is replayed at later positions with the same chunk: launch the largest grid that
+		// chunk can need (workgroups past the valid keys exit at once)
+		const int nblk = full_grid ? (needs_merge ? (a.max_pos + a.chunk - 1) / a.chunk : TG_ATTN_MERGE_MAX)
+		                           : (valid + a.chunk - 1) / a.chunk;
+		tg_launch_attn_decode(a, nblk, g_stream);
 		if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream);
 		// --- merge of the attention partials + O projection (modules.hpp:161-164)
 		g = gemv_base(Ld.o);
@@ -833,7 +842,7 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof) {
 int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax) {
 	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
 	TG_HIP(hipMemcpyAsync(s->ctr + 4, &id, sizeof(int), hipMemcpyHostToDevice, g_stream));
-	if (int rc = enqueue_decode_step(s, nullptr)) return rc;
+	if (int rc = enqueue_decode_step(s, nullptr, false)) return rc;
 	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)s->m->cfg.n_vocab, hipMemcpyDeviceToHost, g_stream));
 	int32_t tok = -1;
 	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
@@ -847,16 +856,63 @@ int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax)
 	return TG_OK;
 }
 
+static uint64_t decode_graph_key(const tg_session *s) {
+	const tg_config &c = s->m->cfg;
+	bool ml = false, mg = false;
+	const int cl = attn_chunk_for(std::min(s->pos + 1, c.n_pos_local), &ml);
+	const int cg = attn_chunk_for(std::min(s->pos + 1, c.n_pos), &mg);
+	return (uint64_t)cl | ((uint64_t)ml << 15) | ((uint64_t)cg << 16) | ((uint64_t)mg << 31);
+}
+
 int tg_decode_enqueue(tg_session *s, int n_steps) {
 	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
-	for (int i = 0; i < n_steps; i++)
-		if (int rc = enqueue_decode_step(s, nullptr)) return rc;
+	const tg_config &c = s->m->cfg;
+	for (int i = 0; i < n_steps; i++) {
+		if (!g_use_graphs) {
+			if (int rc = enqueue_decode_step(s, nullptr, false)) return rc;
+			continue;
+		}
+		// One HIP graph per attention launch geometry; every other launch parameter of a decode step
+		// is position independent (positions and the token id live in device memory).
+		const uint64_t key = decode_graph_key(s);
+		auto it = s->graphs.find(key);
+		if (it == s->graphs.end()) {
+			TG_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+			const int rc = enqueue_decode_step(s, nullptr, true);  // advances the host mirrors once
+			hipGraph_t graph = nullptr;
+			const hipError_t e = hipStreamEndCapture(g_stream, &graph);
+			if (rc != TG_OK) {
+				if (graph) (void)hipGraphDestroy(graph);
+				return rc;
+			}
+			if (e != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+			hipGraphExec_t exec = nullptr;
+			const hipError_t e2 = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+			(void)hipGraphDestroy(graph);
+			if (e2 != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e2));
+			s->graphs[key] = exec;
+			TG_HIP(hipGraphLaunch(exec, g_stream));
+		} else {
+			if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
+			if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
+			TG_HIP(hipGraphLaunch(it->second, g_stream));
+			s->pos += 1;
+			s->bp_local += 1;
+			s->bp_global += 1;
+			s->steps += 1;
+		}
+	}
 	if (s->taps) {
 		TG_HIP(hipStreamSynchronize(g_stream));
 		(void)hipFree(s->taps);
 		s->taps = nullptr;
 		s->tap_rows = 0;
 	}
+	return TG_OK;
+}
+
+int tg_set_graphs(int enable) {
+	g_use_graphs = enable != 0;
 	return TG_OK;
 }
 
@@ -870,7 +926,7 @@ int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches)
 	int rc = TG_OK;
 	for (int i = 0; i < n_steps && rc == TG_OK; i++) {
 		prof.used = 0;
-		rc = enqueue_decode_step(s, &prof);
+		rc = enqueue_decode_step(s, &prof, false);
 		if (rc != TG_OK) break;
 		if (hipStreamSynchronize(g_stream) != hipSuccess) {
 			rc = tg_fail(TG_ERR_HIP, "hipStreamSynchronize failed");
