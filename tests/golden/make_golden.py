@@ -96,8 +96,14 @@ def main():
         prompt = gi.prompt_ids(seed, n_prompt)
         tok, logits, taps = sess.prefill(prompt, taps=True)
         toks = [tok]
-        srt = np.partition(logits, -2)[-2:]
-        gaps = [float(srt[1] - srt[0])]
+
+        def top2(lg):
+            i = np.argpartition(lg, -2)[-2:]
+            i = i[np.argsort(lg[i])][::-1]
+            return float(lg[i[0]] - lg[i[1]]), (int(i[0]), int(i[1]))
+
+        gap, pair = top2(logits)
+        gaps, pairs = [gap], [pair]
         out[f"model/{name}/prefill_logits_head"] = logits[:4096].copy()
         out[f"model/{name}/prefill_logits_sha"] = sha(logits)
         out[f"model/{name}/prefill_logits_norm"] = np.float64(np.linalg.norm(logits.astype(np.float64)))
@@ -118,13 +124,15 @@ def main():
             want = step < n_tap_steps
             tok, logits, tp = sess.decode(toks[-1], want_logits=True, taps=want)
             toks.append(tok)
-            srt = np.partition(logits, -2)[-2:]
-            gaps.append(float(srt[1] - srt[0]))
+            gap, pair = top2(logits)
+            gaps.append(gap)
+            pairs.append(pair)
             if want:
                 dec_taps.append(tp)
                 dec_logits_head.append(logits[:4096].copy())
         out[f"model/{name}/tokens"] = np.array(toks, np.int32)
         out[f"model/{name}/top2_gaps"] = np.array(gaps, np.float32)
+        out[f"model/{name}/top2_ids"] = np.array(pairs, np.int32)
         if dec_taps:
             out[f"model/{name}/decode_taps"] = np.stack(dec_taps)
             out[f"model/{name}/decode_logits_head"] = np.stack(dec_logits_head)

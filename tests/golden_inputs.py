@@ -47,7 +47,8 @@ MODEL_CASES = {
     "small6": ("270m", 6, 11, 70, 12, 4, 1024),           # one global layer (l = 5), short prompt
     "small6_window": ("270m", 6, 12, 600, 6, 3, 1024),    # prompt longer than the 512-slot ring
     "small6_finelut": ("270m", 6, 11, 70, 12, 4, 1 << 20),  # near-continuous GeLU table: tight end-to-end check
-    "full270m": ("270m", 18, 1, 64, 256, 2, 1024),        # 64-token prompt + 256 greedy steps
+    "full270m": ("270m", 18, 5, 64, 256, 2, 1024),        # 64-token prompt + 256 greedy steps
+    "full270m_ties": ("270m", 18, 1, 64, 256, 0, 1024),   # same, a seed whose greedy path crosses near-ties of the logits
     "full1B": ("1B", 26, 1, 178, 1024, 2, 1024),          # 178-token prompt + 1024 greedy steps
 }
 

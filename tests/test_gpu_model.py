@@ -138,28 +138,55 @@ def test_decode_from_empty_session(tg, oracle, weight_images, tables):
 def greedy_vs_golden(sess, golden, name, prompt, n_decode):
     toks, s_prefill, s_decode = sess.greedy(prompt, n_decode)
     ref = golden[f"model/{name}/tokens"]
-    gaps = golden[f"model/{name}/top2_gaps"]
     mism = np.nonzero(toks != ref)[0]
-    if mism.size:
-        # only a genuine near-tie of the reference's own logits may flip
-        assert gaps[mism[0]] < 2e-3, f"first mismatch at step {mism[0]}, reference top-2 gap {gaps[mism[0]]}"
-        pytest.fail(f"greedy ids diverge from the reference at step {mism[0]} (a near-tie: top-2 gap {gaps[mism[0]]:.2e})")
-    return s_prefill, s_decode
+    assert mism.size == 0, (f"greedy ids diverge from the reference at step {mism[0]} "
+                            f"(reference top-2 gap there: {golden[f'model/{name}/top2_gaps'][mism[0]]:.3e})")
+
+
+def check_weights(golden, weight_images, name):
+    import hashlib
+    shape, n_layers, seed = gi.MODEL_CASES[name][:3]
+    assert hashlib.sha256(weight_images(shape, n_layers, seed).tobytes()).hexdigest() == str(golden[f"model/{name}/weights_sha"])
 
 
 def test_full_270m_greedy_ids(tg, oracle, golden, weight_images, tables):
     """64-token prompt + 256 greedy steps, 18 layers: ids identical to the compiled reference."""
-    import hashlib
-    image = weight_images("270m", 18, 1)
-    assert hashlib.sha256(image.tobytes()).hexdigest() == str(golden["model/full270m/weights_sha"])
+    check_weights(golden, weight_images, "full270m")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full270m")
     greedy_vs_golden(sess, golden, "full270m", prompt, 256)
+    sess.reset()
+    tok, logits = sess.prefill(prompt)
+    # 18 layers of the 1024-entry table: the checker itself sits 4e-3 from the compiled reference here
+    assert normrel(logits[:4096], golden["model/full270m/prefill_logits_head"]) < 1e-2
+
+
+def test_full_270m_near_ties(tg, oracle, golden, weight_images, tables):
+    """A seed whose greedy path crosses near-ties of the reference's own logits (top-2 gaps down to
+    3e-4 against a logit spread of 0.5).  Teacher-forced with the reference's ids, every step must
+    pick the reference's id, except that at a near-tie (gap < 0.02) the reference's runner-up is the
+    only other acceptable answer."""
+    check_weights(golden, weight_images, "full270m_ties")
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full270m_ties")
+    ref = golden["model/full270m_ties/tokens"]
+    gaps = golden["model/full270m_ties/top2_gaps"]
+    pairs = golden["model/full270m_ties/top2_ids"]
+    tok, _ = sess.prefill(prompt, want_logits=False)
+    picks = [tok]
+    for i in range(256):
+        tok, _ = sess.decode(int(ref[i]), want_logits=False)
+        picks.append(tok)
+    picks = np.array(picks, np.int32)
+    mism = np.nonzero(picks != ref)[0]
+    assert mism.size <= 4, mism
+    for i in mism:
+        assert gaps[i] < 0.02 and picks[i] == pairs[i][1], (i, gaps[i], picks[i], pairs[i])
 
 
 def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
     """178-token prompt + 1024 greedy steps, 26 layers (the benchmark workload)."""
     if "model/full1B/tokens" not in golden:
         pytest.skip("fixture was written without the 1B case")
+    check_weights(golden, weight_images, "full1B")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full1B")
     greedy_vs_golden(sess, golden, "full1B", prompt, 1024)
     # last-position activations of the prefill against the reference's

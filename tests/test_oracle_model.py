@@ -71,14 +71,10 @@ def test_prompt_longer_than_window(oracle, golden, weight_images):
 def test_full_270m_greedy_ids(oracle, golden, weight_images):
     """64-token prompt + 256 greedy steps on the 18-layer 270m shape."""
     sess, toks, logits, taps, dtaps = run_case(oracle, weight_images, "full270m", taps_steps=0)
-    ref = golden["model/full270m/tokens"]
-    gaps = golden["model/full270m/top2_gaps"]
-    mism = np.nonzero(toks != ref)[0]
-    if mism.size:  # only acceptable at a genuine near-tie of the reference's own logits
-        assert gaps[mism[0]] < 2e-3, (mism[0], gaps[mism[0]])
-    else:
-        assert np.array_equal(toks, ref)
+    assert np.array_equal(toks, golden["model/full270m/tokens"])
+    # 18 layers of the 1024-entry table between a strict-IEEE and a -ffast-math build
     assert normrel(logits[:4096], golden["model/full270m/prefill_logits_head"]) < 1e-2
+    assert normrel(taps[:, -1, :], golden["model/full270m/prefill_taps_last"]) < 1e-2
 
 
 def test_1b_prefill_and_first_steps(oracle, golden, weight_images):
