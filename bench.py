@@ -95,7 +95,11 @@ def main():
     ap.add_argument("--seed", type=int, default=20251)
     ap.add_argument("--cpu-steps", type=int, default=128, help="decode steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=32)
-    ap.add_argument("--no-graphs", action="store_true", help="plain stream launches instead of HIP graph replay")
+    ap.add_argument("--graphs", action="store_true", help="replay captured HIP graphs instead of plain stream launches")
+    ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
+    ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
+    ap.add_argument("--counter-run", action="store_true",
+                    help="for rocprofv3 --pmc: prefill, a few decode steps and 4 launches of a 256 MiB copy kernel; no timing")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is single-GPU (batch-1 decode has no data parallelism to spread); run with --gpus 1",
@@ -106,7 +110,11 @@ def main():
     from tiny_gemma_amd import weights as tgw
 
     dev = tg.init(0)
-    tg.lib().tg_set_graphs(0 if args.no_graphs else 1)
+    tg.lib().tg_set_graphs(1 if args.graphs else 0)
+    if args.prefetch_blocks is not None:
+        tg.check(tg.lib().tg_set_prefetch_blocks(args.prefetch_blocks))
+    if args.gemv_max_blocks is not None:
+        tg.lib().tg_set_gemv_max_blocks(args.gemv_max_blocks)
     n_prompt, step_bytes, lm_bytes = MODELS[args.model]
     cfg = tg.named_config(args.model)
     if n_prompt + args.warmup + args.steps + args.profile_steps + 1 > cfg.n_pos:
@@ -129,6 +137,16 @@ def main():
     t0 = time.perf_counter()
     sess.prefill(prompt, want_logits=False)
     t_prefill = time.perf_counter() - t0
+
+    if args.counter_run:
+        sess.decode_enqueue(min(args.steps, 8))
+        n = 256 << 20
+        a, b = tg.DeviceBuffer(n), tg.DeviceBuffer(n)
+        for _ in range(4):
+            tg.check(tg.lib().tg_dev_copy(b.p, a.p, n))
+        tg.synchronize()
+        print(json.dumps({"counter_run": True, "copy_bytes": n}))
+        return
 
     ev = HipEvents()
     stream = tg.lib().tg_stream()
@@ -175,7 +193,7 @@ def main():
             "prompt_tokens": n_prompt,
             "decode_position_start": n_prompt + args.warmup,
             "seed": args.seed,
-            "launch": "stream" if args.no_graphs else "hipGraph replay",
+            "launch": "hipGraph replay" if args.graphs else "stream",
         },
         "roofline": {
             "kernel": "tg_gemv_lmhead_argmax",

@@ -80,6 +80,9 @@ int tg_dev_alloc(void **p, size_t bytes);
 int tg_dev_free(void *p);
 int tg_copy_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int tg_copy_d2h(void *dst_host, const void *src_dev, size_t bytes);
+/* device-to-device streaming copy kernel (bytes % 16 == 0), asynchronous: the known-size kernel
+ * that hardware byte counters are calibrated against */
+int tg_dev_copy(void *dst_dev, const void *src_dev, size_t bytes);
 /* y_dev[outDim] = scales * (x_dev . W); asynchronous on tg_stream(); overwrites y_dev */
 int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logits_variant);
 /* C_dev[m][outDim] = scales * (A_dev[m][inDim] . W); asynchronous */
@@ -120,8 +123,13 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 /* Enqueues n_steps decode steps without host synchronisation (each step feeds the device-side
  * argmax of the previous one).  Ids are read back with tg_session_read_ids after tg_synchronize. */
 int tg_decode_enqueue(tg_session *s, int n_steps);
-/* tg_decode_enqueue replays captured HIP graphs of a decode step by default; 0 = plain stream launches */
+/* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
 int tg_set_graphs(int enable);
+/* tuning knob: a GEMV launch uses at most n workgroups, which then loop over column tiles (0: one per tile) */
+int tg_set_gemv_max_blocks(int n);
+/* tuning knob: extra workgroups per decode launch that pull the NEXT launch's weights out of HBM into
+ * the caches while the current launch is latency bound (multiple of 8; 0 = off).  A hint only. */
+int tg_set_prefetch_blocks(int n);
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
 
 /* Kernel classes of one decode step, in launch order per layer; the head runs once per step. */
@@ -129,6 +137,10 @@ enum { TG_KC_QKV = 0, TG_KC_ATTN, TG_KC_OPROJ, TG_KC_UPGATE, TG_KC_DOWN, TG_KC_L
 /* Runs n_steps decode steps like tg_decode_enqueue, with a HIP event recorded on tg_stream()
  * before every launch: ms_sum[k] / launches[k] is the average event-to-event time of class k. */
 int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches);
+/* Re-launches the kernel of class k (layer `layer`; the head ignores it) of the NEXT decode step `repeat`
+ * times on the session's current buffers, back to back, without advancing the session: for timing one
+ * kernel in isolation with events on tg_stream().  The kernels are idempotent on their inputs. */
+int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repeat);
 
 /* Debug taps: the residual stream of the most recent forward after block b
  * (b = 0: embedding; 2l+1: after attention of layer l; 2l+2: after the MLP of layer l).

@@ -211,7 +211,7 @@ def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
             tg.synchronize()
             chunks.append(sess.taps(rows=1).copy())
         results.append((sess.read_ids(16).copy(), chunks))
-    tg.lib().tg_set_graphs(1)
+    tg.lib().tg_set_graphs(0)
     for ids, chunks in results[1:]:
         assert np.array_equal(ids, results[0][0])
         for a, b in zip(chunks, results[0][1]):

@@ -74,6 +74,7 @@ def lib():
     L.tg_dev_free.argtypes = [C.c_void_p]
     L.tg_copy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
     L.tg_copy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    L.tg_dev_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
     L.tg_qgemv_dev.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_qgemm_dev.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_model_create.argtypes = [C.POINTER(Config), C.POINTER(C.c_void_p)]

@@ -19,7 +19,9 @@ namespace {
 
 thread_local std::string g_err;
 bool g_inited = false;
-bool g_use_graphs = true;
+int g_prefetch_blocks = 128;   // extra workgroups per launch that prefetch the next launch's weights (0: off; multiple of 8)
+int g_gemv_max_blocks = 1024;  // workgroups per GEMV launch before workgroups start looping over tiles
+bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GPU-side dispatch, not by host launches)
 int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
@@ -148,7 +150,18 @@ TgGemv gemv_base(const PackedMat &p) {
 	g.ntiles = p.ntiles;
 	g.C = p.C;
 	g.lc_shift = p.lc_shift;
+	g.max_blocks = g_gemv_max_blocks;
 	return g;
+}
+
+// Prefetch job for the GEMV tiles of `p` (see TgPrefetch).
+TgPrefetch prefetch_of(const PackedMat &p) {
+	TgPrefetch f;
+	f.ptr = g_prefetch_blocks > 0 ? p.W : nullptr;
+	f.slab = (uint32_t)p.K * (uint32_t)p.C;
+	f.ntiles = p.ntiles;
+	f.nblocks = g_prefetch_blocks;
+	return f;
 }
 
 int upload_floats(float **dst, const float *src, size_t n) {
@@ -309,6 +322,12 @@ int tg_dev_free(void *p) {
 int tg_copy_h2d(void *dst, const void *src, size_t bytes) {
 	TG_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
 	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+int tg_dev_copy(void *dst, const void *src, size_t bytes) {
+	if (!dst || !src || bytes % 16) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	tg_launch_copy(dst, src, bytes, g_stream);
+	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
 int tg_copy_d2h(void *dst, const void *src, size_t bytes) {
@@ -724,12 +743,22 @@ struct StepProfile {
 	}
 };
 
-static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid) {
+// For tg_debug_repeat_kernel: launch only the kernels of one class of one layer, `repeat` times.
+struct StepOnly {
+	int kclass, layer, repeat;
+};
+
+static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid, const StepOnly *only = nullptr) {
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
 	const int L = c.n_layers, h = c.hidden_size;
 	if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
 	if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
+#define TG_DO(k, l, stmt)                                                        \
+	if (!only || (only->kclass == (k) && only->layer == (l)))                        \
+		for (int r_ = 0; r_ < (only ? only->repeat : 1); r_++) {                     \
+			stmt;                                                                    \
+		}
 #define TG_MARK(k)                                 \
 	if (prof) {                                    \
 		TG_HIP(prof->mark(k));                     \
@@ -742,6 +771,7 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 		g.w_pre = Ld.apre;
 		g.xr_out = s->xr + (size_t)(2 * l) * h;
 		g.y = s->qkv;
+		g.pf = prefetch_of(Ld.o);
 		TG_MARK(TG_KC_QKV);
 		if (l == 0) {
 			g.wte = m->wte;
@@ -749,12 +779,12 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 			g.tok = s->ctr + 4;
 			g.vocab = c.n_vocab;
 			g.emb_scale = (float)sqrt((double)h);  // ops.hpp:586
-			tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream);
+			TG_DO(TG_KC_QKV, l, tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream));
 		} else {
 			g.pend = s->d_out;
 			g.w_post = m->L[(size_t)l - 1].mpost;
 			g.x = s->xr + (size_t)(2 * l - 1) * h;
-			tg_launch_gemv(g, TG_ROLE_QKV, g_stream);
+			TG_DO(TG_KC_QKV, l, tg_launch_gemv(g, TG_ROLE_QKV, g_stream));
 		}
 		// --- q/k norm, RoPE, KV write, attention (modules.hpp:146-161)
 		TgAttnDecode a;
@@ -775,13 +805,13 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 		a.part_acc = s->part_acc;
 		a.part_ml = s->part_ml;
 		a.n_head = c.n_head;
+		a.pf = prefetch_of(Ld.ug);
 		TG_MARK(TG_KC_ATTN);
 		// a captured step is replayed at later positions with the same chunk: launch the largest grid that
 		// chunk can need (workgroups past the valid keys exit at once)
 		const int nblk = full_grid ? (needs_merge ? (a.max_pos + a.chunk - 1) / a.chunk : TG_ATTN_MERGE_MAX)
 		                           : (valid + a.chunk - 1) / a.chunk;
-		tg_launch_attn_decode(a, nblk, g_stream);
-		if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream);
+		TG_DO(TG_KC_ATTN, l, tg_launch_attn_decode(a, nblk, g_stream); if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream));
 		// --- merge of the attention partials + O projection (modules.hpp:161-164)
 		g = gemv_base(Ld.o);
 		g.pos = s->ctr;
@@ -790,8 +820,9 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 		g.part_acc = needs_merge ? s->merged_acc : s->part_acc;
 		g.part_ml = needs_merge ? s->merged_ml : s->part_ml;
 		g.y = s->o_out;
+		g.pf = prefetch_of(Ld.d);
 		TG_MARK(TG_KC_OPROJ);
-		tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream);
+		TG_DO(TG_KC_OPROJ, l, tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream));
 		// --- post-norm + residual, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
 		g = gemv_base(Ld.ug);
 		g.hidden = h;
@@ -805,14 +836,15 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 		g.gmin = s->gmin;
 		g.geps = s->geps;
 		g.lut_size = s->lut_size;
+		if (l + 1 < L) g.pf = prefetch_of(m->L[(size_t)l + 1].qkv);
 		TG_MARK(TG_KC_UPGATE);
-		tg_launch_gemv(g, TG_ROLE_UPGATE, g_stream);
+		TG_DO(TG_KC_UPGATE, l, tg_launch_gemv(g, TG_ROLE_UPGATE, g_stream));
 		// --- down projection (modules.hpp:216-217)
 		g = gemv_base(Ld.d);
 		g.x = s->hbuf;
 		g.y = s->d_out;
 		TG_MARK(TG_KC_DOWN);
-		tg_launch_gemv(g, TG_ROLE_DOWN, g_stream);
+		TG_DO(TG_KC_DOWN, l, tg_launch_gemv(g, TG_ROLE_DOWN, g_stream));
 	}
 	// --- last post-norm + residual, final norm, LM head, argmax (modules.hpp:242-246, ops.hpp:744)
 	TgGemv g = gemv_base(m->lm);
@@ -826,12 +858,14 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid)
 	g.blk_val = s->blk_val;
 	g.blk_idx = s->blk_idx;
 	TG_MARK(TG_KC_LMHEAD);
-	tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream);
+	TG_DO(TG_KC_LMHEAD, 0, tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream));
 	TG_MARK(TG_KC_ARGMAX);
-	tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
+	if (!only) tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
 	TG_MARK(-1);
 #undef TG_MARK
+#undef TG_DO
 	TG_HIP(hipGetLastError());
+	if (only) return TG_OK;
 	s->pos += 1;
 	s->bp_local += 1;
 	s->bp_global += 1;
@@ -908,6 +942,24 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 		s->taps = nullptr;
 		s->tap_rows = 0;
 	}
+	return TG_OK;
+}
+
+int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repeat) {
+	if (!s || kernel_class < 0 || kernel_class > TG_KC_LMHEAD || repeat < 1 || layer < 0 || layer >= s->m->cfg.n_layers)
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	StepOnly only{kernel_class, kernel_class == TG_KC_LMHEAD ? 0 : layer, repeat};
+	return enqueue_decode_step(s, nullptr, false, &only);
+}
+
+int tg_set_prefetch_blocks(int n) {
+	if (n < 0 || (n & 7)) return tg_fail(TG_ERR_BAD_ARG, "prefetch workgroups must be a non-negative multiple of 8");
+	g_prefetch_blocks = n;
+	return TG_OK;
+}
+
+int tg_set_gemv_max_blocks(int n) {
+	g_gemv_max_blocks = n;
 	return TG_OK;
 }
 

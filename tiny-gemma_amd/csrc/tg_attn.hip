@@ -101,6 +101,10 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	__shared__ float sc[NH][MAXCHUNK];
 	__shared__ float s_m[NH], s_l[NH];
 
+	if ((int)blockIdx.x >= a.nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
+		tg_prefetch_block(a.pf, a.nblocks);
+		return;
+	}
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int pos = a.pos[0];                      // position_ptr before this token (decode.hpp:154)
 	const int bp = a.pos[a.bp_index];           // buffer_ptr before this token (decode.hpp:59)
@@ -315,8 +319,11 @@ __global__ __launch_bounds__(ANT) void attn_prefill_kernel(float *o, const float
 
 }  // namespace
 
-void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s) {
-	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)max_blocks), dim3(ANT), 0, s, a);
+void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t s) {
+	TgAttnDecode a = a_in;
+	a.nblocks = max_blocks;
+	if (a.pf.ptr == nullptr) a.pf.nblocks = 0;
+	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(max_blocks + a.pf.nblocks)), dim3(ANT), 0, s, a);
 }
 
 void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s) {

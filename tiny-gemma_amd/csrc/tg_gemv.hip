@@ -26,9 +26,26 @@ namespace {
 
 constexpr int NT = 256;     // threads per workgroup (4 waves)
 constexpr int NWAVE = 4;
-constexpr int UNROLL = 4;   // 16-byte weight loads per lane per batch (two batches in flight)
+constexpr int DEPTH = 8;    // 16-byte weight loads in flight per lane
+constexpr uint32_t STEP_BYTES = NT * 16u;  // the workgroup reads 4 KiB of its slab per step
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#ifndef TG_W_AUX
+#define TG_W_AUX 0  // cache policy bits of the weight loads
+#endif
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+	return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ i32x4 ldw(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+	return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, TG_W_AUX);
+}
+__device__ __forceinline__ f32x4 ldx(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+	i32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+	return __builtin_bit_cast(f32x4, t);
+}
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -57,7 +74,7 @@ __device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin,
 	return lut[idx];
 }
 
-__device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const float4 xv) {
+__device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const f32x4 xv) {
 	const int d0 = v.x, d1 = v.y, d2 = v.z, d3 = v.w;
 	acc[0] = fmaf(xv.x, b2f(d0, 0), acc[0]); acc[0] = fmaf(xv.y, b2f(d0, 1), acc[0]);
 	acc[0] = fmaf(xv.z, b2f(d0, 2), acc[0]); acc[0] = fmaf(xv.w, b2f(d0, 3), acc[0]);
@@ -72,27 +89,43 @@ __device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const float4 
 template <int PRO, int EPI>
 __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
-	__shared__ __attribute__((aligned(16))) float red[NWAVE][TG_CT];
+	__shared__ __attribute__((aligned(16))) float red2[2][NWAVE][TG_CT];  // double buffered across the tile loop
 	__shared__ float sred[NWAVE];
 	__shared__ float wgt[4][TG_ATTN_MERGE_MAX];
-	__shared__ float s_bv[NWAVE];
-	__shared__ int s_bi[NWAVE];
+	__shared__ float s_bv[2][NWAVE];
+	__shared__ int s_bi[2][NWAVE];
 
+	if ((int)blockIdx.x >= g.nmain) {  // extra workgroups: prefetch the next launch's weights and leave
+		tg_prefetch_block(g.pf, g.nmain);
+		return;
+	}
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-	const int tile = blockIdx.x;
+	int tile = blockIdx.x;
 	const int C = g.C, LC = C >> 2, lcs = g.lc_shift;  // LC = 1 << lcs lanes across the tile's columns
 	const int KL = NT >> lcs;                          // lanes along K
-	const int cl = tid & (LC - 1), kpos = tid >> lcs;
+	const int kpos = tid >> lcs;
 	const int kgs = g.K >> 2;
-	const i32x4 *Wt = reinterpret_cast<const i32x4 *>(g.W) + (size_t)tile * kgs * LC + cl;
-	const int nit = (kgs + KL - 1) / KL;  // uniform trip count; lanes past the end are predicated off
+	const int nit = (kgs + KL - 1) / KL;  // steps; one step = the 256 lanes reading 4 KiB of the slab
 
-	// first batch of weight loads is issued before the prologue: it does not depend on x
-	i32x4 v[UNROLL];
+	// The tile slab and (for the PLAIN prologue) the input vector are read through buffer
+	// descriptors: the per-step address is a scalar offset, so addressing costs no vector
+	// instructions, and pieces past the end of the slab (lanes beyond K in the last step) read as 0.
+	const uint32_t slab = (uint32_t)g.K * (uint32_t)C;
+	__amdgpu_buffer_rsrc_t rw = make_rsrc(g.W + (size_t)tile * slab, slab);
+	const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.x, (PRO == TG_PRO_PLAIN) ? (uint32_t)g.K * 4u : 0u);
+	const uint32_t voff = (uint32_t)tid * 16u, xoff = (uint32_t)kpos * 16u, xstep = (uint32_t)KL * 16u;
+
+	// first DEPTH steps are issued before the prologue: they do not depend on it
+	i32x4 v[DEPTH];
+	f32x4 xq[DEPTH];
 #pragma unroll
-	for (int u = 0; u < UNROLL; u++) {
-		const int kg = kpos + u * KL;
-		v[u] = (u < nit && kg < kgs) ? __builtin_nontemporal_load(Wt + (size_t)kg * LC) : i32x4{0, 0, 0, 0};
+	for (int u = 0; u < DEPTH; u++) {
+		v[u] = i32x4{0, 0, 0, 0};
+		xq[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+		if (u < nit) {
+			v[u] = ldw(rw, voff, (uint32_t)u * STEP_BYTES);
+			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
+		}
 	}
 
 	// ---------------- prologue: input vector ----------------
@@ -152,7 +185,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			const float irms = 1.0f / sqrtf(ss / (float)h + eps);
 			for (int d = tid; d < h; d += NT) xs[d] = (xs[d] * irms) * (g.w_post[d] + 1.0f) + g.x[d];
 		}
-		if (g.xr_out != nullptr && tile == 0)
+		if (g.xr_out != nullptr && blockIdx.x == 0)
 			for (int d = tid; d < h; d += NT) g.xr_out[d] = xs[d];
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
 		float ss = 0.0f;
@@ -163,27 +196,56 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		__syncthreads();
 	}
 
-	// ---------------- main loop: stream the tile, next batch in flight while this one is consumed ----------------
+	// A workgroup walks tiles blockIdx.x, blockIdx.x + nmain, ...: the prologue above is paid once.
+	const int xlast = g.K - 4;
+	for (int it = 0;; it++) {
+	float(*red)[TG_CT] = red2[it & 1];
+	// ---------------- main loop: rotating pipeline of DEPTH loads per lane ----------------
 	float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-	for (int i0 = 0; i0 < nit; i0 += UNROLL) {
-		i32x4 vn[UNROLL];
+	auto xval = [&](int u, int step) -> f32x4 {
+		if (PRO == TG_PRO_PLAIN) return xq[u];
+		int idx = 4 * (kpos + step * KL);
+		idx = idx < xlast ? idx : xlast;  // lanes past K: their weights read as 0, any finite x will do
+		return *reinterpret_cast<const f32x4 *>(&xs[idx]);
+	};
+	int st = 0;
+	for (; st + 2 * DEPTH <= nit; st += DEPTH) {
 #pragma unroll
-		for (int u = 0; u < UNROLL; u++) {
-			const int kg = kpos + (i0 + UNROLL + u) * KL;
-			vn[u] = (i0 + UNROLL + u < nit && kg < kgs) ? __builtin_nontemporal_load(Wt + (size_t)kg * LC) : i32x4{0, 0, 0, 0};
+		for (int u = 0; u < DEPTH; u++) {
+			fma16(acc, v[u], xval(u, st + u));
+			v[u] = ldw(rw, voff, (uint32_t)(st + DEPTH + u) * STEP_BYTES);
+			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)(st + DEPTH + u) * xstep);
 		}
-		float4 xv[UNROLL];
+	}
+	// drain: fewer than 2*DEPTH steps left (all conditions are uniform)
 #pragma unroll
-		for (int u = 0; u < UNROLL; u++) {
-			int kg = kpos + (i0 + u) * KL;
-			kg = (kg < kgs) ? kg : 0;  // weights of a predicated-off piece are zero; any finite x will do
-			xv[u] = (PRO == TG_PRO_PLAIN) ? *reinterpret_cast<const float4 *>(g.x + 4 * kg)
-			                              : *reinterpret_cast<const float4 *>(&xs[4 * kg]);
+	for (int u = 0; u < DEPTH; u++) {
+		if (st + u < nit) {
+			fma16(acc, v[u], xval(u, st + u));
+			if (st + DEPTH + u < nit) {
+				v[u] = ldw(rw, voff, (uint32_t)(st + DEPTH + u) * STEP_BYTES);
+				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)(st + DEPTH + u) * xstep);
+			}
 		}
+	}
+	st += DEPTH;
 #pragma unroll
-		for (int u = 0; u < UNROLL; u++) fma16(acc, v[u], xv[u]);
+	for (int u = 0; u < DEPTH; u++)
+		if (st + u < nit) fma16(acc, v[u], xval(u, st + u));
+
+	// the next tile's first loads go out before this tile's reduction and epilogue
+	const int cur = tile;
+	tile += g.nmain;
+	const bool more = tile < g.ntiles;
+	if (more) {
+		rw = make_rsrc(g.W + (size_t)tile * slab, slab);
 #pragma unroll
-		for (int u = 0; u < UNROLL; u++) v[u] = vn[u];
+		for (int u = 0; u < DEPTH; u++) {
+			if (u < nit) {
+				v[u] = ldw(rw, voff, (uint32_t)u * STEP_BYTES);
+				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
+			}
+		}
 	}
 
 	// ---------------- reduction over the lanes along K (fixed order) ----------------
@@ -194,52 +256,52 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	if (lane < LC) *reinterpret_cast<float4 *>(&red[w][lane * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
 	__syncthreads();
 
-	// ---------------- epilogue ----------------
+	// ---------------- epilogue of tile `cur` ----------------
 	if (EPI == TG_EPI_STORE) {
 		if (tid < C) {
-			const int col = tile * C + tid;
+			const int col = cur * C + tid;
 			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
 			g.y[col] = sum * g.scales[col];
 		}
-		return;
-	}
-	if (EPI == TG_EPI_GEGLU) {
+	} else if (EPI == TG_EPI_GEGLU) {
 		// modules.hpp:211-215: gelu(gate) * up; the tile holds C/2 up columns, then the same C/2 gate columns
 		const int C2 = C >> 1;
 		if (tid < C2) {
 			const float su = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
 			const float sg = (red[0][tid + C2] + red[1][tid + C2]) + (red[2][tid + C2] + red[3][tid + C2]);
-			const float up = su * g.scales[tile * C + tid];
-			const float gate = sg * g.scales[tile * C + C2 + tid];
-			g.y[tile * C2 + tid] = gelu_lut(gate, g.lut, g.gmin, g.geps, g.lut_size) * up;
+			const float up = su * g.scales[cur * C + tid];
+			const float gate = sg * g.scales[cur * C + C2 + tid];
+			g.y[cur * C2 + tid] = gelu_lut(gate, g.lut, g.gmin, g.geps, g.lut_size) * up;
 		}
-		return;
-	}
-	// TG_EPI_LOGITS: logits + first stage of the greedy argmax
-	// (ops.hpp:749-757: strict '>' scan from index 0, so the lowest index wins ties)
-	float bv = -INFINITY;
-	int bi = 0x7fffffff;
-	if (tid < C) {
-		const int col = tile * C + tid;
-		const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
-		const float val = sum * g.scales[col];
-		if (g.y != nullptr) g.y[col] = val;
-		if (val > bv) { bv = val; bi = col; }
-	}
+	} else {
+		// TG_EPI_LOGITS: logits + first stage of the greedy argmax
+		// (ops.hpp:749-757: strict '>' scan from index 0, so the lowest index wins ties)
+		float bv = -INFINITY;
+		int bi = 0x7fffffff;
+		if (tid < C) {
+			const int col = cur * C + tid;
+			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
+			const float val = sum * g.scales[col];
+			if (g.y != nullptr) g.y[col] = val;
+			if (val > bv) { bv = val; bi = col; }
+		}
 #pragma unroll
-	for (int o = 32; o > 0; o >>= 1) {
-		const float ov = __shfl_xor(bv, o, 64);
-		const int oi = __shfl_xor(bi, o, 64);
-		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+		for (int o = 32; o > 0; o >>= 1) {
+			const float ov = __shfl_xor(bv, o, 64);
+			const int oi = __shfl_xor(bi, o, 64);
+			if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+		}
+		if (lane == 0) { s_bv[it & 1][w] = bv; s_bi[it & 1][w] = bi; }
+		__syncthreads();
+		if (tid == 0) {
+			for (int i = 1; i < NWAVE; i++)
+				if (s_bv[it & 1][i] > bv || (s_bv[it & 1][i] == bv && s_bi[it & 1][i] < bi)) { bv = s_bv[it & 1][i]; bi = s_bi[it & 1][i]; }
+			g.blk_val[cur] = bv;
+			g.blk_idx[cur] = bi;
+		}
 	}
-	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
-	__syncthreads();
-	if (tid == 0) {
-		for (int i = 1; i < NWAVE; i++)
-			if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
-		g.blk_val[tile] = bv;
-		g.blk_idx[tile] = bi;
-	}
+	if (!more) break;
+	}  // tile loop
 }
 
 // One named entry point per role, so that profiles separate the projections.
@@ -295,8 +357,12 @@ __global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, con
 
 }  // namespace
 
-void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s) {
-	dim3 grid((unsigned)g.ntiles), block(NT);
+void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
+	// more than max_blocks tiles: workgroups loop over tiles, so the prologue is paid once per workgroup
+	TgGemv g = g_in;
+	g.nmain = (g.max_blocks > 0 && g.ntiles > g.max_blocks) ? g.max_blocks : g.ntiles;
+	if (g.pf.ptr == nullptr) g.pf.nblocks = 0;
+	dim3 grid((unsigned)(g.nmain + g.pf.nblocks)), block(NT);
 	switch (role) {
 		case TG_ROLE_QKV_EMBED: hipLaunchKernelGGL(tg_gemv_qkv_embed, grid, block, 0, s, g); break;
 		case TG_ROLE_QKV: hipLaunchKernelGGL(tg_gemv_qkv, grid, block, 0, s, g); break;

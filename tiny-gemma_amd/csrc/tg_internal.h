@@ -33,6 +33,33 @@
 #define TG_ATTN_MERGE_MAX 16 // attention partials the output projection merges in its prologue
 #define TG_ATTN_MAX_BLOCKS 256  // attention workgroups per launch, upper bound
 
+// ---- weight prefetch riding along with a launch ------------------------------------------------
+// Batch-1 decode is a chain of ~130 dependent, latency-bound launches per token during which HBM
+// is mostly idle.  A launch can therefore carry extra workgroups whose only job is to touch the
+// weights of the NEXT launch, pulling them out of HBM into the memory-side cache and the L2 while
+// the current launch works through its own latency chain.  A hint only: results do not depend on it.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2); prefetch workgroup G touches
+// the slabs of the consumer tiles t with t % 8 == G % 8, the tiles the consumer's workgroups on the
+// same XCD will read.
+struct TgPrefetch {
+	const int8_t *ptr;   // first tile slab of the matrix to prefetch (null: nothing)
+	uint32_t slab;       // bytes per tile slab
+	int ntiles;          // slabs
+	int nblocks;         // extra workgroups appended to the grid (multiple of 8)
+};
+
+__device__ __forceinline__ void tg_prefetch_block(const TgPrefetch &p, int first_extra_block) {
+	const int pb = (int)blockIdx.x - first_extra_block;
+	const int x = (int)(blockIdx.x & 7u), q = pb >> 3, Q = p.nblocks >> 3;
+	for (int t = x + 8 * q; t < p.ntiles; t += 8 * Q) {
+		const int8_t *sl = p.ptr + (size_t)t * p.slab;
+		for (uint32_t off = threadIdx.x * 128u; off < p.slab; off += 256u * 128u) {
+			const int v = *(const int *)(sl + off);  // one dword per 128-byte line brings the line in
+			asm volatile("" ::"v"(v));               // the value is not needed, the load is
+		}
+	}
+}
+
 // ---- GEMV launch description --------------------------------------------------------------
 enum { TG_PRO_PLAIN = 0, TG_PRO_NORM = 1, TG_PRO_RESNORM = 2, TG_PRO_EMBED = 3, TG_PRO_ATTN_MERGE = 4 };
 enum { TG_EPI_STORE = 0, TG_EPI_GEGLU = 1, TG_EPI_LOGITS = 2 };
@@ -45,6 +72,8 @@ struct TgGemv {
 	int ntiles;            // grid.x
 	int C;                 // columns per tile: 4, 8, ..., 128
 	int lc_shift;          // log2(C/4)
+	int max_blocks;        // 0: one workgroup per tile; else workgroups loop over tiles when ntiles exceeds it
+	int nmain;             // set by the launcher: workgroups that compute (the rest of the grid prefetches)
 	// prologue (the TG_PRO_* mode is fixed by the kernel role)
 	int hidden;            // length of the residual stream (NORM/RESNORM/EMBED); equals K there
 	const float *x;        // PLAIN: the input [K]; NORM: vector to normalise; RESNORM: residual
@@ -69,6 +98,7 @@ struct TgGemv {
 	int lut_size;
 	float *blk_val;        // LOGITS: per-workgroup maximum and its index, [ntiles]
 	int *blk_idx;
+	TgPrefetch pf;         // weights of the next launch (optional)
 };
 
 struct TgAttnDecode {
@@ -83,6 +113,8 @@ struct TgAttnDecode {
 	float *part_acc;         // [nblocks][n_head][hd]
 	float *part_ml;          // [nblocks][n_head][2]
 	int n_head;
+	int nblocks;             // attention workgroups in the grid; workgroups past them prefetch
+	TgPrefetch pf;           // weights of the next launch (optional)
 };
 
 enum { TG_ROLE_PLAIN = 0, TG_ROLE_QKV_EMBED, TG_ROLE_QKV, TG_ROLE_OPROJ, TG_ROLE_UPGATE, TG_ROLE_DOWN, TG_ROLE_LMHEAD,
@@ -106,6 +138,8 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 // C[m][N] = (A[m][K] . W) * scales, W packed; epi GEGLU writes C[m][N/2]
 void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
+
+void tg_launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
 
 // ---- errors -----------------------------------------------------------------------------------
 int tg_fail(int code, const std::string &msg);

@@ -146,7 +146,17 @@ __global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *
 	}
 }
 
+// Plain streaming copy of n 16-byte pieces: the known-size kernel that hardware byte counters are
+// scaled against.
+__global__ __launch_bounds__(RNT) void tg_copy_kernel(uint4 *dst, const uint4 *src, size_t n) {
+	for (size_t i = (size_t)blockIdx.x * RNT + threadIdx.x; i < n; i += (size_t)gridDim.x * RNT) dst[i] = src[i];
+}
+
 }  // namespace
+
+void tg_launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s) {
+	hipLaunchKernelGGL(tg_copy_kernel, dim3(4096), dim3(RNT), 0, s, (uint4 *)dst, (const uint4 *)src, bytes / 16);
+}
 
 void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,
                           hipStream_t s) {
