@@ -28,6 +28,9 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as ge  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of one tg_gemv_lmhead_argmax launch from two `rocprofv3 --pmc` runs (FETCH_SIZE x 1.9998 +
+# WRITE_SIZE x 1.0000, both in KiB, scaled on a 256 MiB copy kernel): profiles/decode_1B_hbm_traffic.md
+LMHEAD_TRAFFIC_BYTES = {"1B": 304_438_104}
 
 MODELS = {
     # name: (prompt tokens, decode bytes of weights+scales per token, LM-head GEMV algorithmic bytes)
@@ -172,6 +175,16 @@ def main():
     per_kernel_us = {n: 1e3 * ms_sum[i] / max(1, launches[i]) for i, n in enumerate(names)}
     lm_s = 1e-6 * per_kernel_us["lmhead_argmax"]
     achieved = lm_bytes / lm_s / 1e9
+    # the same kernel re-launched 50x back to back on the session's buffers (dispatch latency amortised)
+    L = tg.lib()
+    L.tg_debug_repeat_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
+    tg.check(L.tg_debug_repeat_kernel(sess.h, 5, 0, 5))
+    tg.synchronize()
+    ev.record(e0, stream)
+    tg.check(L.tg_debug_repeat_kernel(sess.h, 5, 0, 50))
+    ev.record(e1, stream)
+    tg.synchronize()
+    lm_iso_us = ev.elapsed_ms(e0, e1) * 1e3 / 50
 
     tok_s = args.steps / wall
     out = {
@@ -202,9 +215,12 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": LMHEAD_TRAFFIC_BYTES.get(args.model),
             "algorithmic_bytes_per_launch": lm_bytes,
             "avg_launch_us": per_kernel_us["lmhead_argmax"],
+            "timing": "HIP events around every launch of the kernel inside real decode steps (includes dispatch latency)",
+            "back_to_back_us": lm_iso_us,
+            "back_to_back_GBps": lm_bytes / lm_iso_us / 1e3,
         },
         "decode_step": {
             "gpu_ms_per_step_events": gpu_ms / args.steps,
