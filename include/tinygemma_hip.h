@@ -125,6 +125,9 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 int tg_decode_enqueue(tg_session *s, int n_steps);
 /* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
 int tg_set_graphs(int enable);
+/* prefill GEMM: 1 (default) = MFMA with fp16 hi/lo split activations (fp32-rounding-level accuracy),
+ * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */
+int tg_set_gemm_mode(int mfma);
 /* tuning knob: a GEMV launch uses at most n workgroups, which then loop over column tiles (0: one per tile) */
 int tg_set_gemv_max_blocks(int n);
 /* tuning knob: extra workgroups per decode launch that pull the NEXT launch's weights out of HBM into

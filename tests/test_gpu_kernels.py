@@ -84,14 +84,59 @@ def test_unsupported_shapes_raise(tg):
             tg.launch_qgemm(np.zeros((2, n), np.float32), np.zeros((2, i), np.float32), W, s, 2, i, n)
 
 
+@pytest.fixture
+def exact_gemm(tg):
+    """The vector-ALU GEMM that keeps the reference's per-element order (tg_set_gemm_mode(0))."""
+    tg.lib().tg_set_gemm_mode(0)
+    yield
+    tg.lib().tg_set_gemm_mode(1)
+
+
 @pytest.mark.parametrize("name", list(gi.GEMM_CASES))
-def test_qgemm_bit_exact(tg, oracle, golden, name):
+def test_qgemm_exact_mode_bit_exact(tg, oracle, golden, exact_gemm, name):
     m, i, n, seed = gi.GEMM_CASES[name]
     A, W, s = gi.gemm_inputs(m, i, n, seed)
     Cm = np.full((m, n), np.nan, np.float32)  # launch_qgemm overwrites C (linalg.hpp:244)
     tg.launch_qgemm(Cm, A, W, s, m, i, n)
     assert np.array_equal(Cm, oracle.qgemm(A, W, s))
     assert np.array_equal(Cm.reshape(-1)[:2048], golden[f"gemm/{name}/head"])
+
+
+@pytest.mark.parametrize("name", list(gi.GEMM_CASES))
+def test_qgemm_mfma(tg, oracle, golden, name):
+    """Default prefill GEMM: fp16 MFMA on power-of-two scaled hi/lo split activations.  22 mantissa bits of
+    the activations and exact int8 -> fp16 weights: norm-relative error at the fp32-rounding level (<= 3e-6)."""
+    m, i, n, seed = gi.GEMM_CASES[name]
+    A, W, s = gi.gemm_inputs(m, i, n, seed)
+    Cm = np.full((m, n), np.nan, np.float32)
+    tg.launch_qgemm(Cm, A, W, s, m, i, n)
+    ref = oracle.qgemm(A, W, s)
+    assert not np.isnan(Cm).any()
+    assert normrel(Cm, ref) < 3e-6
+    assert np.abs(Cm - ref).max() <= 2e-5 * np.abs(ref).max()
+    assert normrel(Cm.reshape(-1)[:2048], golden[f"gemm/{name}/head"]) < 3e-6
+
+
+def test_qgemm_mfma_exact_cases(tg):
+    """Integer activations and power-of-two scales are exact through the hi/lo split (lo = 0);
+    rows of very different magnitude (1e-6 ... 1e4, and an all-zero row) keep their own scaling."""
+    rng = np.random.default_rng(7)
+    A = rng.integers(-8, 9, (70, 1152)).astype(np.float32)
+    A[3] = 0.0
+    W = rng.integers(-127, 128, (1152, 1024), dtype=np.int8)
+    s = np.full(1024, 2.0 ** -7, np.float32)
+    Cm = np.empty((70, 1024), np.float32)
+    tg.launch_qgemm(Cm, A, W, s, 70, 1152, 1024)
+    exact = (A.astype(np.int64) @ W.astype(np.int64)).astype(np.float64) * 2.0 ** -7
+    assert np.array_equal(Cm.astype(np.float64), exact)
+    A = rng.standard_normal((9, 640)).astype(np.float32) * np.float32(10.0) ** rng.integers(-6, 5, (9, 1)).astype(np.float32)
+    W = rng.integers(-127, 128, (640, 256), dtype=np.int8)
+    s = rng.uniform(0.001, 0.02, 256).astype(np.float32)
+    Cm = np.empty((9, 256), np.float32)
+    tg.launch_qgemm(Cm, A, W, s, 9, 640, 256)
+    ref = (A.astype(np.float64) @ W.astype(np.float64)) * s.astype(np.float64)
+    for r in range(9):
+        assert normrel(Cm[r], ref[r]) < 3e-6
 
 
 def test_device_resident_gemv_matches_host_entry(tg, oracle):

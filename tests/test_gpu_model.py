@@ -61,6 +61,16 @@ def compare_run(sess, osess, prompt, n_decode, tol, tol_first):
     return np.array(toks, np.int32), worst
 
 
+def test_prefill_exact_gemm_mode(tg, oracle, golden, weight_images, tables):
+    """The forward with the exact-order vector-ALU GEMM (tg_set_gemm_mode(0)) instead of MFMA."""
+    tg.lib().tg_set_gemm_mode(0)
+    try:
+        model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut")
+        compare_run(sess, osess, prompt, 2, tol=5e-5, tol_first=3e-6)
+    finally:
+        tg.lib().tg_set_gemm_mode(1)
+
+
 def test_embedding_tap_is_exact(tg, oracle, weight_images, tables):
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
     sess.prefill(prompt, want_logits=False)

@@ -19,6 +19,11 @@ namespace {
 
 thread_local std::string g_err;
 bool g_inited = false;
+int g_gemm_mfma = 1;            // prefill GEMM: 1 = MFMA (fp16 hi/lo split), 0 = exact-order fp32 on the vector ALUs
+_Float16 *g_apack = nullptr;    // scratch of the stand-alone GEMM entry points
+size_t g_apack_halfs = 0;
+float *g_rowscale = nullptr;
+size_t g_rowscale_n = 0;
 int g_prefetch_blocks = 128;   // extra workgroups per launch that prefetch the next launch's weights (0: off; multiple of 8)
 int g_gemv_max_blocks = 1024;  // workgroups per GEMV launch before workgroups start looping over tiles
 bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GPU-side dispatch, not by host launches)
@@ -152,6 +157,17 @@ TgGemv gemv_base(const PackedMat &p) {
 	g.lc_shift = p.lc_shift;
 	g.max_blocks = g_gemv_max_blocks;
 	return g;
+}
+
+// C[m][N] = scales * (A[m][K] . W) through the selected GEMM; apack/rowscale are scratch for the MFMA path.
+void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
+                 int lut_size, _Float16 *apack, float *rowscale) {
+	if (g_gemm_mfma) {
+		tg_launch_split_pack(A, lda, m, p.K, apack, rowscale, g_stream);
+		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, g_stream);
+	} else {
+		tg_launch_gemm(C, A, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, g_stream);
+	}
 }
 
 // Prefetch job for the GEMV tiles of `p` (see TgPrefetch).
@@ -376,7 +392,21 @@ int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logi
 int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	if (!w->p.Wg) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "no GEMM tiling was built for this matrix (outDim too large)");
-	tg_launch_gemm(C_dev, A_dev, w->p.Wg, w->p.scales_g, m, w->p.K, w->p.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+	if (g_gemm_mfma) {
+		const size_t need = tg_gemm_mfma_apack_halfs(m, w->p.K), need_rs = (size_t)((m + 127) / 128) * 128;
+		if (need > g_apack_halfs || need_rs > g_rowscale_n) {
+			TG_HIP(hipStreamSynchronize(g_stream));
+			if (g_apack) (void)hipFree(g_apack);
+			if (g_rowscale) (void)hipFree(g_rowscale);
+			g_apack = nullptr;
+			g_rowscale = nullptr;
+			TG_HIP(hipMalloc((void **)&g_apack, need * sizeof(_Float16)));
+			TG_HIP(hipMalloc((void **)&g_rowscale, need_rs * sizeof(float)));
+			g_apack_halfs = need;
+			g_rowscale_n = need_rs;
+		}
+	}
+	launch_gemm(C_dev, A_dev, w->p.K, w->p, m, TG_EPI_STORE, nullptr, 0, 0, 0, g_apack, g_rowscale);
 	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
@@ -952,6 +982,11 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
 	return enqueue_decode_step(s, nullptr, false, &only);
 }
 
+int tg_set_gemm_mode(int mfma) {
+	g_gemm_mfma = mfma != 0;
+	return TG_OK;
+}
+
 int tg_set_prefetch_blocks(int n) {
 	if (n < 0 || (n & 7)) return tg_fail(TG_ERR_BAD_ARG, "prefetch workgroups must be a non-negative multiple of 8");
 	g_prefetch_blocks = n;
@@ -1021,9 +1056,10 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	const int qo = c.n_head * hd, nq = qo + 2 * hd;
 	const size_t S = (size_t)n;
 	int *d_ids = nullptr;
-	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr;
+	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr;
+	_Float16 *apack = nullptr;
 	auto cleanup = [&]() {
-		void *ps[] = {d_ids, x, xn, qkv, ao, t, hb};
+		void *ps[] = {d_ids, x, xn, qkv, ao, t, hb, rowscale, apack};
 		for (void *p : ps)
 			if (p) (void)hipFree(p);
 	};
@@ -1042,6 +1078,10 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	TG_TRY(hipMalloc((void **)&ao, sizeof(float) * S * qo));
 	TG_TRY(hipMalloc((void **)&t, sizeof(float) * S * h));
 	TG_TRY(hipMalloc((void **)&hb, sizeof(float) * S * f));
+	if (g_gemm_mfma) {
+		TG_TRY(hipMalloc((void **)&apack, sizeof(_Float16) * tg_gemm_mfma_apack_halfs(n, std::max(f, qo))));
+		TG_TRY(hipMalloc((void **)&rowscale, sizeof(float) * (size_t)((n + 127) / 128) * 128));
+	}
 	const bool keep_taps = n <= PREFILL_TAP_MAX_ROWS;
 	if (s->taps) {
 		(void)hipFree(s->taps);
@@ -1065,7 +1105,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		const LayerDev &Ld = m->L[(size_t)l];
 		const int mp = s->max_pos[(size_t)l];
 		// Q|K|V (modules.hpp:106-108)
-		tg_launch_gemm(qkv, xn, Ld.qkv.Wg, Ld.qkv.scales_g, n, h, Ld.qkv.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		launch_gemm(qkv, xn, h, Ld.qkv, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
 		tg_launch_qk_norm_rope_rows(qkv, qkv + qo, qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
@@ -1073,13 +1113,13 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
 		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, g_stream);
 		// O (modules.hpp:127-128)
-		tg_launch_gemm(t, ao, Ld.o.Wg, Ld.o.scales_g, n, qo, Ld.o.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
 		tg_launch_norm_rows(xn, t, Ld.mpre, Ld.apost, x, x, n, h, g_stream);
 		TG_TRY(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
-		tg_launch_gemm(hb, xn, Ld.ug.Wg, Ld.ug.scales_g, n, h, Ld.ug.ntiles_g, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, g_stream);
-		tg_launch_gemm(t, hb, Ld.d.Wg, Ld.d.scales_g, n, f, Ld.d.ntiles_g, TG_EPI_STORE, nullptr, 0, 0, 0, g_stream);
+		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale);
+		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
 		tg_launch_norm_rows(xn, t, next_pre, Ld.mpost, x, x, n, h, g_stream);

@@ -141,6 +141,12 @@ void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *sca
 
 void tg_launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
 
+// MFMA prefill GEMM (tg_gemm_mfma.hip): A is first split into scaled fp16 hi/lo halves in operand order
+size_t tg_gemm_mfma_apack_halfs(int M, int K);
+void tg_launch_split_pack(const float *A, int lda, int M, int K, _Float16 *apack, float *rowscale, hipStream_t s);
+void tg_launch_gemm_mfma(float *C, const _Float16 *apack, const float *rowscale, const int8_t *Wg, const float *scales, int M, int K,
+                         int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
+
 // ---- errors -----------------------------------------------------------------------------------
 int tg_fail(int code, const std::string &msg);
 #define TG_HIP(expr)                                                                           \
