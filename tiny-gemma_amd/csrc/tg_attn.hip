@@ -95,9 +95,14 @@ __device__ __forceinline__ void chunk_scores(const float (*qs)[HD], const float 
 	}
 }
 
+// Keys of a chunk whose K rows / V elements are fetched before anything else in the kernel (the rest, for
+// chunks longer than this, is fetched inside the loops).
+constexpr int PRE = 32;
+
 __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) {
-	__shared__ float qs[NH][HD];
-	__shared__ float knew[HD], vnew[HD];
+	__shared__ __attribute__((aligned(16))) float qs[NH][HD];
+	__shared__ __attribute__((aligned(16))) float knew[HD];
+	__shared__ float vnew[HD];
 	__shared__ float sc[NH][MAXCHUNK];
 	__shared__ float s_m[NH], s_l[NH];
 
@@ -105,14 +110,34 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 		tg_prefetch_block(a.pf, a.nblocks);
 		return;
 	}
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, sub = lane >> 4, sl = lane & 15;
 	const int pos = a.pos[0];                      // position_ptr before this token (decode.hpp:154)
-	const int bp = a.pos[a.bp_index];           // buffer_ptr before this token (decode.hpp:59)
+	const int bp = a.pos[a.bp_index];              // buffer_ptr before this token (decode.hpp:59)
 	const int cur = bp % a.max_pos;
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;  // decode.hpp:45-47 after update_single
 	const int nb = (valid + a.chunk - 1) / a.chunk;
 	const int b = blockIdx.x;
 	if (b >= nb) return;
+	const int k0 = b * a.chunk;
+	const int n = (valid - k0 < a.chunk) ? valid - k0 : a.chunk;
+
+	// Cache rows of the first PRE keys of this chunk go out first: they depend on nothing computed here.
+	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: thread = output dim.
+	float4 kpre[PRE / 16][4];
+	float vpre[PRE];
+#pragma unroll
+	for (int p = 0; p < PRE / 16; p++) {
+		const int jj = 16 * p + w * 4 + sub;
+		const int j = k0 + (jj < n ? jj : 0);
+		const float *kr = a.kc + (size_t)(j == cur ? k0 : j) * HD;  // slot `cur` is replaced below; any valid row will do
+#pragma unroll
+		for (int i = 0; i < 4; i++) kpre[p][i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
+	}
+#pragma unroll
+	for (int u = 0; u < PRE; u++) {
+		const int j = k0 + (u < n ? u : 0);
+		vpre[u] = a.vc[(size_t)(j == cur ? k0 : j) * HD + tid];
+	}
 
 	// q heads: one wave each; k: wave 0 again
 	{
@@ -134,9 +159,47 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 		a.vc[(size_t)cur * HD + tid] = vnew[tid];
 	}
 
-	const int k0 = b * a.chunk;
-	const int n = (valid - k0 < a.chunk) ? valid - k0 : a.chunk;
-	chunk_scores(qs, a.kc, HD, knew, cur, k0, n, sc, tid);
+	// scores: q_h . k_j for the 4 heads; the token being decoded (slot cur) comes from knew
+	{
+		float4 q[NH][4];
+#pragma unroll
+		for (int h = 0; h < NH; h++)
+#pragma unroll
+			for (int i = 0; i < 4; i++) q[h][i] = *reinterpret_cast<const float4 *>(&qs[h][i * 64 + sl * 4]);
+		auto pass = [&](int base, const float4 *kin) {
+			const int jj = base + w * 4 + sub;
+			const bool ok = jj < n;
+			const int j = k0 + (ok ? jj : 0);
+			float4 kv[4];
+#pragma unroll
+			for (int i = 0; i < 4; i++) kv[i] = (j == cur) ? *reinterpret_cast<const float4 *>(&knew[i * 64 + sl * 4]) : kin[i];
+#pragma unroll
+			for (int h = 0; h < NH; h++) {
+				float d = 0.0f;
+#pragma unroll
+				for (int i = 0; i < 4; i++) {
+					d = fmaf(q[h][i].x, kv[i].x, d);
+					d = fmaf(q[h][i].y, kv[i].y, d);
+					d = fmaf(q[h][i].z, kv[i].z, d);
+					d = fmaf(q[h][i].w, kv[i].w, d);
+				}
+				d = sum16(d);
+				if (ok && sl == 0) sc[h][jj] = d;
+			}
+		};
+#pragma unroll
+		for (int p = 0; p < PRE / 16; p++)
+			if (16 * p < n) pass(16 * p, kpre[p]);
+		for (int base = PRE; base < n; base += 16) {
+			const int jj = base + w * 4 + sub;
+			const int j = k0 + (jj < n ? jj : 0);
+			const float *kr = a.kc + (size_t)(j == cur ? k0 : j) * HD;
+			float4 kv[4];
+#pragma unroll
+			for (int i = 0; i < 4; i++) kv[i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
+			pass(base, kv);
+		}
+	}
 	__syncthreads();
 
 	// softmax statistics of this chunk: wave h owns head h
@@ -157,7 +220,15 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 
 	// P.V: thread = output dim, 4 heads
 	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
-	for (int j0 = 0; j0 < n; j0 += 8) {
+#pragma unroll
+	for (int u = 0; u < PRE; u++) {
+		if (u < n) {
+			const float vv = (k0 + u == cur) ? vnew[tid] : vpre[u];
+#pragma unroll
+			for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][u], vv, acc[h]);
+		}
+	}
+	for (int j0 = PRE; j0 < n; j0 += 8) {
 		float vv[8];
 #pragma unroll
 		for (int u = 0; u < 8; u++) {

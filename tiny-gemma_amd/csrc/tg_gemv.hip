@@ -129,12 +129,20 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	}
 
 	// ---------------- prologue: input vector ----------------
+	// Every global load of a prologue that does not depend on another one is issued up front, next
+	// to the weight loads above, so that the prologue costs one memory round trip, not several.
 	if (PRO == TG_PRO_ATTN_MERGE) {
 		// merge of the flash-decoding partials of the attention launch that precedes this projection:
 		//   out_h = sum_b acc_{b,h} * exp(m_{b,h} - M_h) / sum_b l_{b,h} * exp(m_{b,h} - M_h)
 		const int pos = g.pos[0];
 		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
 		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
+		float a[4][TG_ATTN_MERGE_MAX];
+#pragma unroll
+		for (int h = 0; h < 4; h++)
+#pragma unroll
+			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
+				a[h][b] = (b < nb) ? g.part_acc[((size_t)b * 4 + h) * 256 + tid] : 0.0f;
 		if (tid < 4 * TG_ATTN_MERGE_MAX) {
 			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
 			const bool ok = b < nb;
@@ -152,47 +160,75 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		__syncthreads();
 #pragma unroll
 		for (int h = 0; h < 4; h++) {
-			float a[TG_ATTN_MERGE_MAX];
-#pragma unroll
-			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
-				a[b] = (b < nb) ? g.part_acc[((size_t)b * 4 + h) * 256 + tid] : 0.0f;
 			float o = 0.0f;
 #pragma unroll
-			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) o = fmaf(a[b], wgt[h][b], o);
+			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) o = fmaf(a[h][b], wgt[h][b], o);
 			xs[h * 256 + tid] = o;
 		}
 		__syncthreads();
 	} else if (PRO != TG_PRO_PLAIN) {
 		const int h = g.hidden;
 		const float eps = 1e-06f;
+		constexpr int PER = (TG_MAX_HIDDEN + NT - 1) / NT;  // elements of the residual stream per lane
+		float t[PER], wpre[PER];
+#pragma unroll
+		for (int i = 0; i < PER; i++) {
+			const int d = tid + i * NT;
+			wpre[i] = (d < h) ? g.w_pre[d] : 0.0f;
+		}
 		if (PRO == TG_PRO_EMBED) {
 			// ops.hpp:537-568: s[d] * (sqrt(hidden) * q)
 			int tok = *g.tok;
 			tok = tok < 0 ? 0 : (tok >= g.vocab ? g.vocab - 1 : tok);
 			const int8_t *row = g.wte + (size_t)tok * h;
-			for (int d = tid; d < h; d += NT) xs[d] = g.wte_scales[d] * (g.emb_scale * (float)row[d]);
+#pragma unroll
+			for (int i = 0; i < PER; i++) {
+				const int d = tid + i * NT;
+				t[i] = (d < h) ? g.wte_scales[d] * (g.emb_scale * (float)row[d]) : 0.0f;
+			}
 		} else if (PRO == TG_PRO_NORM) {
-			for (int d = tid; d < h; d += NT) xs[d] = g.x[d];
+#pragma unroll
+			for (int i = 0; i < PER; i++) {
+				const int d = tid + i * NT;
+				t[i] = (d < h) ? g.x[d] : 0.0f;
+			}
 		} else {
 			// modules.hpp:166-168 / 218-219: x = rmsnorm(block_out, post) + residual
-			float ss = 0.0f;
-			for (int d = tid; d < h; d += NT) {
-				float p = g.pend[d];
-				xs[d] = p;
-				ss = fmaf(p, p, ss);
+			float p[PER], r[PER], wpo[PER];
+#pragma unroll
+			for (int i = 0; i < PER; i++) {
+				const int d = tid + i * NT;
+				const bool ok = d < h;
+				p[i] = ok ? g.pend[d] : 0.0f;
+				r[i] = ok ? g.x[d] : 0.0f;
+				wpo[i] = ok ? g.w_post[d] : 0.0f;
 			}
+			float ss = 0.0f;
+#pragma unroll
+			for (int i = 0; i < PER; i++) ss = fmaf(p[i], p[i], ss);
 			ss = block_sum(ss, sred);
 			const float irms = 1.0f / sqrtf(ss / (float)h + eps);
-			for (int d = tid; d < h; d += NT) xs[d] = (xs[d] * irms) * (g.w_post[d] + 1.0f) + g.x[d];
+#pragma unroll
+			for (int i = 0; i < PER; i++) t[i] = (p[i] * irms) * (wpo[i] + 1.0f) + r[i];
 		}
-		if (g.xr_out != nullptr && blockIdx.x == 0)
-			for (int d = tid; d < h; d += NT) g.xr_out[d] = xs[d];
+		if (g.xr_out != nullptr && blockIdx.x == 0) {
+#pragma unroll
+			for (int i = 0; i < PER; i++) {
+				const int d = tid + i * NT;
+				if (d < h) g.xr_out[d] = t[i];
+			}
+		}
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
 		float ss = 0.0f;
-		for (int d = tid; d < h; d += NT) ss = fmaf(xs[d], xs[d], ss);
+#pragma unroll
+		for (int i = 0; i < PER; i++) ss = fmaf(t[i], t[i], ss);  // lanes past h hold 0
 		ss = block_sum(ss, sred);
 		const float irms = 1.0f / sqrtf(ss / (float)h + eps);
-		for (int d = tid; d < h; d += NT) xs[d] = (xs[d] * irms) * (g.w_pre[d] + 1.0f);
+#pragma unroll
+		for (int i = 0; i < PER; i++) {
+			const int d = tid + i * NT;
+			if (d < h) xs[d] = (t[i] * irms) * (wpre[i] + 1.0f);
+		}
 		__syncthreads();
 	}
 
