@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--graphs", action="store_true", help="replay captured HIP graphs instead of plain stream launches")
     ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
     ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
+    ap.add_argument("--prefetch-plan", type=int, default=None, help="tuning knob")
     ap.add_argument("--counter-run", action="store_true",
                     help="for rocprofv3 --pmc: prefill, a few decode steps and 4 launches of a 256 MiB copy kernel; no timing")
     args = ap.parse_args()
@@ -116,6 +117,8 @@ def main():
     tg.lib().tg_set_graphs(1 if args.graphs else 0)
     if args.prefetch_blocks is not None:
         tg.check(tg.lib().tg_set_prefetch_blocks(args.prefetch_blocks))
+    if args.prefetch_plan is not None:
+        tg.lib().tg_set_prefetch_plan(args.prefetch_plan)
     if args.gemv_max_blocks is not None:
         tg.lib().tg_set_gemv_max_blocks(args.gemv_max_blocks)
     n_prompt, step_bytes, lm_bytes = MODELS[args.model]

@@ -24,6 +24,7 @@ _Float16 *g_apack = nullptr;    // scratch of the stand-alone GEMM entry points
 size_t g_apack_halfs = 0;
 float *g_rowscale = nullptr;
 size_t g_rowscale_n = 0;
+int g_prefetch_plan = 0;        // which launch prefetches which weights (experiment knob)
 int g_prefetch_blocks = 128;   // extra workgroups per launch that prefetch the next launch's weights (0: off; multiple of 8)
 int g_gemv_max_blocks = 1024;  // workgroups per GEMV launch before workgroups start looping over tiles
 bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GPU-side dispatch, not by host launches)
@@ -802,6 +803,7 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		g.xr_out = s->xr + (size_t)(2 * l) * h;
 		g.y = s->qkv;
 		g.pf = prefetch_of(Ld.o);
+		if (g_prefetch_plan == 1) g.pf2 = prefetch_of(Ld.ug);
 		TG_MARK(TG_KC_QKV);
 		if (l == 0) {
 			g.wte = m->wte;
@@ -829,13 +831,16 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		a.max_pos = s->max_pos[(size_t)l];
 		a.pos = s->ctr;
 		a.bp_index = Ld.is_sw ? 1 : 2;
+		// a captured step is replayed at other positions: only then are the counters read from device memory
+		a.host_pos = full_grid ? -1 : s->pos;
+		a.host_bp = full_grid ? -1 : (Ld.is_sw ? s->bp_local : s->bp_global);
 		const int valid = std::min(s->pos + 1, a.max_pos);
 		bool needs_merge = false;
 		a.chunk = attn_chunk_for(valid, &needs_merge);
 		a.part_acc = s->part_acc;
 		a.part_ml = s->part_ml;
 		a.n_head = c.n_head;
-		a.pf = prefetch_of(Ld.ug);
+		a.pf = prefetch_of(g_prefetch_plan == 1 ? Ld.d : Ld.ug);
 		TG_MARK(TG_KC_ATTN);
 		// a captured step is replayed at later positions with the same chunk: launch the largest grid that
 		// chunk can need (workgroups past the valid keys exit at once)
@@ -845,12 +850,13 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		// --- merge of the attention partials + O projection (modules.hpp:161-164)
 		g = gemv_base(Ld.o);
 		g.pos = s->ctr;
+		g.host_pos = a.host_pos;
 		g.attn_max_pos = a.max_pos;
 		g.attn_chunk = needs_merge ? a.max_pos : a.chunk;  // merged: a single partial
 		g.part_acc = needs_merge ? s->merged_acc : s->part_acc;
 		g.part_ml = needs_merge ? s->merged_ml : s->part_ml;
 		g.y = s->o_out;
-		g.pf = prefetch_of(Ld.d);
+		if (g_prefetch_plan == 0) g.pf = prefetch_of(Ld.d);
 		TG_MARK(TG_KC_OPROJ);
 		TG_DO(TG_KC_OPROJ, l, tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream));
 		// --- post-norm + residual, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
@@ -984,6 +990,11 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
 
 int tg_set_gemm_mode(int mfma) {
 	g_gemm_mfma = mfma != 0;
+	return TG_OK;
+}
+
+int tg_set_prefetch_plan(int plan) {
+	g_prefetch_plan = plan;
 	return TG_OK;
 }
 

@@ -107,12 +107,12 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	__shared__ float s_m[NH], s_l[NH];
 
 	if ((int)blockIdx.x >= a.nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
-		tg_prefetch_block(a.pf, a.nblocks);
+		tg_prefetch_dispatch(a.pf, a.pf2, a.nblocks);
 		return;
 	}
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, sub = lane >> 4, sl = lane & 15;
-	const int pos = a.pos[0];                      // position_ptr before this token (decode.hpp:154)
-	const int bp = a.pos[a.bp_index];              // buffer_ptr before this token (decode.hpp:59)
+	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];          // position_ptr before this token (decode.hpp:154)
+	const int bp = a.host_bp >= 0 ? a.host_bp : a.pos[a.bp_index];    // buffer_ptr before this token (decode.hpp:59)
 	const int cur = bp % a.max_pos;
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;  // decode.hpp:45-47 after update_single
 	const int nb = (valid + a.chunk - 1) / a.chunk;
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, f
 	__shared__ float wg[TG_ATTN_MAX_BLOCKS];
 	__shared__ float sred[4];
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x;
-	const int pos = a.pos[0];
+	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;
 	const int nb = (valid + a.chunk - 1) / a.chunk;
 	const bool ok = tid < nb;
@@ -394,7 +394,8 @@ void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t
 	TgAttnDecode a = a_in;
 	a.nblocks = max_blocks;
 	if (a.pf.ptr == nullptr) a.pf.nblocks = 0;
-	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(max_blocks + a.pf.nblocks)), dim3(ANT), 0, s, a);
+	if (a.pf2.ptr == nullptr) a.pf2.nblocks = 0;
+	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(max_blocks + a.pf.nblocks + a.pf2.nblocks)), dim3(ANT), 0, s, a);
 }
 
 void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s) {

@@ -96,7 +96,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	__shared__ int s_bi[2][NWAVE];
 
 	if ((int)blockIdx.x >= g.nmain) {  // extra workgroups: prefetch the next launch's weights and leave
-		tg_prefetch_block(g.pf, g.nmain);
+		tg_prefetch_dispatch(g.pf, g.pf2, g.nmain);
 		return;
 	}
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -134,7 +134,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	if (PRO == TG_PRO_ATTN_MERGE) {
 		// merge of the flash-decoding partials of the attention launch that precedes this projection:
 		//   out_h = sum_b acc_{b,h} * exp(m_{b,h} - M_h) / sum_b l_{b,h} * exp(m_{b,h} - M_h)
-		const int pos = g.pos[0];
+		const int pos = g.host_pos >= 0 ? g.host_pos : g.pos[0];
 		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
 		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
 		float a[4][TG_ATTN_MERGE_MAX];
@@ -398,7 +398,8 @@ void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
 	TgGemv g = g_in;
 	g.nmain = (g.max_blocks > 0 && g.ntiles > g.max_blocks) ? g.max_blocks : g.ntiles;
 	if (g.pf.ptr == nullptr) g.pf.nblocks = 0;
-	dim3 grid((unsigned)(g.nmain + g.pf.nblocks)), block(NT);
+	if (g.pf2.ptr == nullptr) g.pf2.nblocks = 0;
+	dim3 grid((unsigned)(g.nmain + g.pf.nblocks + g.pf2.nblocks)), block(NT);
 	switch (role) {
 		case TG_ROLE_QKV_EMBED: hipLaunchKernelGGL(tg_gemv_qkv_embed, grid, block, 0, s, g); break;
 		case TG_ROLE_QKV: hipLaunchKernelGGL(tg_gemv_qkv, grid, block, 0, s, g); break;

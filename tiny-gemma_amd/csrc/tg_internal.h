@@ -49,6 +49,7 @@ struct TgPrefetch {
 };
 
 __device__ __forceinline__ void tg_prefetch_block(const TgPrefetch &p, int first_extra_block) {
+	if (p.ptr == nullptr) return;
 	const int pb = (int)blockIdx.x - first_extra_block;
 	const int x = (int)(blockIdx.x & 7u), q = pb >> 3, Q = p.nblocks >> 3;
 	for (int t = x + 8 * q; t < p.ntiles; t += 8 * Q) {
@@ -58,6 +59,12 @@ __device__ __forceinline__ void tg_prefetch_block(const TgPrefetch &p, int first
 			asm volatile("" ::"v"(v));               // the value is not needed, the load is
 		}
 	}
+}
+
+// Two jobs: the first pf.nblocks extra workgroups serve pf, the following pf2.nblocks serve pf2.
+__device__ __forceinline__ void tg_prefetch_dispatch(const TgPrefetch &p1, const TgPrefetch &p2, int first_extra_block) {
+	if ((int)blockIdx.x < first_extra_block + p1.nblocks) tg_prefetch_block(p1, first_extra_block);
+	else tg_prefetch_block(p2, first_extra_block + p1.nblocks);
 }
 
 // ---- GEMV launch description --------------------------------------------------------------
@@ -87,6 +94,7 @@ struct TgGemv {
 	int vocab;
 	float emb_scale;       // EMBED: float(sqrt(hidden))
 	const int *pos;        // ATTN_MERGE: device counters (pos[0] = position of this token)
+	int host_pos;          // ATTN_MERGE: the same position as a launch argument, or -1 to read the device counter
 	int attn_max_pos;      // ATTN_MERGE: cache slots of this layer
 	int attn_chunk;        // ATTN_MERGE: keys per attention workgroup
 	const float *part_acc; // ATTN_MERGE: [nb][4][256]
@@ -98,7 +106,7 @@ struct TgGemv {
 	int lut_size;
 	float *blk_val;        // LOGITS: per-workgroup maximum and its index, [ntiles]
 	int *blk_idx;
-	TgPrefetch pf;         // weights of the next launch (optional)
+	TgPrefetch pf, pf2;    // weights of the next launches (optional); the extra workgroups are split between them
 };
 
 struct TgAttnDecode {
@@ -109,12 +117,13 @@ struct TgAttnDecode {
 	int max_pos;             // slots (ring for local layers, linear for global)
 	const int *pos;          // device counters: pos[0] = position_ptr, pos[1]/pos[2] = buffer_ptr of local/global layers
 	int bp_index;            // 1 (local layer) or 2 (global layer)
+	int host_pos, host_bp;   // the same counters as launch arguments (saves a dependent load), or -1 to read the device ones
 	int chunk;               // keys per workgroup
 	float *part_acc;         // [nblocks][n_head][hd]
 	float *part_ml;          // [nblocks][n_head][2]
 	int n_head;
 	int nblocks;             // attention workgroups in the grid; workgroups past them prefetch
-	TgPrefetch pf;           // weights of the next launch (optional)
+	TgPrefetch pf, pf2;      // weights of the next launches (optional)
 };
 
 enum { TG_ROLE_PLAIN = 0, TG_ROLE_QKV_EMBED, TG_ROLE_QKV, TG_ROLE_OPROJ, TG_ROLE_UPGATE, TG_ROLE_DOWN, TG_ROLE_LMHEAD,
