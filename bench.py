@@ -98,6 +98,8 @@ def main():
     ap.add_argument("--seed", type=int, default=20251)
     ap.add_argument("--cpu-steps", type=int, default=128, help="decode steps of the CPU baseline sample (0 = skip)")
     ap.add_argument("--profile-steps", type=int, default=32)
+    ap.add_argument("--long-prefill", type=int, default=4096,
+                    help="tokens of the extra long-prompt prefill measurement, reported beside the headline (0 = skip)")
     ap.add_argument("--graphs", action="store_true", help="replay captured HIP graphs instead of plain stream launches")
     ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
     ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
@@ -189,6 +191,37 @@ def main():
     tg.synchronize()
     lm_iso_us = ev.elapsed_ms(e0, e1) * 1e3 / 50
 
+    # ---- the plain int8 GEMV entry point (launch_qgemv on device-resident operands) at the LM-head shape ----
+    h, V = cfg.hidden_size, cfg.n_vocab
+    tail = image[-(h * V + 4 * V):]
+    qw = tg.QWeight(tail[:h * V].view(np.int8).reshape(h, V), tail[h * V:].view(np.float32))
+    xd = tg.DeviceBuffer.from_numpy(rng.standard_normal(h).astype(np.float32))
+    yd = tg.DeviceBuffer(4 * V)
+    for _ in range(5):
+        qw.gemv(yd, xd)
+    tg.synchronize()
+    ev.record(e0, stream)
+    for _ in range(50):
+        qw.gemv(yd, xd)
+    ev.record(e1, stream)
+    tg.synchronize()
+    bare_us = ev.elapsed_ms(e0, e1) * 1e3 / 50
+    qw.free()
+
+    # ---- long-prompt prefill (the matrix-matrix path) on a fresh session ----
+    long_prefill = None
+    if args.long_prefill > 0:
+        s2 = model.session()
+        lp = rng.integers(0, cfg.n_vocab, args.long_prefill).astype(np.int32)
+        s2.prefill(lp, want_logits=False)
+        s2.reset()
+        tg.synchronize()
+        t0 = time.perf_counter()
+        s2.prefill(lp, want_logits=False)
+        dt = time.perf_counter() - t0
+        long_prefill = {"tokens": args.long_prefill, "ms": 1e3 * dt, "tok_s": args.long_prefill / dt}
+        del s2
+
     tok_s = args.steps / wall
     out = {
         "metric": "decode_tokens_per_s",
@@ -225,6 +258,14 @@ def main():
             "back_to_back_us": lm_iso_us,
             "back_to_back_GBps": lm_bytes / lm_iso_us / 1e3,
         },
+        "gemv_lmhead_shape": {
+            "entry": "tg_qgemv_dev",
+            "shape": [h, V],
+            "avg_launch_us": bare_us,
+            "GBps": lm_bytes / bare_us / 1e3,
+            "frac": lm_bytes / bare_us / 1e3 / HBM_PEAK_GBS,
+            "timing": "HIP events around 50 back-to-back launches of the plain GEMV (no norm prologue, no argmax epilogue)",
+        },
         "decode_step": {
             "gpu_ms_per_step_events": gpu_ms / args.steps,
             "weight_bytes_per_token": step_bytes,
@@ -232,7 +273,7 @@ def main():
             "frac_of_hbm_roofline": step_bytes * tok_s / 1e9 / HBM_PEAK_GBS,
             "avg_kernel_us": per_kernel_us,
         },
-        "prefill": {"tokens": n_prompt, "tok_s_forward_only": n_prompt / t_prefill},
+        "prefill": {"tokens": n_prompt, "tok_s_forward_only": n_prompt / t_prefill, "long_prompt": long_prefill},
         "setup_s": {"generate_weights": t_gen, "upload_and_retile": t_load},
         "device": dev,
     }

@@ -9,8 +9,8 @@
 //            partial (max, sum, unnormalised output) of its chunk; the partials are merged in the
 //            prologue of the output projection (tg_gemv.hip) — via attn_merge_kernel first when
 //            there are many.  Softmax is order independent, so only fp32 rounding differs.
-//   prefill: ops::attention_prefill (ops.hpp:377-526) — causal; local layers see keys
-//            qs-window .. qs inclusive (window+1 keys, ops.hpp:437-443).
+//   prefill: the per-row q/k work only (qk_norm_rope_rows_kernel); the attention itself is in
+//            tg_attn_prefill.hip.
 
 #include "tg_internal.h"
 
@@ -323,70 +323,6 @@ __global__ __launch_bounds__(ANT) void qk_norm_rope_rows_kernel(float *q, float 
 	if (s >= start) vc[(size_t)(s - start) * HD + tid] = v[(size_t)s * ldkv + tid];
 }
 
-// One workgroup per query position, all 4 heads; keys streamed in chunks with a running
-// (max, sum, acc) per head.  q rows are [S][ldq] with head h at column h*256; k, v rows [S][ldkv].
-__global__ __launch_bounds__(ANT) void attn_prefill_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
-                                                           int ldkv, int ldo, int is_sw, int window) {
-	__shared__ float qs[NH][HD];
-	__shared__ float sc[NH][MAXCHUNK];
-	__shared__ float s_m[NH], s_l[NH], s_c[NH];
-
-	const int qi = blockIdx.x, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-#pragma unroll
-	for (int h = 0; h < NH; h++) qs[h][tid] = q[(size_t)qi * ldq + h * HD + tid] * 0.0625f;  // ops.hpp:406,463
-	if (tid < NH) { s_m[tid] = -INFINITY; s_l[tid] = 0.0f; }
-	__syncthreads();
-	int kbeg = 0;
-	if (is_sw) kbeg = (qi >= window) ? qi - window : 0;  // ops.hpp:437-441
-	const int kend = qi + 1;
-	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
-	for (int k0 = kbeg; k0 < kend; k0 += MAXCHUNK) {
-		const int n = (kend - k0 < MAXCHUNK) ? kend - k0 : MAXCHUNK;
-		chunk_scores(qs, k, ldkv, nullptr, -1, k0, n, sc, tid);
-		__syncthreads();
-		{
-			float m = -INFINITY;
-			for (int j = lane; j < n; j += 64) m = fmaxf(m, sc[w][j]);
-			m = wmax(m);
-			const float m_old = s_m[w];
-			const float m_new = fmaxf(m_old, m);
-			float l = 0.0f;
-			for (int j = lane; j < n; j += 64) {
-				const float p = expf(sc[w][j] - m_new);
-				sc[w][j] = p;
-				l += p;
-			}
-			l = wsum(l);
-			if (lane == 0) {
-				const float c = expf(m_old - m_new);  // 0 on the first chunk
-				s_c[w] = c;
-				s_l[w] = fmaf(s_l[w], c, l);
-				s_m[w] = m_new;
-			}
-		}
-		__syncthreads();
-#pragma unroll
-		for (int h = 0; h < NH; h++) acc[h] *= s_c[h];
-		for (int j0 = 0; j0 < n; j0 += 8) {
-			float vv[8];
-#pragma unroll
-			for (int u = 0; u < 8; u++) {
-				const int jj = j0 + u;
-				vv[u] = v[(size_t)(k0 + (jj < n ? jj : 0)) * ldkv + tid];
-			}
-#pragma unroll
-			for (int u = 0; u < 8; u++) {
-				if (j0 + u < n) {
-#pragma unroll
-					for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][j0 + u], vv[u], acc[h]);
-				}
-			}
-		}
-		__syncthreads();
-	}
-#pragma unroll
-	for (int h = 0; h < NH; h++) o[(size_t)qi * ldo + h * HD + tid] = acc[h] / s_l[h];
-}
 
 }  // namespace
 
@@ -411,9 +347,3 @@ void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float
 	                   max_pos, S, ldq, ldkv);
 }
 
-void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, hipStream_t s) {
-	(void)n_head;
-	(void)hd;
-	hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)S), dim3(ANT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window);
-}

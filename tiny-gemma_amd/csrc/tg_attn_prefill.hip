@@ -1,0 +1,172 @@
+// Prefill attention (ops::attention_prefill, ops.hpp:377-526) on the fp32 matrix cores.
+//
+// The reference walks every (query, head) pair over its keys with a renormalising online softmax.
+// Here a workgroup owns 16 consecutive query positions and all 4 query heads (one wave per head: the
+// heads share the single KV head, so each K/V tile is fetched once per workgroup) and streams the
+// keys in tiles of 32 through LDS.  Both products run on v_mfma_f32_16x16x4_f32: fp32 operands, exact
+// fp32 products, fp32 accumulation, so only the summation order differs from the reference.
+//
+//   scores, transposed:  S^T[key][query] = K[key][:] . Q[query][:]      A = K tile (LDS), B = Q (registers)
+//   lane (c = lane % 16, g = lane / 16) then holds S^T[4g + i][c], i = 0..3: the scores of query c,
+//   which is exactly the A-operand order the second product needs:
+//   output:              O[query][d] += P[query][key] * V[key][d]       A = P (registers), B = V tile (LDS)
+//
+// The k index of an MFMA step is arbitrary as long as A and B agree, so step (t, i) of the score product
+// uses k = 16 t + 4 g + i: every lane fetches 4 consecutive floats of its K row with one 16-byte LDS
+// read, and the Q registers are filled with 16-byte global loads.  LDS rows are 260 floats apart: the 16
+// rows of a read hit 16 different groups of 4 banks (scores) and the 4 rows of a V read are 16 banks
+// apart.  Keys outside a query's range (causal; local layers: qs-window .. qs, ops.hpp:437-443) get a
+// score of -inf.
+
+#include "tg_internal.h"
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int HD = 256;    // head_dim
+constexpr int NH = 4;      // query heads (= waves per workgroup)
+constexpr int TQ = 16;     // query positions per workgroup
+constexpr int TK = 32;     // keys per LDS tile
+constexpr int LDS_LD = 260;
+constexpr int PNT = 256;
+
+__global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
+                                                               int ldkv, int ldo, int is_sw, int window) {
+	__shared__ __attribute__((aligned(16))) float Ks[TK][LDS_LD];
+	__shared__ __attribute__((aligned(16))) float Vs[TK][LDS_LD];
+
+	const int tid = threadIdx.x, lane = tid & 63, head = tid >> 6, c = lane & 15, g = lane >> 4;
+	// late query tiles of a causal layer see the most keys: start them first
+	const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ;
+	const int qpos = q0 + c;                         // the query whose scores this lane holds
+	const int qrow = qpos < S ? qpos : S - 1;
+	const int kb = (is_sw && q0 > window) ? q0 - window : 0;
+	const int ke = (q0 + TQ < S) ? q0 + TQ : S;      // exclusive
+	const int ntiles = (ke - kb + TK - 1) / TK;
+	const int klo = is_sw ? qpos - window : 0;       // this query's first key (may be negative)
+
+	// K/V tile staging: thread covers rows (tid/64) + 4u, 16-byte piece tid % 64
+	const int ld_row = tid >> 6, ld_piece = tid & 63;
+	f32x4 kpre[TK / 4], vpre[TK / 4];
+	auto fetch = [&](int tile) {
+#pragma unroll
+		for (int u = 0; u < TK / 4; u++) {
+			int j = kb + tile * TK + ld_row + 4 * u;
+			j = j < ke ? j : ke - 1;
+			kpre[u] = *reinterpret_cast<const f32x4 *>(k + (size_t)j * ldkv + 4 * ld_piece);
+			vpre[u] = *reinterpret_cast<const f32x4 *>(v + (size_t)j * ldkv + 4 * ld_piece);
+		}
+	};
+	fetch(0);
+
+	// Q as B operand: qreg[t][i] = Q[qrow][16 t + 4 g + i] / sqrt(hd)   (ops.hpp:406,463)
+	f32x4 qreg[HD / 16];
+	{
+		const float *qp = q + (size_t)qrow * ldq + head * HD + 4 * g;
+#pragma unroll
+		for (int t = 0; t < HD / 16; t++) {
+			const float4 x = *reinterpret_cast<const float4 *>(qp + 16 * t);
+			qreg[t] = f32x4{x.x * 0.0625f, x.y * 0.0625f, x.z * 0.0625f, x.w * 0.0625f};
+		}
+	}
+
+	f32x4 oacc[HD / 16];  // oacc[dt][i] = O[query 4 g + i][16 dt + c]
+#pragma unroll
+	for (int dt = 0; dt < HD / 16; dt++) oacc[dt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+	float m_run = -INFINITY, l_run = 0.0f;  // of query c (replicated in the 4 lanes sharing c)
+
+	for (int tile = 0; tile < ntiles; tile++) {
+		__syncthreads();  // everyone is done with the previous tile
+#pragma unroll
+		for (int u = 0; u < TK / 4; u++) {
+			*reinterpret_cast<f32x4 *>(&Ks[ld_row + 4 * u][4 * ld_piece]) = kpre[u];
+			*reinterpret_cast<f32x4 *>(&Vs[ld_row + 4 * u][4 * ld_piece]) = vpre[u];
+		}
+		__syncthreads();
+		if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during the products
+
+		// ---- scores of the tile's two groups of 16 keys ----
+		f32x4 s0 = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+#pragma unroll
+		for (int t = 0; t < HD / 16; t++) {
+			const f32x4 a0 = *reinterpret_cast<const f32x4 *>(&Ks[c][16 * t + 4 * g]);
+			const f32x4 a1 = *reinterpret_cast<const f32x4 *>(&Ks[16 + c][16 * t + 4 * g]);
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[i], qreg[t][i], s0, 0, 0, 0);
+				s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[i], qreg[t][i], s1, 0, 0, 0);
+			}
+		}
+		// ---- mask + online softmax for query c ----
+		const int j0 = kb + tile * TK + 4 * g;
+		float tmax = -INFINITY;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int ja = j0 + i, jb = j0 + 16 + i;
+			if (ja > qpos || ja < klo) s0[i] = -INFINITY;
+			if (jb > qpos || jb < klo) s1[i] = -INFINITY;
+			tmax = fmaxf(tmax, fmaxf(s0[i], s1[i]));
+		}
+		tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+		tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+		const float m_new = fmaxf(m_run, tmax);  // finite from the first tile on: it holds a valid key of every query
+		const float alpha = expf(m_run - m_new);
+		float psum = 0.0f;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			s0[i] = expf(s0[i] - m_new);
+			s1[i] = expf(s1[i] - m_new);
+			psum += s0[i] + s1[i];
+		}
+		psum += __shfl_xor(psum, 16, 64);
+		psum += __shfl_xor(psum, 32, 64);
+		l_run = fmaf(l_run, alpha, psum);
+		m_run = m_new;
+		// rescale the output rows this lane holds (queries 4 g + i)
+		float ar[4];
+#pragma unroll
+		for (int i = 0; i < 4; i++) ar[i] = __shfl(alpha, 4 * g + i, 64);
+#pragma unroll
+		for (int dt = 0; dt < HD / 16; dt++) {
+#pragma unroll
+			for (int i = 0; i < 4; i++) oacc[dt][i] *= ar[i];
+		}
+		// ---- O += P V : step i of key group kt uses key 16 kt + 4 g + i ----
+#pragma unroll
+		for (int dt = 0; dt < HD / 16; dt++) {
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(s0[i], Vs[4 * g + i][16 * dt + c], oacc[dt], 0, 0, 0);
+			}
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(s1[i], Vs[16 + 4 * g + i][16 * dt + c], oacc[dt], 0, 0, 0);
+			}
+		}
+	}
+
+	float lr[4];
+#pragma unroll
+	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int qo = q0 + 4 * g + i;
+		if (qo < S) {
+			float *op = o + (size_t)qo * ldo + head * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+		}
+	}
+}
+
+}  // namespace
+
+// q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
+void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
+                            int ldo, int is_sw, int window, hipStream_t s) {
+	(void)n_head;
+	(void)hd;
+	hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)((S + TQ - 1) / TQ)), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
+	                   window);
+}
