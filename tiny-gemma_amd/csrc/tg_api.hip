@@ -19,9 +19,9 @@ namespace {
 
 thread_local std::string g_err;
 bool g_inited = false;
-int g_gemm_mfma = 1;            // prefill GEMM: 1 = MFMA (fp16 hi/lo split), 0 = exact-order fp32 on the vector ALUs
-_Float16 *g_apack = nullptr;    // scratch of the stand-alone GEMM entry points
-size_t g_apack_halfs = 0;
+int g_gemm_mfma = 1;            // prefill GEMM: 1 = int8 MFMA on three digit planes, 0 = exact-order fp32 on the vector ALUs
+int8_t *g_apack = nullptr;      // scratch of the stand-alone GEMM entry points
+size_t g_apack_bytes = 0;
 float *g_rowscale = nullptr;
 size_t g_rowscale_n = 0;
 int g_prefetch_plan = 0;        // which launch prefetches which weights (experiment knob)
@@ -42,7 +42,8 @@ int ensure_init() {
 
 // A matrix on the device.  `W` is the GEMV layout: ntiles tiles of C columns, each a contiguous
 // [K/4][C][4] slab (C chosen per matrix so that narrow matrices still give hundreds of
-// workgroups).  `Wg` (optional) is the same matrix in 128-column tiles for the prefill GEMM.
+// workgroups).  `Wg` (optional) is the same matrix in 128-column tiles of [K/16][128][16] for the
+// int8 MFMA prefill GEMM (B-operand order).
 struct PackedMat {
 	int8_t *W = nullptr;
 	float *scales = nullptr;   // per virtual column, GEMV tile order
@@ -79,9 +80,25 @@ void pack_host(int8_t *dst, const int8_t *src, int K, int N, int C) {
 	}
 }
 
+// host: [K][N] row-major -> tiles of 128 columns, each [K/16][128][16 consecutive k] (MFMA B-operand order)
+void pack_host_mfma(int8_t *dst, const int8_t *src, int K, int N) {
+	const int k16s = K / 16;
+	for (int t = 0; t < N / TG_CT; t++) {
+		for (int kb = 0; kb < k16s; kb++) {
+			int8_t *d = dst + ((size_t)t * k16s + kb) * TG_CT * 16;
+			for (int j = 0; j < 16; j++) {
+				const int8_t *r = src + (size_t)(16 * kb + j) * N + (size_t)t * TG_CT;
+				for (int c = 0; c < TG_CT; c++) d[16 * c + j] = r[c];
+			}
+		}
+	}
+}
+
+// C > 0: GEMV tiling of C columns; C = 0: MFMA tiling
 int upload_tiles(int8_t **Wd, float **sd, const int8_t *host_rowmajor, const float *host_scales, int K, int N, int C) {
 	std::vector<int8_t> tmp((size_t)K * N);
-	pack_host(tmp.data(), host_rowmajor, K, N, C);
+	if (C > 0) pack_host(tmp.data(), host_rowmajor, K, N, C);
+	else pack_host_mfma(tmp.data(), host_rowmajor, K, N);
 	TG_HIP(hipMalloc((void **)Wd, (size_t)K * N));
 	TG_HIP(hipMalloc((void **)sd, (size_t)N * sizeof(float)));
 	TG_HIP(hipMemcpy(*Wd, tmp.data(), (size_t)K * N, hipMemcpyHostToDevice));
@@ -100,7 +117,7 @@ int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_s
 	if (int rc = upload_tiles(&p->W, &p->scales, host_rowmajor, host_scales, K, N, p->C)) return rc;
 	if (with_gemm) {
 		p->ntiles_g = N / TG_CT;
-		if (int rc = upload_tiles(&p->Wg, &p->scales_g, host_rowmajor, host_scales, K, N, TG_CT)) return rc;
+		if (int rc = upload_tiles(&p->Wg, &p->scales_g, host_rowmajor, host_scales, K, N, 0)) return rc;
 	}
 	return TG_OK;
 }
@@ -133,10 +150,10 @@ int upload_up_gate(PackedMat *p, const int8_t *up, const float *ups, const int8_
 	p->ntiles = p->N / p->C;
 	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, p->C);
 	if (int rc = upload_tiles(&p->W, &p->scales, cat.data(), catsc.data(), K, 2 * f, p->C)) return rc;
-	// GEMM layout: 128-column tiles, tile 2t = up columns [128t, 128t+128), tile 2t+1 = the same gate columns
+	// MFMA layout: 128-column tiles of 64 up columns followed by the same 64 gate columns
 	p->ntiles_g = p->N / TG_CT;
-	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, 2 * TG_CT);
-	return upload_tiles(&p->Wg, &p->scales_g, cat.data(), catsc.data(), K, 2 * f, TG_CT);
+	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, TG_CT);
+	return upload_tiles(&p->Wg, &p->scales_g, cat.data(), catsc.data(), K, 2 * f, 0);
 }
 
 void free_packed(PackedMat *p) {
@@ -162,12 +179,13 @@ TgGemv gemv_base(const PackedMat &p) {
 
 // C[m][N] = scales * (A[m][K] . W) through the selected GEMM; apack/rowscale are scratch for the MFMA path.
 void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
-                 int lut_size, _Float16 *apack, float *rowscale) {
+                 int lut_size, int8_t *apack, float *rowscale) {
 	if (g_gemm_mfma) {
-		tg_launch_split_pack(A, lda, m, p.K, apack, rowscale, g_stream);
+		tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, g_stream);
 		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, g_stream);
 	} else {
-		tg_launch_gemm(C, A, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, g_stream);
+		(void)lda;  // the exact kernel reads dense rows (lda == K at every call site)
+		tg_launch_gemm(C, A, p.W, p.scales, m, p.K, p.ntiles, p.C, epi, lut, gmin, geps, lut_size, g_stream);
 	}
 }
 
@@ -392,18 +410,18 @@ int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logi
 
 int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
-	if (!w->p.Wg) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "no GEMM tiling was built for this matrix (outDim too large)");
+	if (g_gemm_mfma && !w->p.Wg) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "no MFMA tiling was built for this matrix (outDim too large)");
 	if (g_gemm_mfma) {
-		const size_t need = tg_gemm_mfma_apack_halfs(m, w->p.K), need_rs = (size_t)((m + 127) / 128) * 128;
-		if (need > g_apack_halfs || need_rs > g_rowscale_n) {
+		const size_t need = tg_gemm_mfma_apack_bytes(m, w->p.K), need_rs = 2 * tg_gemm_mfma_rows(m);
+		if (need > g_apack_bytes || need_rs > g_rowscale_n) {
 			TG_HIP(hipStreamSynchronize(g_stream));
 			if (g_apack) (void)hipFree(g_apack);
 			if (g_rowscale) (void)hipFree(g_rowscale);
 			g_apack = nullptr;
 			g_rowscale = nullptr;
-			TG_HIP(hipMalloc((void **)&g_apack, need * sizeof(_Float16)));
+			TG_HIP(hipMalloc((void **)&g_apack, need));
 			TG_HIP(hipMalloc((void **)&g_rowscale, need_rs * sizeof(float)));
-			g_apack_halfs = need;
+			g_apack_bytes = need;
 			g_rowscale_n = need_rs;
 		}
 	}
@@ -1068,7 +1086,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	const size_t S = (size_t)n;
 	int *d_ids = nullptr;
 	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr;
-	_Float16 *apack = nullptr;
+	int8_t *apack = nullptr;
 	auto cleanup = [&]() {
 		void *ps[] = {d_ids, x, xn, qkv, ao, t, hb, rowscale, apack};
 		for (void *p : ps)
@@ -1090,8 +1108,8 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	TG_TRY(hipMalloc((void **)&t, sizeof(float) * S * h));
 	TG_TRY(hipMalloc((void **)&hb, sizeof(float) * S * f));
 	if (g_gemm_mfma) {
-		TG_TRY(hipMalloc((void **)&apack, sizeof(_Float16) * tg_gemm_mfma_apack_halfs(n, std::max(f, qo))));
-		TG_TRY(hipMalloc((void **)&rowscale, sizeof(float) * (size_t)((n + 127) / 128) * 128));
+		TG_TRY(hipMalloc((void **)&apack, tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h))));
+		TG_TRY(hipMalloc((void **)&rowscale, sizeof(float) * 2 * tg_gemm_mfma_rows(n)));
 	}
 	const bool keep_taps = n <= PREFILL_TAP_MAX_ROWS;
 	if (s->taps) {

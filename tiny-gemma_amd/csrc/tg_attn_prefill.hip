@@ -77,13 +77,13 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 	float m_run = -INFINITY, l_run = 0.0f;  // of query c (replicated in the 4 lanes sharing c)
 
 	for (int tile = 0; tile < ntiles; tile++) {
-		__syncthreads();  // everyone is done with the previous tile
+		tg_lds_barrier();  // everyone is done with the previous tile
 #pragma unroll
 		for (int u = 0; u < TK / 4; u++) {
 			*reinterpret_cast<f32x4 *>(&Ks[ld_row + 4 * u][4 * ld_piece]) = kpre[u];
 			*reinterpret_cast<f32x4 *>(&Vs[ld_row + 4 * u][4 * ld_piece]) = vpre[u];
 		}
-		__syncthreads();
+		tg_lds_barrier();
 		if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during the products
 
 		// ---- scores of the tile's two groups of 16 keys ----

@@ -1,200 +1,271 @@
-// Prefill int8-weight GEMM on the matrix cores (gfx950 MFMA), replacing gemm::launch_qgemm
-// (csrc/include/linalg.hpp:210-308 of the reference):  C[m][n] = scales[n] * sum_k A[m][k] * float(W[k][n]).
+// Prefill int8-weight GEMM on the integer matrix cores (gfx950 v_mfma_i32_32x32x32_i8), replacing
+// gemm::launch_qgemm (csrc/include/linalg.hpp:210-308 of the reference):
+//     C[m][n] = scales[n] * sum_k A[m][k] * float(W[k][n]).
 //
-// The reference accumulates every element in one fp32 fused chain.  MFMA has no fp32-input mode fast
-// enough to matter (fp32 MFMA peaks at 157 TFLOP/s, fp16 at 2.5 PFLOP/s) and rounding the activations to
-// one 16-bit value would cost 1e-3 of accuracy, which the model's step-function GeLU table turns into
-// visible drift.  So the contraction is done at fp32-equivalent accuracy on fp16 MFMA:
+// The reference accumulates every element in one fp32 fused chain.  The weights are already int8, so the
+// contraction is moved to integer arithmetic altogether:
 //
-//   * int8 weights are converted to fp16 exactly (|w| <= 127);
-//   * each activation row is scaled by a power of two so that its largest magnitude lies in
-//     [2^10, 2^11) (exact), then split a' = hi + lo with hi = fp16(a'), lo = fp16(a' - hi):
-//     22 mantissa bits, |lo| <= 0.5, no subnormal hi for anything that matters;
-//   * hi.w and lo.w are exact in fp32 (11 + 7 bits); both are accumulated into the same fp32 MFMA
-//     accumulator, i.e. the kernel runs a [hi|lo] x [W;W] product: 2 MFMA per weight tile;
-//   * the epilogue multiplies by the row's inverse power of two and the column scale.
+//   * each activation row is scaled by a power of two (exact) so that its largest magnitude lies in
+//     [2^21, 2^22) and rounded to an integer xi (22 bits + sign: the row maximum keeps close to fp32
+//     precision, smaller elements keep the same absolute precision);
+//   * xi is written as three signed base-256 digits, xi = 65536 a2 + 256 a1 + a0, each an int8;
+//   * three int8 x int8 -> int32 MFMA contractions (one per digit plane) run against the untouched int8
+//     weights; |sum| <= 127 * 128 * K < 2^31 for every legal K, so the integer sums are exact;
+//   * the epilogue recombines the planes in fp32 and applies the row's inverse power of two and the
+//     column scale.
 //
-// Data flow: a pre-pass (split_pack_rows_kernel) writes the hi/lo halves directly in MFMA A-operand
-// order, so every wave fetches its A operands with fully coalesced 16-byte loads straight from global
-// memory (a wave owns 32 rows: nothing to share, no LDS).  Weight tiles (128 columns, shared by the 4
-// waves of a workgroup) are loaded from the packed int8 slab, converted once per workgroup and staged in
-// LDS in B-operand order (double buffered, one barrier per 64 rows of K).
+// Nothing in the inner loop converts anything: weight tiles go global -> LDS as raw bytes and are read
+// back as MFMA B operands, digit planes are stored in A-operand order by the quantising pre-pass and are
+// fetched straight from global memory with 16-byte loads (a wave owns its 32 rows: nothing to share).
+//
+// Layouts
+//   weights (built at load time): [tile of 128 columns][K/16][128 columns][16 consecutive k]
+//   activations: [tile of 32 rows][K/32][3 planes][64 lanes][16 bytes], lane = row % 32 + 32 * ((k % 32) / 16)
+// The k order inside an MFMA step is irrelevant as long as both operands use the same one: lane half hb of
+// both operands carries k = 16 hb .. 16 hb + 15 of the step.
+//
+// For the fused up|gate matrix a tile holds 64 up columns followed by the same 64 gate columns, so
+// gelu(gate) * up (modules.hpp:190-195) is formed in the epilogue and the workgroup writes 64 columns.
 
 #include "tg_internal.h"
 
+#include <type_traits>
+
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int GNT = 256;    // threads per workgroup: 4 waves, each owns 32 rows x 128 (or 256) columns
-constexpr int KSTAGE = 64;  // rows of K per LDS stage
+constexpr int GNT = 256;     // threads per workgroup: 4 waves, each owns 32 rows x 128 columns
+constexpr int KSTAGE = 64;   // rows of K per LDS stage
+constexpr int QBITS = 22;    // row maxima are scaled into [2^(QBITS-1), 2^QBITS)
+constexpr int LUT_LDS_MAX = 4096;  // GeLU tables up to this many entries are staged in LDS (Bs holds 16 KB)
 
-__device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin, float geps, int size) {
-	int idx = (int)((x - gmin) / geps);
+// ginv != 0: the table step is a power of two and ginv its exact reciprocal, so the product equals the quotient
+__device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin, float geps, float ginv, int size) {
+	int idx = (ginv != 0.0f) ? (int)((x - gmin) * ginv) : (int)((x - gmin) / geps);
 	if (idx < 0) return 0.0f;
 	if (idx >= size) return x;
 	return lut[idx];
 }
 
-// A [M][lda] fp32 -> Apack [mtiles][K/16][2][64][8] fp16 (hi block, then lo block, each in A-operand lane
-// order: lane = row % 32 + 32 * ((k % 16) / 8), 8 consecutive k per lane) and rowscale[m] = 2^-e.
-// One workgroup per tile of 32 rows; rows >= M are written as zeros.
-__global__ __launch_bounds__(GNT) void split_pack_rows_kernel(const float *A, int lda, int M, int K, _Float16 *Apack, float *rowscale) {
-	__shared__ float smax[8][32];
-	const int t = threadIdx.x, r = t & 31, kb = t >> 5;
-	const int mtile = blockIdx.x, m = mtile * 32 + r;
-	const bool valid = m < M;
-	const float *row = A + (size_t)(valid ? m : 0) * lda;
-	const int k8s = K >> 3;
+// One wave per row: mul[m] = 2^s with max|A[m][:]| * 2^s in [2^21, 2^22), inv[m] = 2^-s.
+__global__ __launch_bounds__(GNT) void row_scale_kernel(const float *A, int lda, int M, int K, float *mul, float *inv, int Mpad) {
+	const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (m >= Mpad) return;
 	float amax = 0.0f;
-	if (valid) {
-		for (int kk = kb; kk < k8s; kk += 8) {
-			const float4 a0 = *reinterpret_cast<const float4 *>(row + 8 * kk), a1 = *reinterpret_cast<const float4 *>(row + 8 * kk + 4);
-			amax = fmaxf(amax, fmaxf(fmaxf(fabsf(a0.x), fabsf(a0.y)), fmaxf(fabsf(a0.z), fabsf(a0.w))));
-			amax = fmaxf(amax, fmaxf(fmaxf(fabsf(a1.x), fabsf(a1.y)), fmaxf(fabsf(a1.z), fabsf(a1.w))));
+	if (m < M) {
+		const f32x4 *row = reinterpret_cast<const f32x4 *>(A + (size_t)m * lda);
+		for (int i = lane; i < (K >> 2); i += 64) {
+			const f32x4 a = row[i];
+			amax = fmaxf(amax, fmaxf(fmaxf(fabsf(a[0]), fabsf(a[1])), fmaxf(fabsf(a[2]), fabsf(a[3]))));
 		}
 	}
-	smax[kb][r] = amax;
-	__syncthreads();
 #pragma unroll
-	for (int i = 0; i < 8; i++) amax = fmaxf(amax, smax[i][r]);
-	int e = 0;
-	float scale = 1.0f, inv = 1.0f;
-	if (amax > 0.0f && amax < INFINITY) {
-		(void)frexpf(amax, &e);          // amax = f * 2^e, f in [0.5, 1)
-		scale = ldexpf(1.0f, 11 - e);    // amax * scale in [2^10, 2^11)
-		inv = ldexpf(1.0f, e - 11);
-	}
-	if (kb == 0) rowscale[mtile * 32 + r] = inv;
-	_Float16 *tilebase = Apack + (size_t)mtile * (size_t)(K >> 4) * 1024;
-	for (int kk = kb; kk < k8s; kk += 8) {
-		float a[8];
-		if (valid) {
-			const float4 a0 = *reinterpret_cast<const float4 *>(row + 8 * kk), a1 = *reinterpret_cast<const float4 *>(row + 8 * kk + 4);
-			a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w; a[4] = a1.x; a[5] = a1.y; a[6] = a1.z; a[7] = a1.w;
-		} else {
-#pragma unroll
-			for (int i = 0; i < 8; i++) a[i] = 0.0f;
+	for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+	if (lane == 0) {
+		float s = 1.0f, r = 1.0f;
+		if (amax > 0.0f && amax < INFINITY) {
+			int e;
+			(void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+			s = ldexpf(1.0f, QBITS - e);
+			r = ldexpf(1.0f, e - QBITS);
 		}
-		half8 hi, lo;
-#pragma unroll
-		for (int i = 0; i < 8; i++) {
-			const float s = a[i] * scale;
-			const _Float16 h = (_Float16)s;
-			hi[i] = h;
-			lo[i] = (_Float16)(s - (float)h);
-		}
-		_Float16 *dst = tilebase + (size_t)(kk >> 1) * 1024 + (size_t)(r + 32 * (kk & 1)) * 8;
-		*reinterpret_cast<half8 *>(dst) = hi;
-		*reinterpret_cast<half8 *>(dst + 512) = lo;
+		mul[m] = s;
+		inv[m] = r;
 	}
 }
 
-// NTB = B tiles per workgroup: 1 (plain) or 2 (the up|gate pair of one block of columns, for gelu(gate)*up)
-template <int NTB>
-__global__ __launch_bounds__(GNT) void gemm_mfma_kernel(float *C, const _Float16 *Apack, const float *rowscale, const int8_t *Wg,
-                                                        const float *scales, int M, int K, int ldc, const float *lut, float gmin,
-                                                        float geps, int lut_size) {
-	// B operands of one stage: [tile][kblk (8 rows of K)][column][8 halfs], double buffered
-	__shared__ __attribute__((aligned(16))) _Float16 Bs[2][NTB][KSTAGE / 8][TG_CT][8];
-
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-	const int tile0 = blockIdx.x * NTB;
-	const int mtile = blockIdx.y * 4 + w;
-	const int kgs = K >> 2, nstage = K / KSTAGE;
-	const size_t slab = (size_t)K * TG_CT;
-
-	// this thread's two 16-byte pieces of every B stage: piece p = tid and tid + 256
-	// (p / 32 = kg within the stage, p % 32 = group of 4 columns)
-	const i32x4 *wsrc[NTB];
+// A [M][lda] fp32 -> digit planes in A-operand order.  Workgroup = 32 rows x 128 k; thread = one lane's 16
+// bytes of one (k step, half): row r = tid % 32, k = 128 blockIdx.y + 16 (tid / 32) .. + 15.
+__global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda, int M, int K, const float *mul, int8_t *Apack) {
+	const int tid = threadIdx.x, r = tid & 31, kq = tid >> 5;
+	const int mtile = blockIdx.x, m = mtile * 32 + r;
+	const int k0 = blockIdx.y * 128 + 16 * kq;
+	i32x4 pl[3] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+	if (m < M) {
+		const float s = mul[m];
+		const f32x4 *src = reinterpret_cast<const f32x4 *>(A + (size_t)m * lda + k0);
 #pragma unroll
-	for (int tb = 0; tb < NTB; tb++) wsrc[tb] = reinterpret_cast<const i32x4 *>(Wg + (size_t)(tile0 + tb) * slab) + tid;
-	const half8 *asrc = reinterpret_cast<const half8 *>(Apack + (size_t)mtile * (size_t)(K >> 4) * 1024) + lane;
-
-	i32x4 braw[NTB][2];
-	half8 acur[8], anext[8];  // [k16 step within the stage][hi, lo]
-	auto load_stage = [&](int st, half8 *areg) {
+		for (int q = 0; q < 4; q++) {
+			const f32x4 a = src[q];
+			unsigned d0 = 0, d1 = 0, d2 = 0;
 #pragma unroll
-		for (int tb = 0; tb < NTB; tb++) {
-			braw[tb][0] = wsrc[tb][(size_t)st * (KSTAGE / 4) * 32];
-			braw[tb][1] = wsrc[tb][(size_t)st * (KSTAGE / 4) * 32 + 256];
-		}
-#pragma unroll
-		for (int s = 0; s < 4; s++) {
-			areg[2 * s] = asrc[(size_t)(st * 4 + s) * 128];
-			areg[2 * s + 1] = asrc[(size_t)(st * 4 + s) * 128 + 64];
-		}
-	};
-	auto store_b = [&](int buf) {
-#pragma unroll
-		for (int tb = 0; tb < NTB; tb++) {
-#pragma unroll
-			for (int q = 0; q < 2; q++) {
-				const int p = tid + 256 * q, kgl = p >> 5, cl = p & 31;
-				const int d[4] = {braw[tb][q].x, braw[tb][q].y, braw[tb][q].z, braw[tb][q].w};
-#pragma unroll
-				for (int j = 0; j < 4; j++) {
-					half4 h;
-					h[0] = (_Float16)(int8_t)(d[j]);
-					h[1] = (_Float16)(int8_t)(d[j] >> 8);
-					h[2] = (_Float16)(int8_t)(d[j] >> 16);
-					h[3] = (_Float16)(int8_t)(d[j] >> 24);
-					*reinterpret_cast<half4 *>(&Bs[buf][tb][kgl >> 1][4 * cl + j][4 * (kgl & 1)]) = h;
-				}
+			for (int i = 0; i < 4; i++) {
+				const int xi = (int)rintf(a[i] * s);
+				const int a0 = (xi << 24) >> 24;
+				const int r1 = (xi - a0) >> 8;
+				const int a1 = (r1 << 24) >> 24;
+				const int a2 = (r1 - a1) >> 8;
+				d0 |= (unsigned)(a0 & 255) << (8 * i);
+				d1 |= (unsigned)(a1 & 255) << (8 * i);
+				d2 |= (unsigned)(a2 & 255) << (8 * i);
 			}
+			pl[0][q] = (int)d0;
+			pl[1][q] = (int)d1;
+			pl[2][q] = (int)d2;
 		}
+	}
+	const int kb = k0 >> 5, hb = (k0 >> 4) & 1;
+	i32x4 *dst = reinterpret_cast<i32x4 *>(Apack) + ((size_t)mtile * (size_t)(K >> 5) + kb) * 3 * 64 + (r + 32 * hb);
+#pragma unroll
+	for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
+}
+
+// GEGLU: fused up|gate tile with gelu(gate) * up; LUTLDS: the GeLU table is small enough to be staged in LDS
+template <bool GEGLU, bool LUTLDS>
+__global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
+                                                      const float *scales, int M, int K, int ldc, const float *lut, float gmin,
+                                                      float geps, float ginv, int lut_size) {
+	// B operands of one stage: [k / 16][column][16 bytes], double buffered
+	__shared__ __attribute__((aligned(16))) i32x4 Bs[2][KSTAGE / 16][TG_CT];
+	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
+
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hb = lane >> 5;
+	// Workgroups are handed to the 8 XCDs (each with its own L2) round-robin in launch order.  Give every
+	// XCD a contiguous share of the (row block, column tile) grid, row blocks varying fastest, so that the
+	// workgroups resident on one XCD at a time share a few activation slabs and weight tiles in its L2.
+	int tile, mblock;
+	{
+		const int ntiles = (int)gridDim.x, mblocks = (int)gridDim.y, total = ntiles * mblocks;
+		const int lin = (int)blockIdx.x + ntiles * (int)blockIdx.y;
+		if ((total & 7) == 0) {
+			const int chunk = total >> 3, v = (lin & 7) * chunk + (lin >> 3);
+			if ((mblocks & 7) == 0) {
+				const int mbx = mblocks >> 3, xcd = lin & 7, i = v - xcd * chunk;
+				mblock = xcd * mbx + i % mbx;
+				tile = i / mbx;
+			} else {
+				mblock = v % mblocks;
+				tile = v / mblocks;
+			}
+		} else {
+			tile = (int)blockIdx.x;
+			mblock = (int)blockIdx.y;
+		}
+	}
+	const int mtile = mblock * 4 + w;
+	const int nstage = K / KSTAGE;
+	if (GEGLU && LUTLDS) {  // the table is read once per output element; visible after the first barrier
+		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
+	}
+
+	// a stage of B is 8 KB contiguous: 512 pieces of 16 bytes, two per thread
+	const i32x4 *bsrc = reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + tid;
+	const i32x4 *asrc = reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane;
+	i32x4 *bdst = &Bs[0][0][0] + tid;
+
+	// Software pipeline, all through registers (one wave per SIMD: nothing else hides latency):
+	//   A of stage s is requested 3 stages before its use and lives in areg[s % 4];
+	//   B of stage s is requested 4 stages ahead into breg[s % 4], written to LDS buffer s % 2 during
+	//   stage s - 1 and read during stage s; one barrier per stage.
+	i32x4 areg[4][6];  // [ring slot][k step within the stage * 3 + plane]
+	i32x4 breg[4][2];
+	auto load_b = [&](int st, i32x4 *r) {
+		r[0] = bsrc[(size_t)st * 512];
+		r[1] = bsrc[(size_t)st * 512 + 256];
+	};
+	auto store_b = [&](int buf, const i32x4 *r) {
+		bdst[buf * 512] = r[0];
+		bdst[buf * 512 + 256] = r[1];
+	};
+	auto load_a = [&](int st, i32x4 *r) {
+#pragma unroll
+		for (int i = 0; i < 6; i++) r[i] = asrc[(size_t)(st * 6 + i) * 64];
 	};
 
-	f32x16 acc[NTB][4];
+	i32x16 acc[3][4];
 #pragma unroll
-	for (int tb = 0; tb < NTB; tb++)
+	for (int p = 0; p < 3; p++)
 #pragma unroll
 		for (int j = 0; j < 4; j++)
 #pragma unroll
-			for (int i = 0; i < 16; i++) acc[tb][j][i] = 0.0f;
+			for (int i = 0; i < 16; i++) acc[p][j][i] = 0;
 
-	load_stage(0, acur);
-	for (int st = 0; st < nstage; st++) {
-		const int buf = st & 1;
-		store_b(buf);
-		__syncthreads();
-		if (st + 1 < nstage) load_stage(st + 1, anext);
+	auto compute = [&](int buf, const i32x4 *a) {
 #pragma unroll
-		for (int s = 0; s < 4; s++) {
+		for (int ks = 0; ks < 2; ks++) {
+			i32x4 b[4];
 #pragma unroll
-			for (int tb = 0; tb < NTB; tb++) {
+			for (int j = 0; j < 4; j++) b[j] = Bs[buf][2 * ks + hb][32 * j + c];
 #pragma unroll
-				for (int j = 0; j < 4; j++) {
-					const half8 b = *reinterpret_cast<const half8 *>(&Bs[buf][tb][2 * s + (lane >> 5)][32 * j + (lane & 31)][0]);
-					acc[tb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(acur[2 * s], b, acc[tb][j], 0, 0, 0);
-					acc[tb][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(acur[2 * s + 1], b, acc[tb][j], 0, 0, 0);
-				}
-			}
+			for (int p = 0; p < 3; p++)
+#pragma unroll
+				for (int j = 0; j < 4; j++) acc[p][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[3 * ks + p], b[j], acc[p][j], 0, 0, 0);
 		}
-#pragma unroll
-		for (int i = 0; i < 8; i++) acur[i] = anext[i];
+	};
+
+	// Every stage issues its loads unconditionally (stage indices are clamped at the end of K, the
+	// surplus loads land in ring slots nobody reads again): with loads under branches the compiler can no
+	// longer count how many are in flight and falls back to waiting for all of them.
+	const int last = nstage - 1;
+	auto clamp = [&](int st) { return st < last ? st : last; };
+	auto stage = [&](int st, auto uc) {
+		constexpr int u = decltype(uc)::value;
+		load_a(clamp(st + 3), areg[(u + 3) & 3]);
+		load_b(clamp(st + 4), breg[u]);
+		// LDS buffer (st+1) % 2 was last read in stage st-1, which every wave has left
+		store_b((u + 1) & 1, breg[(u + 1) & 3]);
+		compute(u & 1, areg[u]);
+		tg_lds_barrier();
+	};
+	load_b(0, breg[0]);
+	load_a(0, areg[0]);
+	load_b(clamp(1), breg[1]);
+	load_a(clamp(1), areg[1]);
+	load_b(clamp(2), breg[2]);
+	load_a(clamp(2), areg[2]);
+	load_b(clamp(3), breg[3]);
+	store_b(0, breg[0]);
+	tg_lds_barrier();
+	int st0 = 0;
+	for (; st0 + 4 <= nstage; st0 += 4) {
+		stage(st0, std::integral_constant<int, 0>{});
+		stage(st0 + 1, std::integral_constant<int, 1>{});
+		stage(st0 + 2, std::integral_constant<int, 2>{});
+		stage(st0 + 3, std::integral_constant<int, 3>{});
+	}
+	if (nstage & 2) {  // nstage is even (K is a multiple of 128)
+		stage(st0, std::integral_constant<int, 0>{});
+		stage(st0 + 1, std::integral_constant<int, 1>{});
 	}
 
-	// epilogue: accumulator element i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32 of the 32x32 tile
+	// epilogue: accumulator element i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32 of the 32x32 tile.
+	// All factors are fetched up front (rowinv is padded to whole row tiles) so that no load sits between
+	// the conversions and the stores.
 	const int mbase = mtile * 32;
+	f32x4 rs4[4];
 #pragma unroll
-	for (int j = 0; j < 4; j++) {
-		const int n = 32 * j + (lane & 31);
+	for (int q = 0; q < 4; q++) rs4[q] = *reinterpret_cast<const f32x4 *>(rowinv + mbase + 8 * q + 4 * hb);
+	float sc[4];
 #pragma unroll
-		for (int i = 0; i < 16; i++) {
-			const int m = mbase + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+	for (int j = 0; j < 4; j++) sc[j] = scales[tile * TG_CT + 32 * j + c];
+	auto value = [&](int j, int i) {
+		const float v = fmaf((float)acc[2][j][i], 65536.0f, fmaf((float)acc[1][j][i], 256.0f, (float)acc[0][j][i]));
+		return (v * rs4[i >> 2][i & 3]) * sc[j];
+	};
+#pragma unroll
+	for (int i = 0; i < 16; i++) {
+		const int m = mbase + 8 * (i >> 2) + 4 * hb + (i & 3);
+		if (GEGLU) {
+			float o[2];
+#pragma unroll
+			for (int j = 0; j < 2; j++) {
+				const float gate = value(j + 2, i);
+				o[j] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) * value(j, i);
+			}
 			if (m < M) {
-				const float rs = rowscale[m];
-				if (NTB == 1) {
-					C[(size_t)m * ldc + (size_t)tile0 * TG_CT + n] = (acc[0][j][i] * rs) * scales[tile0 * TG_CT + n];
-				} else {
-					const float up = (acc[0][j][i] * rs) * scales[tile0 * TG_CT + n];
-					const float gate = (acc[NTB - 1][j][i] * rs) * scales[(tile0 + 1) * TG_CT + n];
-					C[(size_t)m * ldc + (size_t)blockIdx.x * TG_CT + n] = gelu_lut(gate, lut, gmin, geps, lut_size) * up;
-				}
+#pragma unroll
+				for (int j = 0; j < 2; j++) C[(size_t)m * ldc + (size_t)tile * (TG_CT / 2) + 32 * j + c] = o[j];
+			}
+		} else {
+			float o[4];
+#pragma unroll
+			for (int j = 0; j < 4; j++) o[j] = value(j, i);
+			if (m < M) {
+#pragma unroll
+				for (int j = 0; j < 4; j++) C[(size_t)m * ldc + (size_t)tile * TG_CT + 32 * j + c] = o[j];
 			}
 		}
 	}
@@ -202,22 +273,33 @@ __global__ __launch_bounds__(GNT) void gemm_mfma_kernel(float *C, const _Float16
 
 }  // namespace
 
-size_t tg_gemm_mfma_apack_halfs(int M, int K) { return (size_t)((M + 127) / 128) * 128 * (size_t)K * 2; }
+// scratch sizes for M rows of K: digit planes (bytes) and row factors (floats, two arrays of this length)
+size_t tg_gemm_mfma_apack_bytes(int M, int K) { return (size_t)((M + 127) / 128) * 128 * (size_t)K * 3; }
+size_t tg_gemm_mfma_rows(int M) { return (size_t)((M + 127) / 128) * 128; }
 
-// A [M][lda] fp32 -> packed halves + row scales; apack must hold tg_gemm_mfma_apack_halfs(M, K), rowscale ceil(M/128)*128 floats
-void tg_launch_split_pack(const float *A, int lda, int M, int K, _Float16 *apack, float *rowscale, hipStream_t s) {
-	const int mtiles = ((M + 127) / 128) * 4;
-	hipLaunchKernelGGL(split_pack_rows_kernel, dim3((unsigned)mtiles), dim3(GNT), 0, s, A, lda, M, K, apack, rowscale);
+// A [M][lda] fp32 -> digit planes + row factors; rowfac holds 2 * tg_gemm_mfma_rows(M) floats (multipliers, then inverses)
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, hipStream_t s) {
+	const int Mpad = (int)tg_gemm_mfma_rows(M);
+	hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)(Mpad / 4)), dim3(GNT), 0, s, A, lda, M, K, rowfac, rowfac + Mpad, Mpad);
+	hipLaunchKernelGGL(quant_pack_kernel, dim3((unsigned)(Mpad / 32), (unsigned)(K / 128)), dim3(GNT), 0, s, A, lda, M, K, rowfac, apack);
 }
 
-void tg_launch_gemm_mfma(float *C, const _Float16 *apack, const float *rowscale, const int8_t *Wg, const float *scales, int M, int K,
+// ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns
+void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, hipStream_t s) {
 	const unsigned mblocks = (unsigned)((M + 127) / 128);
-	if (epi == TG_EPI_GEGLU) {
-		hipLaunchKernelGGL(gemm_mfma_kernel<2>, dim3((unsigned)(ntiles / 2), mblocks), dim3(GNT), 0, s, C, apack, rowscale, Wg, scales, M,
-		                   K, (ntiles / 2) * TG_CT, lut, gmin, geps, lut_size);
+	const float *rowinv = rowfac + tg_gemm_mfma_rows(M);
+	const dim3 grid((unsigned)ntiles, mblocks), block(GNT);
+	int e = 0;
+	const float ginv = (epi == TG_EPI_GEGLU && geps > 0.0f && frexpf(geps, &e) == 0.5f && e > -100 && e < 100) ? 1.0f / geps : 0.0f;
+	if (epi == TG_EPI_GEGLU && lut_size <= LUT_LDS_MAX) {
+		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
+		                   gmin, geps, ginv, lut_size);
+	} else if (epi == TG_EPI_GEGLU) {
+		hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
+		                   gmin, geps, ginv, lut_size);
 	} else {
-		hipLaunchKernelGGL(gemm_mfma_kernel<1>, dim3((unsigned)ntiles, mblocks), dim3(GNT), 0, s, C, apack, rowscale, Wg, scales, M, K,
-		                   ntiles * TG_CT, lut, gmin, geps, lut_size);
+		hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * TG_CT, lut, gmin,
+		                   geps, ginv, lut_size);
 	}
 }

@@ -144,17 +144,23 @@ void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float
                                  hipStream_t s);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
                             int ldo, int is_sw, int window, hipStream_t s);
-// C[m][N] = (A[m][K] . W) * scales, W packed; epi GEGLU writes C[m][N/2]
-void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int epi,
+// exact-order GEMM on the GEMV tiling (ntiles tiles of Ct columns): C[m][N] = (A[m][K] . W) * scales; epi GEGLU writes C[m][N/2]
+void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
 
 void tg_launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
 
-// MFMA prefill GEMM (tg_gemm_mfma.hip): A is first split into scaled fp16 hi/lo halves in operand order
-size_t tg_gemm_mfma_apack_halfs(int M, int K);
-void tg_launch_split_pack(const float *A, int lda, int M, int K, _Float16 *apack, float *rowscale, hipStream_t s);
-void tg_launch_gemm_mfma(float *C, const _Float16 *apack, const float *rowscale, const int8_t *Wg, const float *scales, int M, int K,
+// int8 MFMA prefill GEMM (tg_gemm_mfma.hip): A is first quantised per row into three int8 digit planes in operand order
+size_t tg_gemm_mfma_apack_bytes(int M, int K);
+size_t tg_gemm_mfma_rows(int M);  // rowfac scratch holds twice this many floats
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, hipStream_t s);
+void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load of the wave (its fence covers all address spaces), which would drain a software pipeline
+// of prefetched tiles at every stage; here loads issued earlier stay in flight across the barrier.
+__device__ __forceinline__ void tg_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // ---- errors -----------------------------------------------------------------------------------
 int tg_fail(int code, const std::string &msg);

@@ -77,16 +77,25 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 	}
 }
 
-// 64 rows x 128 columns per workgroup; thread (ty = tid/32, tx = tid%32) owns rows ty*8..+7 and
-// columns tx*4..+3 of the tile.  For the fused up|gate matrix (epi GEGLU) the workgroup walks the
-// tile pair (2t, 2t+1) and writes gelu(gate) * up.
+// Exact-order GEMM: every element is one fp32 fused chain over k = 0..K-1 like the reference's
+// (linalg.hpp:210-308), so results are bit-identical to it.  64 rows x 128 output columns per workgroup;
+// thread (ty = tid/32, tx = tid%32) owns rows ty*8..+7 and columns tx*4..+3.  Weights are read from the
+// GEMV tiling (tiles of Ct columns, [K/4][Ct][4]); for the fused up|gate matrix (epi GEGLU) a tile holds
+// Ct/2 up columns then the same Ct/2 gate columns and the workgroup writes gelu(gate) * up.
 template <int EPI>
 __global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *A, const int8_t *Wp, const float *scales, int m,
-                                                         int K, int ntiles, const float *lut, float gmin, float geps, int lut_size) {
+                                                         int K, int Ct, int ldc, const float *lut, float gmin, float geps,
+                                                         int lut_size) {
 	constexpr int NTILE = (EPI == TG_EPI_GEGLU) ? 2 : 1;
 	const int tid = threadIdx.x, tx = tid & 31, ty = tid >> 5;
 	const int row0 = blockIdx.y * 64 + ty * 8;
 	const int kgs = K >> 2;
+	const int n0 = blockIdx.x * 128 + tx * 4;  // first output column of this thread
+	const int cw = (EPI == TG_EPI_GEGLU) ? Ct / 2 : Ct;
+	const int tile = n0 / cw, cc = n0 % cw;
+	int vcol[NTILE];  // virtual column (tile order) of the thread's first column, per operand
+	vcol[0] = tile * Ct + cc;
+	if (NTILE == 2) vcol[NTILE - 1] = tile * Ct + cw + cc;
 	float acc[NTILE][8][4];
 #pragma unroll
 	for (int t = 0; t < NTILE; t++)
@@ -97,6 +106,11 @@ __global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *
 	const float *arow[8];
 #pragma unroll
 	for (int r = 0; r < 8; r++) arow[r] = A + (size_t)((row0 + r < m) ? row0 + r : m - 1) * K;
+	const uint4 *wsrc[NTILE];
+#pragma unroll
+	for (int t = 0; t < NTILE; t++)
+		wsrc[t] = reinterpret_cast<const uint4 *>(Wp + ((size_t)tile * kgs * Ct + (size_t)(vcol[t] - tile * Ct)) * 4);
+	const size_t kstep = (size_t)Ct / 4;  // 16-byte pieces per k group
 
 	for (int kg = 0; kg < kgs; kg++) {
 		float4 av[8];
@@ -104,8 +118,7 @@ __global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *
 		for (int r = 0; r < 8; r++) av[r] = *reinterpret_cast<const float4 *>(arow[r] + 4 * kg);
 #pragma unroll
 		for (int t = 0; t < NTILE; t++) {
-			const int tile = blockIdx.x * NTILE + t;
-			const uint4 wv = *(reinterpret_cast<const uint4 *>(Wp) + ((size_t)tile * kgs + kg) * (TG_CT / 4) + tx);
+			const uint4 wv = wsrc[t][(size_t)kg * kstep];
 			const int d[4] = {(int)wv.x, (int)wv.y, (int)wv.z, (int)wv.w};
 #pragma unroll
 			for (int c = 0; c < 4; c++) {
@@ -122,27 +135,23 @@ __global__ __launch_bounds__(RNT) void gemm_exact_kernel(float *C, const float *
 			}
 		}
 	}
-	const int N = ntiles * TG_CT;
 #pragma unroll
 	for (int r = 0; r < 8; r++) {
 		if (row0 + r >= m) continue;
+		float4 o;
+		float *op = &o.x;
 		if (EPI == TG_EPI_GEGLU) {
-			const int cu = (blockIdx.x * 2) * TG_CT + tx * 4, cg = cu + TG_CT;
-			float4 o;
-			float *op = &o.x;
 #pragma unroll
 			for (int c = 0; c < 4; c++) {
-				const float up = acc[0][r][c] * scales[cu + c];
-				const float gate = acc[NTILE - 1][r][c] * scales[cg + c];
+				const float up = acc[0][r][c] * scales[vcol[0] + c];
+				const float gate = acc[NTILE - 1][r][c] * scales[vcol[NTILE - 1] + c];
 				op[c] = gelu_lut(gate, lut, gmin, geps, lut_size) * up;
 			}
-			*reinterpret_cast<float4 *>(C + (size_t)(row0 + r) * (N / 2) + blockIdx.x * TG_CT + tx * 4) = o;
 		} else {
-			const int c0 = blockIdx.x * TG_CT + tx * 4;
-			float4 o = make_float4(acc[0][r][0] * scales[c0], acc[0][r][1] * scales[c0 + 1], acc[0][r][2] * scales[c0 + 2],
-			                       acc[0][r][3] * scales[c0 + 3]);
-			*reinterpret_cast<float4 *>(C + (size_t)(row0 + r) * N + c0) = o;
+#pragma unroll
+			for (int c = 0; c < 4; c++) op[c] = acc[0][r][c] * scales[vcol[0] + c];
 		}
+		*reinterpret_cast<float4 *>(C + (size_t)(row0 + r) * ldc + n0) = o;
 	}
 }
 
@@ -169,14 +178,15 @@ void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const 
 	hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, out, in, w_pre, w_post, resid, resid_out, dim);
 }
 
-void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int epi,
+// Wp/scales: GEMV tiling of the matrix (ntiles tiles of Ct columns); C gets ntiles * Ct columns, or half of that for GEGLU
+void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s) {
 	dim3 block(RNT);
+	const int ncols = (epi == TG_EPI_GEGLU) ? ntiles * Ct / 2 : ntiles * Ct;
+	dim3 grid((unsigned)(ncols / 128), (unsigned)((m + 63) / 64));
 	if (epi == TG_EPI_GEGLU) {
-		dim3 grid((unsigned)(ntiles / 2), (unsigned)((m + 63) / 64));
-		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_GEGLU>, grid, block, 0, s, C, A, Wp, scales, m, K, ntiles, lut, gmin, geps, lut_size);
+		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_GEGLU>, grid, block, 0, s, C, A, Wp, scales, m, K, Ct, ncols, lut, gmin, geps, lut_size);
 	} else {
-		dim3 grid((unsigned)ntiles, (unsigned)((m + 63) / 64));
-		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_STORE>, grid, block, 0, s, C, A, Wp, scales, m, K, ntiles, lut, gmin, geps, lut_size);
+		hipLaunchKernelGGL(gemm_exact_kernel<TG_EPI_STORE>, grid, block, 0, s, C, A, Wp, scales, m, K, Ct, ncols, lut, gmin, geps, lut_size);
 	}
 }
