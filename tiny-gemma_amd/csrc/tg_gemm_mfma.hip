@@ -15,8 +15,11 @@
 //     column scale.
 //
 // Nothing in the inner loop converts anything: weight tiles go global -> LDS as raw bytes and are read
-// back as MFMA B operands, digit planes are stored in A-operand order by the quantising pre-pass and are
+// back as MFMA operands, digit planes are stored in operand order by the quantising pre-pass and are
 // fetched straight from global memory with 16-byte loads (a wave owns its 32 rows: nothing to share).
+// The weight fragment is passed as the first MFMA operand and the activation fragment as the second (the
+// two have the same register layout), which leaves C transposed in the accumulators: each lane then owns
+// runs of four consecutive columns of one output row and stores them 16 bytes at a time.
 //
 // Layouts
 //   weights (built at load time): [tile of 128 columns][K/16][128 columns][16 consecutive k]
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 	// Software pipeline, all through registers (one wave per SIMD: nothing else hides latency):
 	//   A of stage s is requested 3 stages before its use and lives in areg[s % 4];
 	//   B of stage s is requested 4 stages ahead into breg[s % 4], written to LDS buffer s % 2 during
-	//   stage s - 1 and read during stage s; one barrier per stage.
+	//   stage s - 1 and read from there (first k step: during stage s - 1, after its barrier); one barrier per stage.
 	i32x4 areg[4][6];  // [ring slot][k step within the stage * 3 + plane]
 	i32x4 breg[4][2];
 	auto load_b = [&](int st, i32x4 *r) {
@@ -183,18 +186,18 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 #pragma unroll
 			for (int i = 0; i < 16; i++) acc[p][j][i] = 0;
 
-	auto compute = [&](int buf, const i32x4 *a) {
+	// B fragments of one k step (32 rows of K): bfrag[j] = columns 32 j .. 32 j + 31
+	auto read_b = [&](int buf, int ks, i32x4 *bfrag) {
 #pragma unroll
-		for (int ks = 0; ks < 2; ks++) {
-			i32x4 b[4];
-#pragma unroll
-			for (int j = 0; j < 4; j++) b[j] = Bs[buf][2 * ks + hb][32 * j + c];
-#pragma unroll
-			for (int p = 0; p < 3; p++)
-#pragma unroll
-				for (int j = 0; j < 4; j++) acc[p][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[3 * ks + p], b[j], acc[p][j], 0, 0, 0);
-		}
+		for (int j = 0; j < 4; j++) bfrag[j] = Bs[buf][2 * ks + hb][32 * j + c];
 	};
+	auto mfma_step = [&](const i32x4 *a, const i32x4 *bfrag) {
+#pragma unroll
+		for (int p = 0; p < 3; p++)
+#pragma unroll
+			for (int j = 0; j < 4; j++) acc[p][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfrag[j], a[p], acc[p][j], 0, 0, 0);
+	};
+	i32x4 b0[4], b1[4];  // fragments of the stage's first / second k step; b0 is fetched one stage ahead
 
 	// Every stage issues its loads unconditionally (stage indices are clamped at the end of K, the
 	// surplus loads land in ring slots nobody reads again): with loads under branches the compiler can no
@@ -205,10 +208,15 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 		constexpr int u = decltype(uc)::value;
 		load_a(clamp(st + 3), areg[(u + 3) & 3]);
 		load_b(clamp(st + 4), breg[u]);
-		// LDS buffer (st+1) % 2 was last read in stage st-1, which every wave has left
+		// LDS buffer (st+1) % 2 was last read before the previous barrier
 		store_b((u + 1) & 1, breg[(u + 1) & 3]);
-		compute(u & 1, areg[u]);
-		tg_lds_barrier();
+		// The single barrier of a stage sits between its two k steps: every LDS read is issued one MFMA
+		// block before its use, and the matrix cores idle only for the skew between the waves.
+		read_b(u & 1, 1, b1);
+		mfma_step(areg[u], b0);
+		tg_lds_barrier();  // all of B(st+1) is in LDS; all reads of buffer st % 2 have completed
+		read_b((u + 1) & 1, 0, b0);
+		mfma_step(areg[u] + 3, b1);
 	};
 	load_b(0, breg[0]);
 	load_a(0, areg[0]);
@@ -219,6 +227,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 	load_b(clamp(3), breg[3]);
 	store_b(0, breg[0]);
 	tg_lds_barrier();
+	read_b(0, 0, b0);
 	int st0 = 0;
 	for (; st0 + 4 <= nstage; st0 += 4) {
 		stage(st0, std::integral_constant<int, 0>{});
@@ -231,41 +240,39 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 		stage(st0 + 1, std::integral_constant<int, 1>{});
 	}
 
-	// epilogue: accumulator element i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32 of the 32x32 tile.
-	// All factors are fetched up front (rowinv is padded to whole row tiles) so that no load sits between
-	// the conversions and the stores.
-	const int mbase = mtile * 32;
-	f32x4 rs4[4];
+	// epilogue.  The weight fragment is the first MFMA operand, so the accumulators hold the tile transposed:
+	// element i of lane l is output column 8*(i/4) + 4*(l/32) + i%4 and output row l%32 of the 32x32 tile,
+	// i.e. four consecutive floats of one row of C per group of four elements: 16-byte stores.
+	const int m = mtile * 32 + c;
+	const float rs = rowinv[m];  // rowinv is padded to whole row tiles
+	f32x4 sc[4][4];              // column scales of [column tile j][group q]
 #pragma unroll
-	for (int q = 0; q < 4; q++) rs4[q] = *reinterpret_cast<const f32x4 *>(rowinv + mbase + 8 * q + 4 * hb);
-	float sc[4];
+	for (int j = 0; j < 4; j++)
 #pragma unroll
-	for (int j = 0; j < 4; j++) sc[j] = scales[tile * TG_CT + 32 * j + c];
+		for (int q = 0; q < 4; q++) sc[j][q] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * j + 8 * q + 4 * hb);
 	auto value = [&](int j, int i) {
 		const float v = fmaf((float)acc[2][j][i], 65536.0f, fmaf((float)acc[1][j][i], 256.0f, (float)acc[0][j][i]));
-		return (v * rs4[i >> 2][i & 3]) * sc[j];
+		return (v * rs) * sc[j][i >> 2][i & 3];
 	};
+	if (m < M) {
+		float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 4 * hb;
 #pragma unroll
-	for (int i = 0; i < 16; i++) {
-		const int m = mbase + 8 * (i >> 2) + 4 * hb + (i & 3);
-		if (GEGLU) {
-			float o[2];
+		for (int j = 0; j < (GEGLU ? 2 : 4); j++) {
 #pragma unroll
-			for (int j = 0; j < 2; j++) {
-				const float gate = value(j + 2, i);
-				o[j] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) * value(j, i);
-			}
-			if (m < M) {
+			for (int q = 0; q < 4; q++) {
+				f32x4 o;
 #pragma unroll
-				for (int j = 0; j < 2; j++) C[(size_t)m * ldc + (size_t)tile * (TG_CT / 2) + 32 * j + c] = o[j];
-			}
-		} else {
-			float o[4];
-#pragma unroll
-			for (int j = 0; j < 4; j++) o[j] = value(j, i);
-			if (m < M) {
-#pragma unroll
-				for (int j = 0; j < 4; j++) C[(size_t)m * ldc + (size_t)tile * TG_CT + 32 * j + c] = o[j];
+				for (int e = 0; e < 4; e++) {
+					const int i = 4 * q + e;
+					if (GEGLU) {
+						const float gate = value(j + 2, i);
+						o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
+						       value(j, i);
+					} else {
+						o[e] = value(j, i);
+					}
+				}
+				*reinterpret_cast<f32x4 *>(crow + 32 * j + 8 * q) = o;
 			}
 		}
 	}
