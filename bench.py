@@ -10,6 +10,9 @@ PCIe inside it (each step feeds the device-side argmax of the previous one).
 Prints one JSON line.  `roofline` is for the dominant kernel of a step, the LM-head GEMV
 (tg_gemv_lmhead_argmax: 1152 x 262144 int8 + scales + x + logits = 304,091,648 algorithmic
 bytes per launch), timed with HIP events on the library's stream during real decode steps.
+Reported beside it: `gemv_lmhead_shape` (the plain GEMV entry point tg_qgemv_dev on the same matrix,
+launched back to back) and `prefill.long_prompt` (a 4096-token prefill of the same model: the
+matrix-matrix path on the int8 matrix cores).
 `cpu_baseline` times the reference's single-threaded AVX2 path (oracle/_ref, built from the
 reference's own sources) — or, where that library is absent, the scalar C restatement — on
 this machine's host cores over a bounded sample of the same workload.
@@ -30,7 +33,7 @@ import __graft_entry__ as ge  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one tg_gemv_lmhead_argmax launch from two `rocprofv3 --pmc` runs (FETCH_SIZE x 1.9998 +
 # WRITE_SIZE x 1.0000, both in KiB, scaled on a 256 MiB copy kernel): profiles/decode_1B_hbm_traffic.md
-LMHEAD_TRAFFIC_BYTES = {"1B": 304_438_104}
+LMHEAD_TRAFFIC_BYTES = {"1B": 304_549_348}
 
 MODELS = {
     # name: (prompt tokens, decode bytes of weights+scales per token, LM-head GEMV algorithmic bytes)

@@ -125,7 +125,8 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 int tg_decode_enqueue(tg_session *s, int n_steps);
 /* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
 int tg_set_graphs(int enable);
-/* prefill GEMM: 1 (default) = MFMA with fp16 hi/lo split activations (fp32-rounding-level accuracy),
+/* prefill GEMM: 1 (default) = int8 matrix cores on three int8 digit planes of the row-scaled activations
+ * (exact integer accumulation, fp32-rounding-level accuracy),
  * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */
 int tg_set_gemm_mode(int mfma);
 /* tuning knob: a GEMV launch uses at most n workgroups, which then loop over column tiles (0: one per tile) */
@@ -133,6 +134,10 @@ int tg_set_gemv_max_blocks(int n);
 /* tuning knob: extra workgroups per decode launch that pull the NEXT launch's weights out of HBM into
  * the caches while the current launch is latency bound (multiple of 8; 0 = off).  A hint only. */
 int tg_set_prefetch_blocks(int n);
+/* tuning knob: which launch carries which prefetch.  0 (default): the q|k|v launch touches the o matrix, attention
+ * the up|gate matrix, o the down matrix, up|gate the next layer's q|k|v.  1: an alternative kept for measurement
+ * (q|k|v touches o and up|gate, attention touches down). */
+int tg_set_prefetch_plan(int plan);
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
 
 /* Kernel classes of one decode step, in launch order per layer; the head runs once per step. */

@@ -104,8 +104,8 @@ def test_qgemm_exact_mode_bit_exact(tg, oracle, golden, exact_gemm, name):
 
 @pytest.mark.parametrize("name", list(gi.GEMM_CASES))
 def test_qgemm_mfma(tg, oracle, golden, name):
-    """Default prefill GEMM: fp16 MFMA on power-of-two scaled hi/lo split activations.  22 mantissa bits of
-    the activations and exact int8 -> fp16 weights: norm-relative error at the fp32-rounding level (<= 3e-6)."""
+    """Default prefill GEMM: int8 matrix cores on three int8 digit planes of the power-of-two scaled activations
+    (22 bits + sign of the row maximum), exact int32 sums: norm-relative error at the fp32-rounding level (<= 3e-6)."""
     m, i, n, seed = gi.GEMM_CASES[name]
     A, W, s = gi.gemm_inputs(m, i, n, seed)
     Cm = np.full((m, n), np.nan, np.float32)
@@ -118,7 +118,7 @@ def test_qgemm_mfma(tg, oracle, golden, name):
 
 
 def test_qgemm_mfma_exact_cases(tg):
-    """Integer activations and power-of-two scales are exact through the hi/lo split (lo = 0);
+    """Integer activations and power-of-two scales are exact through the digit planes;
     rows of very different magnitude (1e-6 ... 1e4, and an all-zero row) keep their own scaling."""
     rng = np.random.default_rng(7)
     A = rng.integers(-8, 9, (70, 1152)).astype(np.float32)
@@ -137,6 +137,43 @@ def test_qgemm_mfma_exact_cases(tg):
     ref = (A.astype(np.float64) @ W.astype(np.float64)) * s.astype(np.float64)
     for r in range(9):
         assert normrel(Cm[r], ref[r]) < 3e-6
+
+
+def _digit_plane_closed_form(A, W, s):
+    """The int8-MFMA GEMM's documented arithmetic, restated with numpy integers: per-row power-of-two scaling into
+    [2^21, 2^22), round to nearest even, three signed base-256 digits, exact integer contractions, fp32 recombination
+    (two fused multiply-adds), inverse row factor, column scale."""
+    A = A.astype(np.float32)
+    amax = np.abs(A).max(axis=1)
+    _, e = np.frexp(amax)  # amax = f * 2^e, f in [0.5, 1)
+    e = np.where(amax > 0, e, 22)
+    mul = np.ldexp(np.float32(1.0), 22 - e).astype(np.float32)
+    inv = np.ldexp(np.float32(1.0), e - 22).astype(np.float32)
+    xi = np.rint(A * mul[:, None]).astype(np.int64)
+    a0 = ((xi + 128) & 255) - 128
+    r1 = (xi - a0) >> 8
+    a1 = ((r1 + 128) & 255) - 128
+    a2 = (r1 - a1) >> 8
+    assert np.abs(a2).max() <= 127 and np.array_equal(65536 * a2 + 256 * a1 + a0, xi)
+    Wi = W.astype(np.int64)
+    s0, s1, s2 = (a @ Wi for a in (a0, a1, a2))
+    f32 = lambda z: z.astype(np.float32)
+    inner = f32(f32(s1).astype(np.float64) * 256.0 + f32(s0).astype(np.float64))   # one rounding: fused multiply-add
+    v = f32(f32(s2).astype(np.float64) * 65536.0 + inner.astype(np.float64))
+    return (v * inv[:, None]) * s[None, :].astype(np.float32)
+
+
+@pytest.mark.parametrize("shape", [(70, 1152, 1024, 11), (33, 6912, 1152, 12), (200, 1152, 6912, 13), (5, 256, 640, 14)])
+def test_qgemm_mfma_equals_digit_plane_closed_form(tg, shape):
+    """Bit-for-bit: a dropped or mis-weighted digit plane, a wrong rounding of the activations or a wrong row factor
+    cannot hide inside a tolerance here."""
+    m, i, n, seed = shape
+    A, W, s = gi.gemm_inputs(m, i, n, seed)
+    A[0] *= np.float32(1e-5)
+    A[m - 1] *= np.float32(3e4)
+    Cm = np.empty((m, n), np.float32)
+    tg.launch_qgemm(Cm, A, W, s, m, i, n)
+    assert np.array_equal(Cm, _digit_plane_closed_form(A, W, s))
 
 
 def test_device_resident_gemv_matches_host_entry(tg, oracle):

@@ -59,42 +59,6 @@ __device__ __forceinline__ void norm_rope_head(const float *src, const float *w,
 	out[3] = fmaf(c1, x[3], x[1] * s1) * mul;
 }
 
-// scores of keys [k0, k0+n) against the 4 query heads in qs (already scaled by 1/sqrt(hd)).
-// 16 lanes share one key row (coalesced 256-byte pieces); sc[h][j-k0] receives q_h . k_j.
-// Key rows are ldk floats apart.  Slot `cur` is taken from knew (the token being decoded is not
-// in the cache yet).
-__device__ __forceinline__ void chunk_scores(const float (*qs)[HD], const float *kc, int ldk, const float *knew, int cur, int k0,
-                                             int n, float (*sc)[MAXCHUNK], int tid) {
-	const int lane = tid & 63, w = tid >> 6, sub = lane >> 4, sl = lane & 15;
-	float4 q[NH][4];
-#pragma unroll
-	for (int h = 0; h < NH; h++)
-#pragma unroll
-		for (int i = 0; i < 4; i++) q[h][i] = *reinterpret_cast<const float4 *>(&qs[h][i * 64 + sl * 4]);
-	for (int base = 0; base < n; base += 16) {
-		const int jj = base + w * 4 + sub;
-		const bool ok = jj < n;
-		const int j = k0 + (ok ? jj : 0);
-		const float *kr = (j == cur) ? knew : kc + (size_t)j * ldk;
-		float4 kv[4];
-#pragma unroll
-		for (int i = 0; i < 4; i++) kv[i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
-#pragma unroll
-		for (int h = 0; h < NH; h++) {
-			float d = 0.0f;
-#pragma unroll
-			for (int i = 0; i < 4; i++) {
-				d = fmaf(q[h][i].x, kv[i].x, d);
-				d = fmaf(q[h][i].y, kv[i].y, d);
-				d = fmaf(q[h][i].z, kv[i].z, d);
-				d = fmaf(q[h][i].w, kv[i].w, d);
-			}
-			d = sum16(d);
-			if (ok && sl == 0) sc[h][jj] = d;
-		}
-	}
-}
-
 // Keys of a chunk whose K rows / V elements are fetched before anything else in the kernel (the rest, for
 // chunks longer than this, is fetched inside the loops).
 constexpr int PRE = 32;
