@@ -123,6 +123,20 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 /* Enqueues n_steps decode steps without host synchronisation (each step feeds the device-side
  * argmax of the previous one).  Ids are read back with tg_session_read_ids after tg_synchronize. */
 int tg_decode_enqueue(tg_session *s, int n_steps);
+/* ops::minp_logits (ops.hpp:762-859) on host pointers: temperature, softmax, min-p renormalisation of the
+ * denominator and inverse-transform sampling with the caller's uniform number randf in [0, 1).  Like the
+ * reference, tokens below the min-p cut are removed from the denominator only and can still be drawn.
+ * `logits` is not modified (the reference overwrites it with the probabilities).  n_vocab must be a multiple
+ * of 1024 (the reference is fixed to 262144); temp > 0. */
+int tg_minp_logits(const float *logits, int n_vocab, float minp, float temp, float randf, int32_t *token_out);
+/* The sampling branch of the decode loop of gemma::generate (transformer.hpp:229-235): like tg_decode_enqueue,
+ * but step i draws its token with minp_logits and randf[i] (the reference takes them from std::mt19937 +
+ * uniform_real_distribution<float>, transformer.hpp:170-172).  minp >= 1 selects the argmax branch, as there. */
+int tg_decode_enqueue_sampled(tg_session *s, int n_steps, float minp, float temp, const float *randf);
+/* Both branches of gemma::generate on token ids (transformer.hpp:166-256): prefill, first token, n_decode steps.
+ * randf[n_decode + 1] (first entry: the token after the prompt) is only read when minp < 1. */
+int tg_generate(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, float minp, float temp, const float *randf,
+                int32_t *out_ids, double *s_prefill, double *s_decode);
 /* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
 int tg_set_graphs(int enable);
 /* prefill GEMM: 1 (default) = int8 matrix cores on three int8 digit planes of the row-scaled activations

@@ -98,6 +98,7 @@ class Oracle:
         L.tgo_attention_prefill.argtypes = [c_f32p, c_f32p, c_f32p, c_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         L.tgo_attention_decode.argtypes = [c_f32p, c_f32p, c_f32p, c_f32p, C.c_int, C.c_int, C.c_int]
         L.tgo_argmax.argtypes = [c_f32p, C.c_int]
+        L.tgo_minp_logits.argtypes = [c_f32p, C.c_int, C.c_float, C.c_float, C.c_float]
         L.tgo_quantize.argtypes = [c_f32p, C.c_size_t, C.c_size_t, c_i8p, c_f32p]
         L.tgo_normal.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, C.c_float]
         L.tgo_normal.restype = C.c_float
@@ -185,6 +186,12 @@ class Oracle:
 
     def argmax(self, logits):
         return self.L.tgo_argmax(_f(logits), logits.size)
+
+    def minp_logits(self, logits, minp, temp, randf):
+        """Returns (index, probabilities as the reference leaves them in the logits buffer)."""
+        p = np.array(logits, np.float32, copy=True)
+        idx = self.L.tgo_minp_logits(_f(p), p.size, minp, temp, randf)
+        return idx, p
 
     # ---- producer ----
     def quantize(self, w):
@@ -321,6 +328,7 @@ class Ref:
         L.ref_attention_prefill.argtypes = [c_f32p, c_f32p, c_f32p, c_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         L.ref_attention_decode.argtypes = [c_f32p, c_f32p, c_f32p, c_f32p, C.c_int, C.c_int, C.c_int, C.c_int]
         L.ref_argmax.argtypes = [c_f32p]
+        L.ref_minp_logits.argtypes = [c_f32p, C.c_float, C.c_float, C.c_float]
         L.ref_model_create.argtypes = [C.c_int] * 9 + [C.c_float, C.c_float, C.c_int]
         L.ref_model_create.restype = C.c_void_p
         L.ref_model_load.argtypes = [C.c_void_p, C.c_char_p]
@@ -398,6 +406,12 @@ class Ref:
     def argmax(self, logits):
         assert logits.size == 262144
         return self.L.ref_argmax(_f(logits))
+
+    def minp_logits(self, logits, minp, temp, randf):
+        assert logits.size == 262144
+        p = np.array(logits, np.float32, copy=True)
+        idx = self.L.ref_minp_logits(_f(p), minp, temp, randf)
+        return idx, p
 
     def model(self, cfg, path):
         return _RefModel(self, cfg, path)

@@ -199,6 +199,17 @@ int ref_argmax(float *logits) {
 	return t.data[0];
 }
 
+// ops::minp_logits (ops.hpp:762); logits has constants::vocab entries and is overwritten with the
+// probabilities the reference leaves in it.
+int ref_minp_logits(float *logits, float minp, float temp, float randf) {
+	tensor::activation o(1, 1, constants::vocab);
+	std::memcpy(o.data.get(), logits, sizeof(float) * constants::vocab);
+	tensor::tokens t(1, 1);
+	ops::minp_logits(&t, &o, minp, temp, randf);
+	std::memcpy(logits, o.data.get(), sizeof(float) * constants::vocab);
+	return t.data[0];
+}
+
 // gemma::Transformer(Config) (transformer.hpp:33)
 void *ref_model_create(int hidden, int ffn, int layers, int vocab, int n_pos, int n_pos_local, int head_dim, int n_head,
                        int n_kv, float theta, float theta_local, int pattern) {

@@ -291,6 +291,39 @@ int tgo_argmax(const float *logits, int n) {
 	return arg;
 }
 
+/* ops.hpp:762-859.  The reference keeps 4 AVX2 accumulators (32 lanes) for the masked denominator and
+ * folds them as (v0+v1)+(v2+v3), then pairs of lanes (two hadd), then the two 128-bit halves
+ * (simd.hpp:16-32); that order is followed here.  The mask (p < minp * maxp -> 0) is applied inside
+ * the denominator loop only and never stored (ops.hpp:808-826 blend into a local), so every token,
+ * also those below the cut, is scaled by 1/denom and takes part in the draw (ops.hpp:836-857). */
+int tgo_minp_logits(float *l, int n, float minp, float temp, float randf) {
+	for (int i = 0; i < n; i++) l[i] /= temp;              /* :767-769 */
+	float rowmax = -INFINITY;
+	for (int i = 0; i < n; i++) rowmax = fmaxf(rowmax, l[i]); /* :773-787, max is order independent */
+	float maxp = -INFINITY;
+	for (int i = 0; i < n; i++) {                          /* :790-797 */
+		l[i] = expf(l[i] - rowmax);
+		if (l[i] > maxp) maxp = l[i];
+	}
+	const float cut = minp * maxp;                          /* :800 */
+	float lanes[32];
+	for (int j = 0; j < 32; j++) lanes[j] = 0.0f;
+	for (int i = 0; i < n; i += 32)                         /* :807-827 */
+		for (int j = 0; j < 32; j++) lanes[j] += (l[i + j] < cut) ? 0.0f : l[i + j];
+	float a[8];
+	for (int j = 0; j < 8; j++) a[j] = (lanes[j] + lanes[8 + j]) + (lanes[16 + j] + lanes[24 + j]); /* simd.hpp:27-29 */
+	const float denom = ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));            /* simd.hpp:17-22 */
+	const float inv = (float)(1.0 / (double)denom);         /* :836 */
+	for (int i = 0; i < n; i++) l[i] *= inv;                /* :838-846 */
+	float cum = 0.0f;                                       /* :849-857 */
+	int index = 0;
+	for (int i = 0; i < n; i++) {
+		cum += l[i];
+		if (cum >= randf) { index = i; break; }
+	}
+	return index;
+}
+
 /* ------------------------------------------------------------------------------------------ */
 /* quantizer + generator                                                                      */
 /* ------------------------------------------------------------------------------------------ */

@@ -67,6 +67,8 @@ void tgo_embedding(float *out, const int32_t *ids, int n, const int8_t *wte, con
 void tgo_attention_prefill(float *o, const float *q, const float *k, const float *v, int heads, int S, int dim, int is_sw, int sw_context); /* ops.hpp:377-526 */
 void tgo_attention_decode(float *o, const float *q, const float *kc, const float *vc, int heads, int dim, int valid); /* ops.hpp:224-370 */
 int tgo_argmax(const float *logits, int n);                                                         /* ops.hpp:744-760 */
+/* Overwrites logits[n] (n a multiple of 32) with the probabilities the reference leaves there; returns the drawn index. */
+int tgo_minp_logits(float *logits, int n, float minp, float temp, float randf);                     /* ops.hpp:762-859 */
 
 /* ---- quantizer and weight-file producer (py/weight_handlers.py:10-20, py/gemma.py:27-77) ---- */
 /* w is [rows][cols] fp32; q [rows][cols] int8; scales [cols]. Returns -1 if a column is all zero. */

@@ -79,6 +79,11 @@ def main():
     out["argmax"] = np.int32(r.argmax(lg))
     lg[1000] = lg[200000] = lg.max() + 1.0  # tie: the lowest index wins
     out["argmax_tie"] = np.int32(r.argmax(lg))
+    for name, (seed, scale, peaked, minp, temp, randf) in gi.MINP_CASES.items():
+        idx, probs = r.minp_logits(gi.minp_input(seed, scale, peaked), minp, temp, randf)
+        out[f"minp/{name}/index"] = np.int32(idx)
+        out[f"minp/{name}/prob_sum"] = np.float64(probs.astype(np.float64).sum())
+        out[f"minp/{name}/prob_head"] = probs[:256].copy()
 
     # ---- models ----
     for name, (shape, n_layers, seed, n_prompt, n_decode, n_tap_steps, gsize) in gi.MODEL_CASES.items():

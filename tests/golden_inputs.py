@@ -122,6 +122,30 @@ def argmax_input(seed):
     return np.random.default_rng(seed).standard_normal(262144).astype(np.float32)
 
 
+# min-p sampler (ops::minp_logits): name -> (logit seed, logit scale, peaked, minp, temp, randf)
+MINP_CASES = {
+    "flat": (31, 0.5, False, 0.05, 1.0, 0.3),
+    "warm": (32, 2.0, False, 0.2, 0.7, 0.93),
+    "nomask": (33, 6.0, False, 0.0, 1.3, 0.5),
+    "cold": (34, 3.0, False, 0.5, 0.25, 0.999),
+    "masked_mass": (35, 1.0, False, 0.9, 1.0, 0.01),    # below-cut tokens keep their mass: the "probabilities" sum to >> 1
+    "masked_late": (35, 1.0, False, 0.9, 1.0, 0.9999),
+    "peaked": (36, 1.0, True, 0.05, 0.8, 0.77),          # a handful of dominant logits, like a trained model
+    "peaked_tail": (36, 1.0, True, 0.0, 1.0, 0.99),
+    "zero_draw": (37, 2.0, False, 0.1, 1.0, 0.0),        # randf = 0: the very first token
+    "never_reached": (33, 6.0, False, 0.0, 1.3, 1.0),    # the running sum stays below randf: index 0 (ops.hpp:850)
+}
+
+
+def minp_input(seed, scale, peaked):
+    rng = np.random.default_rng(seed)
+    lg = (rng.standard_normal(262144) * scale).astype(np.float32)
+    if peaked:
+        hot = rng.integers(0, 262144, 12)
+        lg[hot] += rng.uniform(8.0, 14.0, 12).astype(np.float32)
+    return lg
+
+
 def prompt_ids(seed, n):
     return np.random.default_rng(1000 + seed).integers(0, 262144, n).astype(np.int32)
 

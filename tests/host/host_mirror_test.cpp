@@ -77,6 +77,30 @@ int main(int argc, char **argv) {
 	std::vector<int> prompt(tokens.data.begin(), tokens.data.end());
 	auto [n_gen, ids, s_prefill, s_decode] = gemma::generate_greedy(prompt, n_decode, &t);
 	for (int id : ids) std::printf("gid %d\n", id);
+
+	// the sampling branch (transformer.hpp:208-211, 232-235): the reference's loop spelled out with ops::minp_logits,
+	// against generate_ids with an equally seeded generator
+	{
+		const float minp = 0.05f, temp = 0.9f;
+		std::mt19937 gen(123), gen2(123);
+		std::uniform_real_distribution<float> unif(0.0, 1.0);
+		decode::DecodeState d2(1, &cfg);
+		gemma::forward_prefill(&o, &tokens, &t, &d2, &rope, &rope_sw, &table);
+		std::vector<int> stepwise;
+		ops::minp_logits(&tokens_decode, &o, minp, temp, unif(gen));
+		stepwise.push_back(tokens_decode.data[0]);
+		size_t off = tokens.y;
+		for (int step = 0; step < n_decode; step++, off++) {
+			gemma::forward_decode(&o, &tokens_decode, &t, &d2, &rope, &rope_sw, off, &table);
+			ops::minp_logits(&tokens_decode, &o, minp, temp, unif(gen));
+			stepwise.push_back(tokens_decode.data[0]);
+		}
+		auto [n2, sids, sp2, sd2] = gemma::generate_ids(prompt, n_decode, &t, minp, temp, gen2);
+		for (size_t i = 0; i < sids.size(); i++) {
+			std::printf("sid %d %d\n", stepwise[i], sids[i]);
+			if (stepwise[i] != sids[i]) failures++;
+		}
+	}
 	std::printf("failures %d\n", failures);
 	return failures ? 1 : 0;
 }

@@ -29,3 +29,6 @@ def test_cpp_mirror_generates_the_reference_ids(tg, oracle, golden, weight_image
     ref = golden["model/small6/tokens"].tolist()
     assert ids == ref and gids == ref
     assert "position 82" in r.stdout and "failures 0" in r.stdout
+    sampled = [l.split()[1:] for l in r.stdout.splitlines() if l.startswith("sid ")]
+    assert len(sampled) == 13 and all(a == b for a, b in sampled)      # stepwise minp_logits loop == generate_ids
+    assert len({a for a, _ in sampled}) > 6                            # and it does sample

@@ -118,3 +118,73 @@ def test_argmax(oracle, golden):
     assert oracle.argmax(lg) == int(golden["argmax"]) == int(np.argmax(lg))
     lg[1000] = lg[200000] = lg.max() + 1.0
     assert oracle.argmax(lg) == int(golden["argmax_tie"]) == 1000  # strict '>' scan: lowest index wins (ops.hpp:749-757)
+
+
+# ---- min-p sampler (ops::minp_logits, ops.hpp:762-859) ----
+def _minp_float64(lg, minp, temp, randf):
+    """Textbook restatement in float64: probabilities over ALL tokens divided by the mass of the tokens at or above
+    minp * max probability, then inverse-transform sampling; (index, probs, running sums).  index -1 = never reached."""
+    t = lg.astype(np.float32) / np.float32(temp)            # the reference divides and subtracts the maximum in fp32
+    p = np.exp((t - t.max()).astype(np.float64))
+    denom = p[p >= minp * p.max()].sum()
+    q = p / denom
+    cum = np.cumsum(q)
+    hit = np.nonzero(cum >= randf)[0]
+    return (int(hit[0]) if hit.size else -1), q, cum
+
+
+@pytest.mark.parametrize("name", list(gi.MINP_CASES))
+def test_minp_logits_against_reference_fixture(oracle, golden, name):
+    seed, scale, peaked, minp, temp, randf = gi.MINP_CASES[name]
+    lg = gi.minp_input(seed, scale, peaked)
+    idx, probs = oracle.minp_logits(lg, minp, temp, randf)
+    assert idx == int(golden[f"minp/{name}/index"])
+    ref_head = golden[f"minp/{name}/prob_head"]
+    assert np.abs(probs[:256] - ref_head).max() <= 3e-6 * ref_head.max()      # the reference's exp is a vectorised libm one
+    assert abs(probs.astype(np.float64).sum() - float(golden[f"minp/{name}/prob_sum"])) <= 3e-6 * float(golden[f"minp/{name}/prob_sum"])
+
+
+@pytest.mark.parametrize("name", list(gi.MINP_CASES))
+def test_minp_logits_against_float64_closed_form(oracle, name):
+    """Pins what a plausible mistake would change: a stored mask (probabilities of below-cut tokens zeroed), a cut
+    relative to the sum instead of the maximum, '>' instead of '>=' in the draw, a missing temperature."""
+    seed, scale, peaked, minp, temp, randf = gi.MINP_CASES[name]
+    lg = gi.minp_input(seed, scale, peaked)
+    idx, probs = oracle.minp_logits(lg, minp, temp, randf)
+    want, q, cum = _minp_float64(lg, minp, temp, randf)
+    # fp32 effect, not a mistake: the reference's 32 sequential lane accumulators absorb terms below half an ulp of a
+    # lane that holds a dominant probability, so its denominator can be low by ~1e-5 relative ("nomask": 8.8e-6)
+    assert np.abs(probs - q).max() <= 2e-5 * q.max()
+    seq_total = float(np.cumsum(probs, dtype=np.float32)[-1])   # what the reference's sequential fp32 scan ends at
+    if seq_total < randf:
+        # the fp32 running sum absorbs small terms and can end below 1 (here below randf) although the probabilities sum
+        # to >= 1 in exact arithmetic: the reference then leaves index 0 (ops.hpp:850)
+        assert idx == 0
+    elif want < 0:
+        assert cum[idx] >= randf - 3e-5
+    else:
+        # identical unless randf sits within fp32 summation error of a boundary of the cumulative distribution
+        assert idx == want or min(abs(cum[idx] - randf), abs(cum[max(idx - 1, 0)] - randf)) < 3e-5, (idx, want)
+    if name == "masked_mass":
+        assert probs.astype(np.float64).sum() > 100.0     # the quirk: below-cut tokens are not removed from the draw
+        assert q[idx] < minp * q.max()                    # ... and one of them is what this case draws
+    if name == "never_reached":
+        assert seq_total < randf and idx == 0             # ops.hpp:850: index stays 0
+
+
+def test_minp_logits_limits(oracle):
+    rng = np.random.default_rng(41)
+    lg = rng.standard_normal(262144).astype(np.float32)
+    # temperature -> 0 makes the draw the argmax for any randf that the top token's mass covers
+    top = int(np.argmax(lg))
+    idx, probs = oracle.minp_logits(lg, 0.0, 1e-3, 0.999)
+    assert probs[top] > 0.9 and idx <= top                # the running sum crosses at the latest at the dominant token
+    # one-hot distribution: every randf in (0, 1] gives that token
+    hot = np.full(262144, -1e4, np.float32)
+    hot[12345] = 0.0
+    for r in (1e-6, 0.5, 1.0):
+        assert oracle.minp_logits(hot, 0.1, 1.0, r)[0] == 12345
+    # uniform distribution: the draw is floor(randf * n) up to fp32 summation error
+    flat = np.zeros(262144, np.float32)
+    for r in (0.25, 0.5, 0.75):
+        assert abs(oracle.minp_logits(flat, 0.0, 1.0, r)[0] - r * 262144) < 64

@@ -14,7 +14,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libtinygemma_hip.so")
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip"]
+SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function"]
 
@@ -92,6 +92,10 @@ def lib():
     L.tg_forward_decode.argtypes = [C.c_void_p, C.c_int32, c_f32p, c_i32p]
     L.tg_generate_greedy.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_int, c_i32p, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.tg_decode_enqueue.argtypes = [C.c_void_p, C.c_int]
+    L.tg_minp_logits.argtypes = [c_f32p, C.c_int, C.c_float, C.c_float, C.c_float, c_i32p]
+    L.tg_decode_enqueue_sampled.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_float, c_f32p]
+    L.tg_generate.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_int, C.c_float, C.c_float, c_f32p, c_i32p,
+                              C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.tg_session_read_ids.argtypes = [C.c_void_p, c_i32p, C.c_int, c_i32p]
     L.tg_session_tap.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_session_kv.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
@@ -130,6 +134,14 @@ def launch_qgemv(Cv, A, B, scales, inDim, outDim, logits=False):
 
 def launch_qgemm(Cm, A, B, scales, m, inDim, outDim):
     check(lib().tg_qgemm(_f(Cm), _f(A), B.ctypes.data_as(c_i8p), _f(scales), m, inDim, outDim))
+
+
+def minp_logits(logits, minp, temp, randf):
+    """ops::minp_logits (ops.hpp:762): the sampled token id; `logits` is left untouched."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    tok = C.c_int32(-1)
+    check(lib().tg_minp_logits(_f(logits), logits.size, minp, temp, randf, C.byref(tok)))
+    return tok.value
 
 
 class DeviceBuffer:
@@ -268,6 +280,22 @@ class Session:
 
     def decode_enqueue(self, n):
         check(lib().tg_decode_enqueue(self.h, n))
+
+    def decode_enqueue_sampled(self, n, minp, temp, randf):
+        randf = np.ascontiguousarray(randf, np.float32)
+        assert randf.size >= n
+        check(lib().tg_decode_enqueue_sampled(self.h, n, minp, temp, _f(randf)))
+
+    def generate(self, prompt, n_decode, minp, temp, randf):
+        """gemma::generate on ids: randf[n_decode + 1] uniform draws, used when minp < 1."""
+        prompt = np.ascontiguousarray(prompt, np.int32)
+        randf = np.ascontiguousarray(randf, np.float32)
+        assert randf.size >= n_decode + 1
+        out = np.empty(n_decode + 1, np.int32)
+        sp, sd = C.c_double(), C.c_double()
+        check(lib().tg_generate(self.h, prompt.ctypes.data_as(c_i32p), prompt.size, n_decode, minp, temp, _f(randf),
+                                out.ctypes.data_as(c_i32p), C.byref(sp), C.byref(sd)))
+        return out, sp.value, sd.value
 
     def read_ids(self, max_ids):
         out = np.empty(max_ids, np.int32)

@@ -253,6 +253,12 @@ struct tg_session {
 	float *taps = nullptr;    // prefill taps [(2L+1)][rows][hidden] (kept only for short prompts)
 	int tap_rows = 0;
 	std::map<uint64_t, hipGraphExec_t> graphs;  // captured decode steps, keyed by the attention launch geometry
+	// min-p sampling (allocated on first use): scratch of the three sampler launches and the caller's uniform draws
+	float *probs = nullptr, *seg = nullptr, *bsum = nullptr, *bmax = nullptr, *randf = nullptr;
+	int randf_cap = 0;
+	bool sampling = false;  // decode steps enqueued now draw their token instead of taking the argmax
+	float s_minp = 1.0f, s_temp = 1.0f;
+	int rand_base = 0;      // token-log index of the token that uses randf[0]
 };
 
 namespace {
@@ -660,7 +666,7 @@ void tg_session_destroy(tg_session *s) {
 	s->graphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
-	              s->tok_log, s->taps};
+	              s->tok_log, s->taps, s->probs, s->seg, s->bsum, s->bmax, s->randf};
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
 	for (float *p : s->kc)
@@ -914,7 +920,13 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 	TG_MARK(TG_KC_LMHEAD);
 	TG_DO(TG_KC_LMHEAD, 0, tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream));
 	TG_MARK(TG_KC_ARGMAX);
-	if (!only) tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
+	if (!only) {
+		if (s->sampling)
+			tg_launch_minp(s->logits, c.n_vocab, s->s_minp, s->s_temp, s->randf, -1, s->rand_base, s->probs, s->seg, s->bsum, s->bmax,
+			               s->ctr, s->tok_log, 0, nullptr, g_stream);
+		else
+			tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
+	}
 	TG_MARK(-1);
 #undef TG_MARK
 #undef TG_DO
@@ -1198,6 +1210,104 @@ int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n
 	if (s_decode) *s_decode = std::chrono::duration<double>(t2 - t1).count();
 	return got == n_decode + 1 ? TG_OK : tg_fail(TG_ERR_STATE, "token log incomplete");
 }
+
+namespace {
+// scratch of the sampler + room for n draws, uploaded from the host
+int sampler_prepare(tg_session *s, const float *randf, int n) {
+	const tg_config &c = s->m->cfg;
+	if (c.n_vocab % 1024 != 0) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "sampler needs a vocabulary that is a multiple of 1024");
+	if (!s->probs) {
+		TG_HIP(hipMalloc((void **)&s->probs, sizeof(float) * (size_t)c.n_vocab));
+		TG_HIP(hipMalloc((void **)&s->seg, sizeof(float) * tg_minp_segments(c.n_vocab)));
+		TG_HIP(hipMalloc((void **)&s->bsum, sizeof(float) * tg_minp_blocks(c.n_vocab)));
+		TG_HIP(hipMalloc((void **)&s->bmax, sizeof(float) * tg_minp_blocks(c.n_vocab)));
+	}
+	if (n > s->randf_cap) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		if (s->randf) (void)hipFree(s->randf);
+		s->randf = nullptr;
+		s->randf_cap = 0;
+		TG_HIP(hipMalloc((void **)&s->randf, sizeof(float) * (size_t)n));
+		s->randf_cap = n;
+	}
+	// the previous batch of draws may still be in use by launches in flight
+	TG_HIP(hipStreamSynchronize(g_stream));
+	TG_HIP(hipMemcpy(s->randf, randf, sizeof(float) * (size_t)n, hipMemcpyHostToDevice));
+	return TG_OK;
+}
+bool sampler_args_ok(float minp, float temp) { return temp > 0.0f && minp >= 0.0f; }
+}  // namespace
+
+int tg_minp_logits(const float *logits, int n_vocab, float minp, float temp, float randf, int32_t *token_out) {
+	if (int rc = ensure_init()) return rc;
+	if (!logits || !token_out || !sampler_args_ok(minp, temp)) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (n_vocab < 1024 || n_vocab % 1024 != 0)
+		return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "Unsupported vocabulary size: " + std::to_string(n_vocab));
+	const size_t nb = tg_minp_blocks(n_vocab), ns = tg_minp_segments(n_vocab);
+	float *buf = nullptr;  // logits | probs | seg | bsum | bmax | randf | token
+	const size_t floats = 2 * (size_t)n_vocab + ns + 2 * nb + 2;
+	TG_HIP(hipMalloc((void **)&buf, sizeof(float) * floats));
+	float *d_logits = buf, *d_probs = buf + n_vocab, *d_seg = d_probs + n_vocab, *d_bsum = d_seg + ns, *d_bmax = d_bsum + nb,
+	      *d_rand = d_bmax + nb;
+	int *d_tok = reinterpret_cast<int *>(d_rand + 1);
+	int rc = TG_OK;
+	if (hipMemcpy(d_logits, logits, sizeof(float) * (size_t)n_vocab, hipMemcpyHostToDevice) != hipSuccess ||
+	    hipMemcpy(d_rand, &randf, sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+		rc = tg_fail(TG_ERR_HIP, "upload failed");
+	if (rc == TG_OK) {
+		tg_launch_minp(d_logits, n_vocab, minp, temp, d_rand, 0, 0, d_probs, d_seg, d_bsum, d_bmax, nullptr, nullptr, 2, d_tok, g_stream);
+		if (hipStreamSynchronize(g_stream) != hipSuccess || hipMemcpy(token_out, d_tok, sizeof(int), hipMemcpyDeviceToHost) != hipSuccess)
+			rc = tg_fail(TG_ERR_HIP, "sampler launch failed");
+	}
+	(void)hipFree(buf);
+	return rc;
+}
+
+int tg_decode_enqueue_sampled(tg_session *s, int n_steps, float minp, float temp, const float *randf) {
+	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (!(minp < 1.0f)) return tg_decode_enqueue(s, n_steps);  // transformer.hpp:232: minp >= 1 selects the argmax branch
+	if (!randf || !sampler_args_ok(minp, temp)) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (n_steps == 0) return TG_OK;
+	if (int rc = sampler_prepare(s, randf, n_steps)) return rc;
+	s->sampling = true;
+	s->s_minp = minp;
+	s->s_temp = temp;
+	s->rand_base = s->steps;
+	int rc = TG_OK;
+	for (int i = 0; i < n_steps && rc == TG_OK; i++) rc = enqueue_decode_step(s, nullptr, false);
+	s->sampling = false;
+	if (rc == TG_OK && s->taps) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		(void)hipFree(s->taps);
+		s->taps = nullptr;
+		s->tap_rows = 0;
+	}
+	return rc;
+}
+
+int tg_generate(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, float minp, float temp, const float *randf,
+                int32_t *out_ids, double *s_prefill, double *s_decode) {
+	if (!(minp < 1.0f)) return tg_generate_greedy(s, prompt, n_prompt, n_decode, out_ids, s_prefill, s_decode);
+	if (!s || !prompt || !out_ids || !randf || n_decode < 0 || !sampler_args_ok(minp, temp)) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	using clk = std::chrono::steady_clock;
+	auto t0 = clk::now();
+	int32_t tok = -1;
+	if (int rc = tg_forward_prefill(s, prompt, n_prompt, nullptr, &tok)) return rc;
+	// the prefill logits are still on the device: draw the first token from them (transformer.hpp:208-211)
+	if (int rc = sampler_prepare(s, randf, 1)) return rc;
+	tg_launch_minp(s->logits, s->m->cfg.n_vocab, minp, temp, s->randf, 0, 0, s->probs, s->seg, s->bsum, s->bmax, s->ctr, s->tok_log, 1,
+	               nullptr, g_stream);
+	TG_HIP(hipStreamSynchronize(g_stream));
+	auto t1 = clk::now();
+	if (int rc = tg_decode_enqueue_sampled(s, n_decode, minp, temp, randf + 1)) return rc;
+	int got = 0;
+	if (int rc = tg_session_read_ids(s, out_ids, n_decode + 1, &got)) return rc;
+	auto t2 = clk::now();
+	if (s_prefill) *s_prefill = std::chrono::duration<double>(t1 - t0).count();
+	if (s_decode) *s_decode = std::chrono::duration<double>(t2 - t1).count();
+	return got == n_decode + 1 ? TG_OK : tg_fail(TG_ERR_STATE, "token log incomplete");
+}
+
 
 // ---------------------------------------------------------------------------------------------
 // debug taps

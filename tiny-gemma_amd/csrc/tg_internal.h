@@ -132,6 +132,13 @@ void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s);
 void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s);
 void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s);
 void tg_launch_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log, int advance, hipStream_t s);
+// min-p sampling (tg_sample.hip): n a multiple of 1024; scratch probs[n], seg[tg_minp_segments(n)], bsum/bmax[tg_minp_blocks(n)];
+// mode 0 = decode step (append + advance), 1 = replace the token written last, 2 = out_tok only;
+// the draw is randf[rand_idx], or randf[ctr[3] - rand_base (- 1 in mode 1)] when rand_idx < 0
+size_t tg_minp_blocks(int n);
+size_t tg_minp_segments(int n);
+void tg_launch_minp(const float *logits, int n, float minp, float temp, const float *randf, int rand_idx, int rand_base, float *probs,
+                    float *seg, float *bsum, float *bmax, int *ctr, int *tok_log, int mode, int *out_tok, hipStream_t s);
 
 // ---- prefill kernels (rows = prompt positions) -----------------------------------------------
 void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,

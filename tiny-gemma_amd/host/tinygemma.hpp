@@ -11,8 +11,8 @@
 //   decode::RoPE, decode::DecodeState             decode.hpp:107-276
 //   gemma::Transformer, read_weights,
 //   gemma::forward_prefill, forward_decode        transformer.hpp:22-165
-//   ops::argmax_logits                            ops.hpp:744
-//   gemma::generate_greedy                        greedy branch of transformer.hpp:167-258 on token ids
+//   ops::argmax_logits, ops::minp_logits          ops.hpp:744, 762
+//   gemma::generate_greedy, gemma::generate_ids   transformer.hpp:167-258 on token ids (argmax / min-p branch)
 //
 // Errors: the reference throws std::runtime_error for an unknown dimension ("Unsupported ROW/COL
 // dimension: N") and an unopenable weight file ("Could not open file."), and assert()s on shape
@@ -24,6 +24,7 @@
 #include <cstdint>
 #include <cstring>
 #include <memory>
+#include <random>
 #include <stdexcept>
 #include <string>
 #include <tuple>
@@ -212,6 +213,25 @@ inline std::tuple<int, std::vector<int>, float, float> generate_greedy(const std
 	check(tg_generate_greedy(d.session, prompt.data(), (int)prompt.size(), n_decode, ids.data(), &sp, &sd));
 	return {n_decode, ids, (float)sp, (float)sd};
 }
+
+// Both branches of gemma::generate on token ids: minp < 1 draws every token with ops::minp_logits and uniform
+// numbers from `gen` in the reference's order (one per produced token, transformer.hpp:170-172, 208-211, 232-235);
+// the reference seeds its std::mt19937 from std::random_device, here the caller owns the generator.
+inline std::tuple<int, std::vector<int>, float, float> generate_ids(const std::vector<int> &prompt, int n_decode, Transformer *t,
+                                                                    const float minp, const float temp, std::mt19937 &gen) {
+	if (!(minp < 1)) return generate_greedy(prompt, n_decode, t);
+	std::uniform_real_distribution<float> unif(0.0, 1.0);
+	std::vector<float> randf((size_t)n_decode + 1);
+	for (float &r : randf) r = unif(gen);
+	decode::RoPE rope(&t->cfg, false), rope_sw(&t->cfg, true);
+	lut::GeLUTable table{-4.0, 4.0, 1024};  // transformer.hpp:197
+	decode::DecodeState d(1, &t->cfg);
+	bind_session(t, &d, &rope, &rope_sw, &table);
+	std::vector<int> ids((size_t)n_decode + 1);
+	double sp = 0, sd = 0;
+	check(tg_generate(d.session, prompt.data(), (int)prompt.size(), n_decode, minp, temp, randf.data(), ids.data(), &sp, &sd));
+	return {n_decode, ids, (float)sp, (float)sd};
+}
 }  // namespace gemma
 
 namespace ops {
@@ -225,6 +245,13 @@ inline void argmax_logits(tensor::tokens *toks, tensor::activation *o) {
 			best = o->data[i];
 		}
 	toks->data[0] = arg;
+}
+
+// ops.hpp:762: the logits buffer is left as it is (the reference overwrites it with the probabilities)
+inline void minp_logits(tensor::tokens *toks, tensor::activation *o, float minp, float temp, float randf) {
+	int32_t tok = 0;
+	check(tg_minp_logits(o->data.data(), (int)o->data.size(), minp, temp, randf, &tok));
+	toks->data[0] = tok;
 }
 }  // namespace ops
 
