@@ -145,12 +145,43 @@ def test_decode_from_empty_session(tg, oracle, weight_images, tables):
     assert sess.position == 3
 
 
-def greedy_vs_golden(sess, golden, name, prompt, n_decode):
+NEAR_TIE = 0.02   # top-2 logit gap of the reference below which its runner-up is an acceptable pick (logit spread ~0.5)
+
+
+def greedy_vs_golden(sess, golden, name, prompt, n_decode, strict=True):
+    """Free-running greedy ids against the compiled reference's.  strict: identical over the whole horizon.
+    Otherwise a divergence may only start at a near-tie of the reference, with the reference's runner-up
+    (after it the two runs legitimately see different contexts)."""
     toks, s_prefill, s_decode = sess.greedy(prompt, n_decode)
     ref = golden[f"model/{name}/tokens"]
+    gaps = golden[f"model/{name}/top2_gaps"]
     mism = np.nonzero(toks != ref)[0]
-    assert mism.size == 0, (f"greedy ids diverge from the reference at step {mism[0]} "
-                            f"(reference top-2 gap there: {golden[f'model/{name}/top2_gaps'][mism[0]]:.3e})")
+    if mism.size == 0:
+        return -1
+    i = int(mism[0])
+    msg = f"greedy ids diverge from the reference at step {i} (reference top-2 gap there: {gaps[i]:.3e})"
+    assert not strict, msg
+    assert gaps[i] < NEAR_TIE and toks[i] == golden[f"model/{name}/top2_ids"][i][1], msg
+    return i
+
+
+def teacher_forced_vs_golden(sess, golden, name, prompt, n_decode, max_mismatches=4):
+    """Fed the reference's ids step by step, every pick must be the reference's; at a near-tie of the reference
+    (gap < NEAR_TIE) its runner-up is the only other acceptable answer."""
+    ref = golden[f"model/{name}/tokens"]
+    gaps = golden[f"model/{name}/top2_gaps"]
+    pairs = golden[f"model/{name}/top2_ids"]
+    tok, _ = sess.prefill(prompt, want_logits=False)
+    picks = [tok]
+    for i in range(n_decode):
+        tok, _ = sess.decode(int(ref[i]), want_logits=False)
+        picks.append(tok)
+    picks = np.array(picks, np.int32)
+    mism = np.nonzero(picks != ref)[0]
+    assert mism.size <= max_mismatches, mism
+    for i in mism:
+        assert gaps[i] < NEAR_TIE and picks[i] == pairs[i][1], (i, gaps[i], picks[i], pairs[i])
+    return mism
 
 
 def check_weights(golden, weight_images, name):
@@ -177,28 +208,22 @@ def test_full_270m_near_ties(tg, oracle, golden, weight_images, tables):
     only other acceptable answer."""
     check_weights(golden, weight_images, "full270m_ties")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full270m_ties")
-    ref = golden["model/full270m_ties/tokens"]
-    gaps = golden["model/full270m_ties/top2_gaps"]
-    pairs = golden["model/full270m_ties/top2_ids"]
-    tok, _ = sess.prefill(prompt, want_logits=False)
-    picks = [tok]
-    for i in range(256):
-        tok, _ = sess.decode(int(ref[i]), want_logits=False)
-        picks.append(tok)
-    picks = np.array(picks, np.int32)
-    mism = np.nonzero(picks != ref)[0]
-    assert mism.size <= 4, mism
-    for i in mism:
-        assert gaps[i] < 0.02 and picks[i] == pairs[i][1], (i, gaps[i], picks[i], pairs[i])
+    teacher_forced_vs_golden(sess, golden, "full270m_ties", prompt, 256)
 
 
 def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
-    """178-token prompt + 1024 greedy steps, 26 layers (the benchmark workload)."""
+    """178-token prompt + 1024 greedy steps, 26 layers (the benchmark workload).  Over 1024 steps of 26 layers with the
+    1024-entry GeLU table the logits sit ~4e-3 from the compiled reference's (so does the strict-IEEE CPU checker), and
+    the reference's own path crosses top-2 gaps of that size (1e-3 at the smallest): the free run may leave the
+    reference's path at such a near-tie, by picking its runner-up; teacher-forced, every other pick must be identical."""
     if "model/full1B/tokens" not in golden:
         pytest.skip("fixture was written without the 1B case")
     check_weights(golden, weight_images, "full1B")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full1B")
-    greedy_vs_golden(sess, golden, "full1B", prompt, 1024)
+    first = greedy_vs_golden(sess, golden, "full1B", prompt, 1024, strict=False)
+    assert first < 0 or first > 256                      # and not early: the first 256 steps hold no gap below 0.01
+    sess.reset()
+    teacher_forced_vs_golden(sess, golden, "full1B", prompt, 1024, max_mismatches=6)
     # last-position activations of the prefill against the reference's
     sess.reset()
     tok, logits = sess.prefill(prompt)

@@ -21,21 +21,9 @@ constexpr int NH = 4;          // query heads sharing the single KV head
 constexpr int ANT = 256;       // threads per workgroup
 constexpr int MAXCHUNK = 256;  // keys per workgroup, upper bound
 
-__device__ __forceinline__ float wsum(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-	return v;
-}
-__device__ __forceinline__ float wmax(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-	return v;
-}
-__device__ __forceinline__ float sum16(float v) {  // over aligned groups of 16 lanes
-#pragma unroll
-	for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-	return v;
-}
+__device__ __forceinline__ float wsum(float v) { return tg_wave_sum(v); }
+__device__ __forceinline__ float wmax(float v) { return tg_wave_max(v); }
+__device__ __forceinline__ float sum16(float v) { return tg_row16_sum(v); }  // over aligned groups of 16 lanes
 
 // One wave normalises and rotates one 256-wide head vector (ops.hpp:126-180, decode.hpp:136-211).
 // Lane l owns dims {l, l+64, l+128, l+192}: both members of every rotation pair (d, d+128).

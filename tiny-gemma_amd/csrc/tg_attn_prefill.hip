@@ -108,8 +108,8 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 			if (jb > qpos || jb < klo) s1[i] = -INFINITY;
 			tmax = fmaxf(tmax, fmaxf(s0[i], s1[i]));
 		}
-		tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-		tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+		tmax = fmaxf(tmax, tg_red_partner<16>(tmax));
+		tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
 		const float m_new = fmaxf(m_run, tmax);  // finite from the first tile on: it holds a valid key of every query
 		const float alpha = expf(m_run - m_new);
 		float psum = 0.0f;
@@ -119,8 +119,8 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 			s1[i] = expf(s1[i] - m_new);
 			psum += s0[i] + s1[i];
 		}
-		psum += __shfl_xor(psum, 16, 64);
-		psum += __shfl_xor(psum, 32, 64);
+		psum += tg_red_partner<16>(psum);
+		psum += tg_red_partner<32>(psum);
 		l_run = fmaf(l_run, alpha, psum);
 		m_run = m_new;
 		// rescale the output rows this lane holds (queries 4 g + i)

@@ -65,8 +65,7 @@ __global__ __launch_bounds__(GNT) void row_scale_kernel(const float *A, int lda,
 			amax = fmaxf(amax, fmaxf(fmaxf(fabsf(a[0]), fabsf(a[1])), fmaxf(fabsf(a[2]), fabsf(a[3]))));
 		}
 	}
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+	amax = tg_wave_max(amax);
 	if (lane == 0) {
 		float s = 1.0f, r = 1.0f;
 		if (amax > 0.0f && amax < INFINITY) {

@@ -47,11 +47,7 @@ __device__ __forceinline__ f32x4 ldx(__amdgpu_buffer_rsrc_t r, uint32_t voff, ui
 	return __builtin_bit_cast(f32x4, t);
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-	return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return tg_wave_sum(v); }
 
 // Sum over the workgroup; every thread gets the same value (fixed order).
 __device__ __forceinline__ float block_sum(float v, float *sred) {
@@ -148,13 +144,12 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			const bool ok = b < nb;
 			const float m = ok ? g.part_ml[((size_t)b * 4 + h) * 2] : -INFINITY;
 			const float l = ok ? g.part_ml[((size_t)b * 4 + h) * 2 + 1] : 0.0f;
-			float M = m;
-#pragma unroll
-			for (int o = TG_ATTN_MERGE_MAX / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+			static_assert(TG_ATTN_MERGE_MAX == 16, "one row of 16 lanes per head");
+			const float M = tg_row16_max(m);
 			const float e = ok ? expf(m - M) : 0.0f;
-			float L = l * e;
-#pragma unroll
-			for (int o = TG_ATTN_MERGE_MAX / 2; o > 0; o >>= 1) L += __shfl_xor(L, o, 64);
+			// __fmul_rn: the product must be rounded before the reduction; contracted into the first add
+			// (fma(l, e, partner)) the two lanes of a pair would no longer hold the same sum
+			const float L = tg_row16_sum(__fmul_rn(l, e));
 			wgt[h][b] = e / L;
 		}
 		__syncthreads();
@@ -285,10 +280,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	}
 
 	// ---------------- reduction over the lanes along K (fixed order) ----------------
-	for (int o = 32; o >= LC; o >>= 1) {
-#pragma unroll
-		for (int j = 0; j < 4; j++) acc[j] += __shfl_xor(acc[j], o, 64);
+	// lanes l and l' hold partial sums of the same columns iff l % LC == l' % LC
+#define TG_STEP(O)                                                   \
+	if (LC <= O) {                                                   \
+		_Pragma("unroll") for (int j = 0; j < 4; j++) acc[j] += tg_red_partner<O>(acc[j]); \
 	}
+	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
+#undef TG_STEP
 	if (lane < LC) *reinterpret_cast<float4 *>(&red[w][lane * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
 	__syncthreads();
 
@@ -321,12 +319,14 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			if (g.y != nullptr) g.y[col] = val;
 			if (val > bv) { bv = val; bi = col; }
 		}
-#pragma unroll
-		for (int o = 32; o > 0; o >>= 1) {
-			const float ov = __shfl_xor(bv, o, 64);
-			const int oi = __shfl_xor(bi, o, 64);
-			if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-		}
+#define TG_STEP(O)                                                                  \
+	{                                                                               \
+		const float ov = tg_red_partner<O>(bv);                                     \
+		const int oi = tg_red_partner<O>(bi);                                       \
+		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }                 \
+	}
+		TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
+#undef TG_STEP
 		if (lane == 0) { s_bv[it & 1][w] = bv; s_bi[it & 1][w] = bi; }
 		__syncthreads();
 		if (tid == 0) {
@@ -367,12 +367,14 @@ __global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, con
 		const int oi = blk_idx[i];
 		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 	}
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) {
-		const float ov = __shfl_xor(bv, o, 64);
-		const int oi = __shfl_xor(bi, o, 64);
-		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+#define TG_STEP(O)                                                      \
+	{                                                                   \
+		const float ov = tg_red_partner<O>(bv);                         \
+		const int oi = tg_red_partner<O>(bi);                           \
+		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }     \
 	}
+	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
+#undef TG_STEP
 	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
 	__syncthreads();
 	if (tid == 0) {

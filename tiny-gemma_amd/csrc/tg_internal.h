@@ -169,6 +169,78 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 // of prefetched tiles at every stage; here loads issued earlier stay in flight across the barrier.
 __device__ __forceinline__ void tg_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// ---- cross-lane reductions without the LDS crossbar --------------------------------------------
+// __shfl_xor compiles to ds_bpermute_b32 (address arithmetic + an LDS round trip, ~100 clocks of
+// dependent latency per step).  The steps of a butterfly reduction have cheaper forms on gfx950:
+// quad permutes and row rotations (DPP modifiers on a VALU move) inside a row of 16 lanes,
+// v_permlane16_swap / v_permlane32_swap across rows.  tg_red_partner<O>(v) is what a reduction that walks
+// O = 32, 16, 8, 4, 2, 1 DOWNWARDS (possibly starting lower) must combine with at step O.  At the 4-step
+// the row rotation delivers lane (l - 4) mod 16 instead of l ^ 4; after the 8-step both hold the same
+// value, so the reduction is bit-identical to the xor butterfly.  Not a general shuffle.
+#if defined(__HIPCC__)
+template <int CTRL>
+__device__ __forceinline__ unsigned tg_dpp_u32(unsigned v) {
+	return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int O>
+__device__ __forceinline__ unsigned tg_red_partner_u32(unsigned v) {
+	static_assert(O == 32 || O == 16 || O == 8 || O == 4 || O == 2 || O == 1, "butterfly step");
+	if constexpr (O == 32) {
+		const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);  // r[0] = {lo, lo}, r[1] = {hi, hi}
+		return (__lane_id() & 32) ? r[0] : r[1];
+	} else if constexpr (O == 16) {
+		const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);  // r[0] = rows {0,0,2,2}, r[1] = rows {1,1,3,3}
+		return (__lane_id() & 16) ? r[0] : r[1];
+	} else if constexpr (O == 8) {
+		return tg_dpp_u32<0x128>(v);  // row_ror:8
+	} else if constexpr (O == 4) {
+		return tg_dpp_u32<0x124>(v);  // row_ror:4
+	} else if constexpr (O == 2) {
+		return tg_dpp_u32<0x4E>(v);   // quad_perm:[2,3,0,1]
+	} else {
+		return tg_dpp_u32<0xB1>(v);   // quad_perm:[1,0,3,2]
+	}
+}
+template <int O>
+__device__ __forceinline__ float tg_red_partner(float v) { return __uint_as_float(tg_red_partner_u32<O>(__float_as_uint(v))); }
+template <int O>
+__device__ __forceinline__ int tg_red_partner(int v) { return (int)tg_red_partner_u32<O>((unsigned)v); }
+
+// sums / maxima over the wave, a row of 16 lanes, or the lanes sharing (lane % LC); all lanes get the result
+__device__ __forceinline__ float tg_wave_sum(float v) {
+	v += tg_red_partner<32>(v);
+	v += tg_red_partner<16>(v);
+	v += tg_red_partner<8>(v);
+	v += tg_red_partner<4>(v);
+	v += tg_red_partner<2>(v);
+	v += tg_red_partner<1>(v);
+	return v;
+}
+__device__ __forceinline__ float tg_wave_max(float v) {
+	v = fmaxf(v, tg_red_partner<32>(v));
+	v = fmaxf(v, tg_red_partner<16>(v));
+	v = fmaxf(v, tg_red_partner<8>(v));
+	v = fmaxf(v, tg_red_partner<4>(v));
+	v = fmaxf(v, tg_red_partner<2>(v));
+	v = fmaxf(v, tg_red_partner<1>(v));
+	return v;
+}
+__device__ __forceinline__ float tg_row16_sum(float v) {
+	v += tg_red_partner<8>(v);
+	v += tg_red_partner<4>(v);
+	v += tg_red_partner<2>(v);
+	v += tg_red_partner<1>(v);
+	return v;
+}
+__device__ __forceinline__ float tg_row16_max(float v) {
+	v = fmaxf(v, tg_red_partner<8>(v));
+	v = fmaxf(v, tg_red_partner<4>(v));
+	v = fmaxf(v, tg_red_partner<2>(v));
+	v = fmaxf(v, tg_red_partner<1>(v));
+	return v;
+}
+#endif
+
 // ---- errors -----------------------------------------------------------------------------------
 int tg_fail(int code, const std::string &msg);
 #define TG_HIP(expr)                                                                           \

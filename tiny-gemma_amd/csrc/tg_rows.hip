@@ -14,11 +14,7 @@ namespace {
 
 constexpr int RNT = 256;
 
-__device__ __forceinline__ float wsum(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-	return v;
-}
+__device__ __forceinline__ float wsum(float v) { return tg_wave_sum(v); }
 
 __device__ __forceinline__ float bsum(float v, float *sred) {
 	v = wsum(v);

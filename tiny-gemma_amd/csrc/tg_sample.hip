@@ -29,16 +29,8 @@ constexpr int NONE = 0x7fffffff;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-	return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-	return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return tg_wave_max(v); }
+__device__ __forceinline__ float wave_sum(float v) { return tg_wave_sum(v); }
 
 // bmax[b] = max over the workgroup's 1024 elements of logits[i] / temp
 __global__ __launch_bounds__(SNT) void minp_max_kernel(const float *logits, float temp, float *bmax) {
