@@ -27,24 +27,41 @@ __device__ __forceinline__ float sum16(float v) { return tg_row16_sum(v); }  // 
 
 // One wave normalises and rotates one 256-wide head vector (ops.hpp:126-180, decode.hpp:136-211).
 // Lane l owns dims {l, l+64, l+128, l+192}: both members of every rotation pair (d, d+128).
-// cs/sn point at the [hd/2] table row of this token's position.
-__device__ __forceinline__ void norm_rope_head(const float *src, const float *w, const float *cs, const float *sn, float mul,
-                                               float out[4], int lane) {
-	float x[4];
+// cs/sn point at the [hd/2] table row of this token's position.  Split in two so that a caller can put
+// all of the loads in front of other, bulkier loads: the wait for a load also waits for every load
+// issued before it.
+struct HeadIn {
+	float x[4], w[4], c0, c1, s0, s1;
+};
+__device__ __forceinline__ void head_load(HeadIn &in, const float *src, const float *w, const float *cs, const float *sn, int lane) {
 #pragma unroll
-	for (int i = 0; i < 4; i++) x[i] = src[lane + 64 * i];
+	for (int i = 0; i < 4; i++) in.x[i] = src[lane + 64 * i];
+#pragma unroll
+	for (int i = 0; i < 4; i++) in.w[i] = w[lane + 64 * i];
+	in.c0 = cs[lane];
+	in.c1 = cs[lane + 64];
+	in.s0 = sn[lane];
+	in.s1 = sn[lane + 64];
+}
+__device__ __forceinline__ void head_finish(const HeadIn &in, float mul, float out[4]) {
+	float x[4];
 	float ss = 0.0f;
 #pragma unroll
-	for (int i = 0; i < 4; i++) ss = fmaf(x[i], x[i], ss);
+	for (int i = 0; i < 4; i++) ss = fmaf(in.x[i], in.x[i], ss);
 	ss = wsum(ss);
 	const float irms = 1.0f / sqrtf(ss / (float)HD + 1e-06f);
 #pragma unroll
-	for (int i = 0; i < 4; i++) x[i] = (x[i] * irms) * (w[lane + 64 * i] + 1.0f);
-	const float c0 = cs[lane], c1 = cs[lane + 64], s0 = sn[lane], s1 = sn[lane + 64];
-	out[0] = fmaf(c0, x[0], (-x[2]) * s0) * mul;
-	out[1] = fmaf(c1, x[1], (-x[3]) * s1) * mul;
-	out[2] = fmaf(c0, x[2], x[0] * s0) * mul;
-	out[3] = fmaf(c1, x[3], x[1] * s1) * mul;
+	for (int i = 0; i < 4; i++) x[i] = (in.x[i] * irms) * (in.w[i] + 1.0f);
+	out[0] = fmaf(in.c0, x[0], (-x[2]) * in.s0) * mul;
+	out[1] = fmaf(in.c1, x[1], (-x[3]) * in.s1) * mul;
+	out[2] = fmaf(in.c0, x[2], x[0] * in.s0) * mul;
+	out[3] = fmaf(in.c1, x[3], x[1] * in.s1) * mul;
+}
+__device__ __forceinline__ void norm_rope_head(const float *src, const float *w, const float *cs, const float *sn, float mul,
+                                               float out[4], int lane) {
+	HeadIn in;
+	head_load(in, src, w, cs, sn, lane);
+	head_finish(in, mul, out);
 }
 
 // Keys of a chunk whose K rows / V elements are fetched before anything else in the kernel (the rest, for
@@ -55,7 +72,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	__shared__ __attribute__((aligned(16))) float qs[NH][HD];
 	__shared__ __attribute__((aligned(16))) float knew[HD];
 	__shared__ float vnew[HD];
-	__shared__ float sc[NH][MAXCHUNK];
+	__shared__ __attribute__((aligned(16))) float sc[NH][MAXCHUNK];
 	__shared__ float s_m[NH], s_l[NH];
 
 	if ((int)blockIdx.x >= a.nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
@@ -73,7 +90,14 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	const int k0 = b * a.chunk;
 	const int n = (valid - k0 < a.chunk) ? valid - k0 : a.chunk;
 
-	// Cache rows of the first PRE keys of this chunk go out first: they depend on nothing computed here.
+	// Everything is requested up front.  The few values the q/k path needs go first (the previous launch's
+	// q|k|v vector, norm weights, RoPE row): a wait for them must not include the cache rows behind them.
+	HeadIn qin, kin;
+	const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
+	head_load(qin, a.qkv + w * HD, a.rms_q, cs, sn, lane);
+	if (w == 0) head_load(kin, a.qkv + NH * HD, a.rms_k, cs, sn, lane);
+	const float vnew_r = a.qkv[NH * HD + HD + tid];
+	// Cache rows of the first PRE keys of this chunk: they depend on nothing computed here.
 	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: thread = output dim.
 	float4 kpre[PRE / 16][4];
 	float vpre[PRE];
@@ -93,17 +117,16 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 
 	// q heads: one wave each; k: wave 0 again
 	{
-		const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
 		float o[4];
-		norm_rope_head(a.qkv + w * HD, a.rms_q, cs, sn, 0.0625f, o, lane);  // ops.hpp:257: q *= 1/sqrt(256)
+		head_finish(qin, 0.0625f, o);  // ops.hpp:257: q *= 1/sqrt(256)
 #pragma unroll
 		for (int i = 0; i < 4; i++) qs[w][lane + 64 * i] = o[i];
 		if (w == 0) {
-			norm_rope_head(a.qkv + NH * HD, a.rms_k, cs, sn, 1.0f, o, lane);
+			head_finish(kin, 1.0f, o);
 #pragma unroll
 			for (int i = 0; i < 4; i++) knew[lane + 64 * i] = o[i];
 		}
-		vnew[tid] = a.qkv[NH * HD + HD + tid];
+		vnew[tid] = vnew_r;
 	}
 	__syncthreads();
 	if (b == 0) {  // KVCache::update_single, decode.hpp:49-70
@@ -173,11 +196,20 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	// P.V: thread = output dim, 4 heads
 	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-	for (int u = 0; u < PRE; u++) {
-		if (u < n) {
-			const float vv = (k0 + u == cur) ? vnew[tid] : vpre[u];
+	for (int u4 = 0; u4 < PRE; u4 += 4) {
+		if (u4 < n) {  // entries past n are read with the group but not used
+			float4 p[NH];
 #pragma unroll
-			for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][u], vv, acc[h]);
+			for (int h = 0; h < NH; h++) p[h] = *reinterpret_cast<const float4 *>(&sc[h][u4]);
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				const int u = u4 + e;
+				if (u < n) {
+					const float vv = (k0 + u == cur) ? vnew[tid] : vpre[u];
+#pragma unroll
+					for (int h = 0; h < NH; h++) acc[h] = fmaf(reinterpret_cast<const float *>(&p[h])[e], vv, acc[h]);
+				}
+			}
 		}
 	}
 	for (int j0 = PRE; j0 < n; j0 += 8) {
