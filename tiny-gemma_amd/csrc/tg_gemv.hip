@@ -111,18 +111,23 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.x, (PRO == TG_PRO_PLAIN) ? (uint32_t)g.K * 4u : 0u);
 	const uint32_t voff = (uint32_t)tid * 16u, xoff = (uint32_t)kpos * 16u, xstep = (uint32_t)KL * 16u;
 
-	// first DEPTH steps are issued before the prologue: they do not depend on it
+	// The first DEPTH steps of the weight stream do not depend on the prologue and are requested before
+	// its arithmetic starts, but BEHIND the prologue's own (small) loads: a wait for a load also waits for
+	// every load issued before it, and the prologue must not wait for 32 KB of weights to see its inputs.
 	i32x4 v[DEPTH];
 	f32x4 xq[DEPTH];
+	auto issue_weights = [&]() {
 #pragma unroll
-	for (int u = 0; u < DEPTH; u++) {
-		v[u] = i32x4{0, 0, 0, 0};
-		xq[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-		if (u < nit) {
-			v[u] = ldw(rw, voff, (uint32_t)u * STEP_BYTES);
-			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
+		for (int u = 0; u < DEPTH; u++) {
+			v[u] = i32x4{0, 0, 0, 0};
+			xq[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+			if (u < nit) {
+				v[u] = ldw(rw, voff, (uint32_t)u * STEP_BYTES);
+				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
+			}
 		}
-	}
+	};
+	if (PRO == TG_PRO_PLAIN) issue_weights();
 
 	// ---------------- prologue: input vector ----------------
 	// Every global load of a prologue that does not depend on another one is issued up front, next
@@ -134,16 +139,21 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
 		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
 		float a[4][TG_ATTN_MERGE_MAX];
+		float m = -INFINITY, l = 0.0f;
+		if (tid < 4 * TG_ATTN_MERGE_MAX && (tid % TG_ATTN_MERGE_MAX) < nb) {
+			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
+			m = g.part_ml[((size_t)b * 4 + h) * 2];
+			l = g.part_ml[((size_t)b * 4 + h) * 2 + 1];
+		}
 #pragma unroll
 		for (int h = 0; h < 4; h++)
 #pragma unroll
 			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
 				a[h][b] = (b < nb) ? g.part_acc[((size_t)b * 4 + h) * 256 + tid] : 0.0f;
+		issue_weights();
 		if (tid < 4 * TG_ATTN_MERGE_MAX) {
 			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
 			const bool ok = b < nb;
-			const float m = ok ? g.part_ml[((size_t)b * 4 + h) * 2] : -INFINITY;
-			const float l = ok ? g.part_ml[((size_t)b * 4 + h) * 2 + 1] : 0.0f;
 			static_assert(TG_ATTN_MERGE_MAX == 16, "one row of 16 lanes per head");
 			const float M = tg_row16_max(m);
 			const float e = ok ? expf(m - M) : 0.0f;
@@ -181,12 +191,14 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				const int d = tid + i * NT;
 				t[i] = (d < h) ? g.wte_scales[d] * (g.emb_scale * (float)row[d]) : 0.0f;
 			}
+			issue_weights();
 		} else if (PRO == TG_PRO_NORM) {
 #pragma unroll
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
 				t[i] = (d < h) ? g.x[d] : 0.0f;
 			}
+			issue_weights();
 		} else {
 			// modules.hpp:166-168 / 218-219: x = rmsnorm(block_out, post) + residual
 			float p[PER], r[PER], wpo[PER];
@@ -198,6 +210,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				r[i] = ok ? g.x[d] : 0.0f;
 				wpo[i] = ok ? g.w_post[d] : 0.0f;
 			}
+			issue_weights();
 			float ss = 0.0f;
 #pragma unroll
 			for (int i = 0; i < PER; i++) ss = fmaf(p[i], p[i], ss);
