@@ -149,7 +149,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		for (int h = 0; h < 4; h++)
 #pragma unroll
 			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
-				a[h][b] = (b < nb) ? g.part_acc[((size_t)b * 4 + h) * 256 + tid] : 0.0f;
+			{
+				// unconditional load from a clamped index, select afterwards: a load under a branch is waited for
+				// at the end of that branch, which would turn these 64 loads into 64 round trips
+				const int bb = b < nb ? b : 0;
+				const float val = g.part_acc[((size_t)bb * 4 + h) * 256 + tid];
+				a[h][b] = (b < nb) ? val : 0.0f;
+			}
 		issue_weights();
 		if (tid < 4 * TG_ATTN_MERGE_MAX) {
 			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
@@ -179,7 +185,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 #pragma unroll
 		for (int i = 0; i < PER; i++) {
 			const int d = tid + i * NT;
-			wpre[i] = (d < h) ? g.w_pre[d] : 0.0f;
+			const float val = g.w_pre[d < h ? d : h - 1];  // clamped index + select: no branch, no wait per load
+			wpre[i] = (d < h) ? val : 0.0f;
 		}
 		if (PRO == TG_PRO_EMBED) {
 			// ops.hpp:537-568: s[d] * (sqrt(hidden) * q)
@@ -189,14 +196,17 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 #pragma unroll
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
-				t[i] = (d < h) ? g.wte_scales[d] * (g.emb_scale * (float)row[d]) : 0.0f;
+				const int dd = d < h ? d : h - 1;
+				const float val = g.wte_scales[dd] * (g.emb_scale * (float)row[dd]);
+				t[i] = (d < h) ? val : 0.0f;
 			}
 			issue_weights();
 		} else if (PRO == TG_PRO_NORM) {
 #pragma unroll
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
-				t[i] = (d < h) ? g.x[d] : 0.0f;
+				const float val = g.x[d < h ? d : h - 1];
+				t[i] = (d < h) ? val : 0.0f;
 			}
 			issue_weights();
 		} else {
@@ -206,9 +216,11 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
 				const bool ok = d < h;
-				p[i] = ok ? g.pend[d] : 0.0f;
-				r[i] = ok ? g.x[d] : 0.0f;
-				wpo[i] = ok ? g.w_post[d] : 0.0f;
+				const int dd = ok ? d : h - 1;
+				const float pv = g.pend[dd], rv = g.x[dd], wv = g.w_post[dd];
+				p[i] = ok ? pv : 0.0f;
+				r[i] = ok ? rv : 0.0f;
+				wpo[i] = ok ? wv : 0.0f;
 			}
 			issue_weights();
 			float ss = 0.0f;

@@ -52,12 +52,22 @@ __device__ __forceinline__ void tg_prefetch_block(const TgPrefetch &p, int first
 	if (p.ptr == nullptr) return;
 	const int pb = (int)blockIdx.x - first_extra_block;
 	const int x = (int)(blockIdx.x & 7u), q = pb >> 3, Q = p.nblocks >> 3;
-	for (int t = x + 8 * q; t < p.ntiles; t += 8 * Q) {
-		const int8_t *sl = p.ptr + (size_t)t * p.slab;
-		for (uint32_t off = threadIdx.x * 128u; off < p.slab; off += 256u * 128u) {
-			const int v = *(const int *)(sl + off);  // one dword per 128-byte line brings the line in
-			asm volatile("" ::"v"(v));               // the value is not needed, the load is
+	// this workgroup's tiles are t = x + 8 q + 8 Q j; their 128-byte lines are walked as one flat index so that
+	// narrow slabs (a few KB) still keep all 256 lanes busy; one dword per line brings the line in
+	const int first = x + 8 * q, stride = 8 * Q;
+	if (first >= p.ntiles) return;
+	const int mytiles = (p.ntiles - first + stride - 1) / stride;
+	const uint32_t lps = p.slab >> 7, total = (uint32_t)mytiles * lps;
+	for (uint32_t i0 = threadIdx.x; i0 < total; i0 += 4u * 256u) {
+		int sink = 0;
+#pragma unroll
+		for (uint32_t k = 0; k < 4; k++) {  // four loads in flight per lane: unconditional (clamped), consumed together
+			uint32_t i = i0 + k * 256u;
+			i = i < total ? i : i0;
+			const uint32_t j = i / lps, line = i - j * lps;
+			sink += *(const int *)(p.ptr + (size_t)(first + (int)j * stride) * p.slab + (size_t)line * 128u);
 		}
+		asm volatile("" ::"v"(sink));  // the values are not needed, the loads are
 	}
 }
 
