@@ -101,18 +101,23 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: thread = output dim.
 	float4 kpre[PRE / 16][4];
 	float vpre[PRE];
+	// Rows are addressed as base + constant * row so that the 40 loads cost no per-load address arithmetic; rows
+	// past the chunk (and slot `cur`, which workgroup 0 rewrites below) are fetched and ignored: every row index is
+	// clamped into the cache, whose max_pos rows are all allocated.
+	{
+		const int lim = a.max_pos - 1 - k0;  // >= 0: last row of the cache, relative to the chunk
+		const float *kbase = a.kc + (size_t)k0 * HD + sl * 4;
+		const float *vbase = a.vc + (size_t)k0 * HD + tid;
 #pragma unroll
-	for (int p = 0; p < PRE / 16; p++) {
-		const int jj = 16 * p + w * 4 + sub;
-		const int j = k0 + (jj < n ? jj : 0);
-		const float *kr = a.kc + (size_t)(j == cur ? k0 : j) * HD;  // slot `cur` is replaced below; any valid row will do
+		for (int p = 0; p < PRE / 16; p++) {
+			int jj = 16 * p + w * 4 + sub;
+			jj = jj < lim ? jj : lim;
+			const float *kr = kbase + (size_t)jj * HD;
 #pragma unroll
-		for (int i = 0; i < 4; i++) kpre[p][i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
-	}
+			for (int i = 0; i < 4; i++) kpre[p][i] = *reinterpret_cast<const float4 *>(kr + i * 64);
+		}
 #pragma unroll
-	for (int u = 0; u < PRE; u++) {
-		const int j = k0 + (u < n ? u : 0);
-		vpre[u] = a.vc[(size_t)(j == cur ? k0 : j) * HD + tid];
+		for (int u = 0; u < PRE; u++) vpre[u] = vbase[(size_t)(u < lim ? u : lim) * HD];
 	}
 
 	// q heads: one wave each; k: wave 0 again
