@@ -138,7 +138,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		const int pos = g.host_pos >= 0 ? g.host_pos : g.pos[0];
 		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
 		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
-		float a[4][TG_ATTN_MERGE_MAX];
+		// wave w merges head w; a lane owns 4 consecutive dims: 16 loads of 16 bytes instead of 64 of 4
+		f32x4 a[TG_ATTN_MERGE_MAX];
 		float m = -INFINITY, l = 0.0f;
 		if (tid < 4 * TG_ATTN_MERGE_MAX && (tid % TG_ATTN_MERGE_MAX) < nb) {
 			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
@@ -146,16 +147,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			l = g.part_ml[((size_t)b * 4 + h) * 2 + 1];
 		}
 #pragma unroll
-		for (int h = 0; h < 4; h++)
-#pragma unroll
-			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++)
-			{
-				// unconditional load from a clamped index, select afterwards: a load under a branch is waited for
-				// at the end of that branch, which would turn these 64 loads into 64 round trips
-				const int bb = b < nb ? b : 0;
-				const float val = g.part_acc[((size_t)bb * 4 + h) * 256 + tid];
-				a[h][b] = (b < nb) ? val : 0.0f;
-			}
+		for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) {
+			// unconditional load from a clamped index, select afterwards: a load under a branch is waited for
+			// at the end of that branch, which would turn these loads into as many round trips
+			const int bb = b < nb ? b : 0;
+			const f32x4 val = *reinterpret_cast<const f32x4 *>(g.part_acc + ((size_t)bb * 4 + w) * 256 + 4 * lane);
+			a[b] = (b < nb) ? val : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+		}
 		issue_weights();
 		if (tid < 4 * TG_ATTN_MERGE_MAX) {
 			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
@@ -169,12 +167,15 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			wgt[h][b] = e / L;
 		}
 		__syncthreads();
+		{
+			f32x4 o = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-		for (int h = 0; h < 4; h++) {
-			float o = 0.0f;
+			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) {
+				const float wb = wgt[w][b];
 #pragma unroll
-			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) o = fmaf(a[h][b], wgt[h][b], o);
-			xs[h * 256 + tid] = o;
+				for (int e = 0; e < 4; e++) o[e] = fmaf(a[b][e], wb, o[e]);
+			}
+			*reinterpret_cast<f32x4 *>(&xs[w * 256 + 4 * lane]) = o;
 		}
 		__syncthreads();
 	} else if (PRO != TG_PRO_PLAIN) {
@@ -387,10 +388,21 @@ __global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, con
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	float bv = -INFINITY;
 	int bi = 0x7fffffff;
-	for (int i = tid; i < n; i += NT) {
-		const float ov = blk_val[i];
-		const int oi = blk_idx[i];
-		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+	// all loads first (clamped indices, no branches), then the comparisons: one memory round trip instead of one per pass
+	for (int i0 = 0; i0 < n; i0 += 8 * NT) {
+		float ovs[8];
+		int ois[8];
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			const int i = i0 + u * NT + tid, ic = i < n ? i : n - 1;
+			ovs[u] = blk_val[ic];
+			ois[u] = blk_idx[ic];
+		}
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			const bool in = i0 + u * NT + tid < n;
+			if (in && (ovs[u] > bv || (ovs[u] == bv && ois[u] < bi))) { bv = ovs[u]; bi = ois[u]; }
+		}
 	}
 #define TG_STEP(O)                                                      \
 	{                                                                   \
