@@ -71,8 +71,9 @@ constexpr int PRE = 32;
 __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) {
 	__shared__ __attribute__((aligned(16))) float qs[NH][HD];
 	__shared__ __attribute__((aligned(16))) float knew[HD];
-	__shared__ float vnew[HD];
+	__shared__ __attribute__((aligned(16))) float vnew[HD];
 	__shared__ __attribute__((aligned(16))) float sc[NH][MAXCHUNK];
+	__shared__ __attribute__((aligned(16))) float pv[ANT / 64][NH][HD];  // per-wave partial outputs of the first PRE keys
 	__shared__ float s_m[NH], s_l[NH];
 
 	if ((int)blockIdx.x >= a.nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
@@ -98,16 +99,16 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	if (w == 0) head_load(kin, a.qkv + NH * HD, a.rms_k, cs, sn, lane);
 	const float vnew_r = a.qkv[NH * HD + HD + tid];
 	// Cache rows of the first PRE keys of this chunk: they depend on nothing computed here.
-	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: thread = output dim.
+	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: wave w takes keys 8w .. 8w+7, a lane 4 dims.
 	float4 kpre[PRE / 16][4];
-	float vpre[PRE];
+	float4 vpre[PRE / 4];
 	// Rows are addressed as base + constant * row so that the 40 loads cost no per-load address arithmetic; rows
 	// past the chunk (and slot `cur`, which workgroup 0 rewrites below) are fetched and ignored: every row index is
 	// clamped into the cache, whose max_pos rows are all allocated.
 	{
 		const int lim = a.max_pos - 1 - k0;  // >= 0: last row of the cache, relative to the chunk
 		const float *kbase = a.kc + (size_t)k0 * HD + sl * 4;
-		const float *vbase = a.vc + (size_t)k0 * HD + tid;
+		const float *vbase = a.vc + (size_t)k0 * HD + 4 * lane;
 #pragma unroll
 		for (int p = 0; p < PRE / 16; p++) {
 			int jj = 16 * p + w * 4 + sub;
@@ -117,7 +118,10 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 			for (int i = 0; i < 4; i++) kpre[p][i] = *reinterpret_cast<const float4 *>(kr + i * 64);
 		}
 #pragma unroll
-		for (int u = 0; u < PRE; u++) vpre[u] = vbase[(size_t)(u < lim ? u : lim) * HD];
+		for (int u = 0; u < PRE / 4; u++) {
+			const int jj = (PRE / 4) * w + u;
+			vpre[u] = *reinterpret_cast<const float4 *>(vbase + (size_t)(jj < lim ? jj : lim) * HD);
+		}
 	}
 
 	// q heads: one wave each; k: wave 0 again
@@ -198,25 +202,43 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const TgAttnDecode a) 
 	}
 	__syncthreads();
 
-	// P.V: thread = output dim, 4 heads
-	float acc[NH] = {0.0f, 0.0f, 0.0f, 0.0f};
+	// P.V of the first PRE keys: wave w owns keys 8w..8w+7, lane = 4 consecutive dims; summed over the waves via LDS
+	{
+		float4 part[NH];
 #pragma unroll
-	for (int u4 = 0; u4 < PRE; u4 += 4) {
-		if (u4 < n) {  // entries past n are read with the group but not used
-			float4 p[NH];
+		for (int h = 0; h < NH; h++) part[h] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+		const int ub = (PRE / 4) * w;
+		if (ub < n) {  // entries of sc past n are read with the group but not used
+			float4 p[NH][2];
 #pragma unroll
-			for (int h = 0; h < NH; h++) p[h] = *reinterpret_cast<const float4 *>(&sc[h][u4]);
+			for (int h = 0; h < NH; h++) {
+				p[h][0] = *reinterpret_cast<const float4 *>(&sc[h][ub]);
+				p[h][1] = *reinterpret_cast<const float4 *>(&sc[h][ub + 4]);
+			}
+			const float4 vn = *reinterpret_cast<const float4 *>(&vnew[4 * lane]);
 #pragma unroll
-			for (int e = 0; e < 4; e++) {
-				const int u = u4 + e;
-				if (u < n) {
-					const float vv = (k0 + u == cur) ? vnew[tid] : vpre[u];
+			for (int u = 0; u < PRE / 4; u++) {
+				if (ub + u < n) {
+					const float4 vv = (k0 + ub + u == cur) ? vn : vpre[u];
 #pragma unroll
-					for (int h = 0; h < NH; h++) acc[h] = fmaf(reinterpret_cast<const float *>(&p[h])[e], vv, acc[h]);
+					for (int h = 0; h < NH; h++) {
+						const float ph = reinterpret_cast<const float *>(&p[h][u >> 2])[u & 3];
+						part[h].x = fmaf(ph, vv.x, part[h].x);
+						part[h].y = fmaf(ph, vv.y, part[h].y);
+						part[h].z = fmaf(ph, vv.z, part[h].z);
+						part[h].w = fmaf(ph, vv.w, part[h].w);
+					}
 				}
 			}
 		}
+#pragma unroll
+		for (int h = 0; h < NH; h++) *reinterpret_cast<float4 *>(&pv[w][h][4 * lane]) = part[h];
 	}
+	__syncthreads();
+	// from here on: thread = output dim, 4 heads
+	float acc[NH];
+#pragma unroll
+	for (int h = 0; h < NH; h++) acc[h] = (pv[0][h][tid] + pv[1][h][tid]) + (pv[2][h][tid] + pv[3][h][tid]);
 	for (int j0 = PRE; j0 < n; j0 += 8) {
 		float vv[8];
 #pragma unroll
