@@ -16,7 +16,9 @@ LIB_PATH = os.path.join(HERE, "libtinygemma_hip.so")
 CSRC = os.path.join(HERE, "csrc")
 SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
+               # leading scalar kernel arguments are preloaded into SGPRs by the dispatcher (no s_load round trip)
+               "-mllvm", "-amdgpu-kernarg-preload-count=14"]
 
 c_f32p = C.POINTER(C.c_float)
 c_i8p = C.POINTER(C.c_int8)
