@@ -27,6 +27,7 @@ namespace {
 constexpr int NT = 256;     // threads per workgroup (4 waves)
 constexpr int NWAVE = 4;
 constexpr int DEPTH = 8;    // 16-byte weight loads in flight per lane
+constexpr int LUT_LDS = 1024;  // GeLU tables up to this size are staged in LDS (one 16-byte load per lane)
 constexpr uint32_t STEP_BYTES = NT * 16u;  // the workgroup reads 4 KiB of its slab per step
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -85,6 +86,7 @@ __device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const f32x4 x
 template <int PRO, int EPI>
 __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
+	__shared__ __attribute__((aligned(16))) float lut_s[(EPI == TG_EPI_GEGLU) ? LUT_LDS : 4];  // GeLU table of the GeGLU epilogue
 	__shared__ __attribute__((aligned(16))) float red2[2][NWAVE][TG_CT];  // double buffered across the tile loop
 	__shared__ float sred[NWAVE];
 	__shared__ float wgt[4][TG_ATTN_MERGE_MAX];
@@ -116,7 +118,20 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	// every load issued before it, and the prologue must not wait for 32 KB of weights to see its inputs.
 	i32x4 v[DEPTH];
 	f32x4 xq[DEPTH];
+	// Column scales of a tile (and, for the GeGLU epilogue, the GeLU table) are requested together with its first
+	// weights: fetched in the epilogue they would add one, for the table two, memory round trips at the end.
+	float sc_a = 0.0f, sc_b = 0.0f;  // thread tid < C: scale of column tid (GeGLU: up column tid and gate column tid)
+	auto load_scales = [&](int t) {
+		const int ncol = (EPI == TG_EPI_GEGLU) ? (C >> 1) : C;
+		const int c = tid < ncol ? tid : 0;
+		sc_a = g.scales[t * C + c];
+		if (EPI == TG_EPI_GEGLU) sc_b = g.scales[t * C + (C >> 1) + c];
+	};
+	f32x4 lutv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+	const bool lut_in_lds = (EPI == TG_EPI_GEGLU) && g.lut_size <= LUT_LDS && (g.lut_size & 3) == 0;
 	auto issue_weights = [&]() {
+		load_scales(tile);
+		if (lut_in_lds) lutv = *reinterpret_cast<const f32x4 *>(g.lut + (4 * tid < g.lut_size ? 4 * tid : 0));
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
 			v[u] = i32x4{0, 0, 0, 0};
@@ -253,6 +268,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		__syncthreads();
 	}
 
+	if (lut_in_lds && 4 * tid < g.lut_size) *reinterpret_cast<f32x4 *>(&lut_s[4 * tid]) = lutv;  // visible after the barrier that precedes the epilogue
 	// A workgroup walks tiles blockIdx.x, blockIdx.x + nmain, ...: the prologue above is paid once.
 	const int xlast = g.K - 4;
 	for (int it = 0;; it++) {
@@ -294,7 +310,9 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	const int cur = tile;
 	tile += g.nmain;
 	const bool more = tile < g.ntiles;
+	const float sc_cur_a = sc_a, sc_cur_b = sc_b;
 	if (more) {
+		load_scales(tile);
 		rw = make_rsrc(g.W + (size_t)tile * slab, slab);
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
@@ -321,7 +339,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		if (tid < C) {
 			const int col = cur * C + tid;
 			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
-			g.y[col] = sum * g.scales[col];
+			g.y[col] = sum * sc_cur_a;
 		}
 	} else if (EPI == TG_EPI_GEGLU) {
 		// modules.hpp:211-215: gelu(gate) * up; the tile holds C/2 up columns, then the same C/2 gate columns
@@ -329,9 +347,9 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		if (tid < C2) {
 			const float su = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
 			const float sg = (red[0][tid + C2] + red[1][tid + C2]) + (red[2][tid + C2] + red[3][tid + C2]);
-			const float up = su * g.scales[cur * C + tid];
-			const float gate = sg * g.scales[cur * C + C2 + tid];
-			g.y[cur * C2 + tid] = gelu_lut(gate, g.lut, g.gmin, g.geps, g.lut_size) * up;
+			const float up = su * sc_cur_a;
+			const float gate = sg * sc_cur_b;
+			g.y[cur * C2 + tid] = gelu_lut(gate, lut_in_lds ? lut_s : g.lut, g.gmin, g.geps, g.lut_size) * up;
 		}
 	} else {
 		// TG_EPI_LOGITS: logits + first stage of the greedy argmax
@@ -341,7 +359,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		if (tid < C) {
 			const int col = cur * C + tid;
 			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
-			const float val = sum * g.scales[col];
+			const float val = sum * sc_cur_a;
 			if (g.y != nullptr) g.y[col] = val;
 			if (val > bv) { bv = val; bi = col; }
 		}
