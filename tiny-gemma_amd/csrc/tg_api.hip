@@ -179,9 +179,9 @@ TgGemv gemv_base(const PackedMat &p) {
 
 // C[m][N] = scales * (A[m][K] . W) through the selected GEMM; apack/rowscale are scratch for the MFMA path.
 void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
-                 int lut_size, int8_t *apack, float *rowscale) {
+                 int lut_size, int8_t *apack, float *rowscale, bool prepacked = false) {
 	if (g_gemm_mfma) {
-		tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, g_stream);
+		if (!prepacked) tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, g_stream);  // else the producer wrote the planes
 		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, g_stream);
 	} else {
 		(void)lda;  // the exact kernel reads dense rows (lda == K at every call site)
@@ -1141,12 +1141,14 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	tg_launch_embed_rows(x, d_ids, n, m->wte, m->wte_scales, h, c.n_vocab, g_stream);
 	TG_TRY(tap(0));
 	// xn = rmsnorm(x, attn_pre of layer 0)
-	tg_launch_norm_rows(xn, x, m->L[0].apre, nullptr, nullptr, nullptr, n, h, g_stream);
+	// With the int8 MFMA GEMM the norm writes the GEMM's digit planes itself and the fp32 row is not stored.
+	const bool pk = g_gemm_mfma;
+	tg_launch_norm_rows(pk ? nullptr : xn, x, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale, g_stream);
 	for (int l = 0; l < L; l++) {
 		const LayerDev &Ld = m->L[(size_t)l];
 		const int mp = s->max_pos[(size_t)l];
 		// Q|K|V (modules.hpp:106-108)
-		launch_gemm(qkv, xn, h, Ld.qkv, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
+		launch_gemm(qkv, xn, h, Ld.qkv, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk);
 		// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
 		tg_launch_qk_norm_rope_rows(qkv, qkv + qo, qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
@@ -1156,14 +1158,17 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		// O (modules.hpp:127-128)
 		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
-		tg_launch_norm_rows(xn, t, Ld.mpre, Ld.apost, x, x, n, h, g_stream);
+		tg_launch_norm_rows(pk ? nullptr : xn, t, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
 		TG_TRY(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
-		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale);
+		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk);
 		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
-		tg_launch_norm_rows(xn, t, next_pre, Ld.mpost, x, x, n, h, g_stream);
+		// the last layer's final norm feeds the LM head GEMV, which reads the fp32 row
+		const bool last = l + 1 == L;
+		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
+		                    g_stream);
 		TG_TRY(tap(2 * l + 2));
 	}
 	// LM head on the last position only (modules.hpp:232-240): xn already holds rmsnorm(x, RMSw)

@@ -42,7 +42,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GNT = 256;     // threads per workgroup: 4 waves, each owns 32 rows x 128 columns
 constexpr int KSTAGE = 64;   // rows of K per LDS stage
-constexpr int QBITS = 22;    // row maxima are scaled into [2^(QBITS-1), 2^QBITS)
 constexpr int LUT_LDS_MAX = 4096;  // GeLU tables up to this many entries are staged in LDS (Bs holds 16 KB)
 
 // ginv != 0: the table step is a power of two and ginv its exact reciprocal, so the product equals the quotient
@@ -67,13 +66,8 @@ __global__ __launch_bounds__(GNT) void row_scale_kernel(const float *A, int lda,
 	}
 	amax = tg_wave_max(amax);
 	if (lane == 0) {
-		float s = 1.0f, r = 1.0f;
-		if (amax > 0.0f && amax < INFINITY) {
-			int e;
-			(void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
-			s = ldexpf(1.0f, QBITS - e);
-			r = ldexpf(1.0f, e - QBITS);
-		}
+		float s, r;
+		tg_row_factors(amax, s, r);
 		mul[m] = s;
 		inv[m] = r;
 	}
@@ -87,30 +81,17 @@ __global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda
 	const int k0 = blockIdx.y * 128 + 16 * kq;
 	i32x4 pl[3] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
 	if (m < M) {
-		const float s = mul[m];
 		const f32x4 *src = reinterpret_cast<const f32x4 *>(A + (size_t)m * lda + k0);
+		float v[16];
 #pragma unroll
 		for (int q = 0; q < 4; q++) {
 			const f32x4 a = src[q];
-			unsigned d0 = 0, d1 = 0, d2 = 0;
 #pragma unroll
-			for (int i = 0; i < 4; i++) {
-				const int xi = (int)rintf(a[i] * s);
-				const int a0 = (xi << 24) >> 24;
-				const int r1 = (xi - a0) >> 8;
-				const int a1 = (r1 << 24) >> 24;
-				const int a2 = (r1 - a1) >> 8;
-				d0 |= (unsigned)(a0 & 255) << (8 * i);
-				d1 |= (unsigned)(a1 & 255) << (8 * i);
-				d2 |= (unsigned)(a2 & 255) << (8 * i);
-			}
-			pl[0][q] = (int)d0;
-			pl[1][q] = (int)d1;
-			pl[2][q] = (int)d2;
+			for (int i = 0; i < 4; i++) v[4 * q + i] = a[i];
 		}
+		tg_quant16(v, mul[m], pl);
 	}
-	const int kb = k0 >> 5, hb = (k0 >> 4) & 1;
-	i32x4 *dst = reinterpret_cast<i32x4 *>(Apack) + ((size_t)mtile * (size_t)(K >> 5) + kb) * 3 * 64 + (r + 32 * hb);
+	i32x4 *dst = tg_plane_dst(Apack, m, k0, K);
 #pragma unroll
 	for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
 }

@@ -154,8 +154,10 @@ void tg_launch_minp(const float *logits, int n, float minp, float temp, const fl
 void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,
                           hipStream_t s);
 // out = rmsnorm(in, w); if resid != null first in = rmsnorm(in, w_post) + resid is formed and stored to resid_out
+// apack/rowfac non-null: the normalised rows are also (out == nullptr: only) written as digit planes + row factors for
+// tg_launch_gemm_mfma (rowfac as tg_launch_quant_pack lays it out for S rows)
 void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
-                         int S, int dim, hipStream_t s);
+                         int S, int dim, int8_t *apack, float *rowfac, hipStream_t s);
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
                                  const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
                                  hipStream_t s);
@@ -248,6 +250,51 @@ __device__ __forceinline__ float tg_row16_max(float v) {
 	v = fmaxf(v, tg_red_partner<2>(v));
 	v = fmaxf(v, tg_red_partner<1>(v));
 	return v;
+}
+#endif
+
+// ---- activation quantisation of the int8 MFMA GEMM (shared by the stand-alone pre-pass and fused producers) ----
+// A row is scaled by a power of two so that its largest magnitude lies in [2^21, 2^22), rounded to an integer and
+// written as three signed base-256 digits (int8 planes), 16 consecutive k per lane, in MFMA operand order:
+//   planes [tile of 32 rows][K/32][3][64 lanes][16 bytes], lane = row % 32 + 32 * ((k % 32) / 16).
+#if defined(__HIPCC__)
+constexpr int TG_QBITS = 22;
+__device__ __forceinline__ void tg_row_factors(float amax, float &mul, float &inv) {
+	mul = 1.0f;
+	inv = 1.0f;
+	if (amax > 0.0f && amax < INFINITY) {
+		int e;
+		(void)frexpf(amax, &e);  // amax = f * 2^e, f in [0.5, 1)
+		mul = ldexpf(1.0f, TG_QBITS - e);
+		inv = ldexpf(1.0f, e - TG_QBITS);
+	}
+}
+typedef int tg_i32x4 __attribute__((ext_vector_type(4)));
+// v[16] consecutive k of one row -> the lane's 16 bytes of each plane
+__device__ __forceinline__ void tg_quant16(const float *v, float mul, tg_i32x4 pl[3]) {
+#pragma unroll
+	for (int q = 0; q < 4; q++) {
+		unsigned d0 = 0, d1 = 0, d2 = 0;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int xi = (int)rintf(v[4 * q + i] * mul);
+			const int a0 = (xi << 24) >> 24;
+			const int r1 = (xi - a0) >> 8;
+			const int a1 = (r1 << 24) >> 24;
+			const int a2 = (r1 - a1) >> 8;
+			d0 |= (unsigned)(a0 & 255) << (8 * i);
+			d1 |= (unsigned)(a1 & 255) << (8 * i);
+			d2 |= (unsigned)(a2 & 255) << (8 * i);
+		}
+		pl[0][q] = (int)d0;
+		pl[1][q] = (int)d1;
+		pl[2][q] = (int)d2;
+	}
+}
+// where the 16 bytes of (row m, k0 = multiple of 16) of plane 0 go; planes are 64 pieces apart
+__device__ __forceinline__ tg_i32x4 *tg_plane_dst(int8_t *apack, int m, int k0, int K) {
+	const int kb = k0 >> 5, hb = (k0 >> 4) & 1;
+	return reinterpret_cast<tg_i32x4 *>(apack) + ((size_t)(m >> 5) * (size_t)(K >> 5) + kb) * 3 * 64 + ((m & 31) + 32 * hb);
 }
 #endif
 

@@ -42,9 +42,21 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 	for (int d = threadIdx.x; d < hidden; d += RNT) x[(size_t)s * hidden + d] = scales[d] * (emb_scale * (float)row[d]);
 }
 
+__device__ __forceinline__ float bmax(float v, float *sred) {
+	v = tg_wave_max(v);
+	__syncthreads();
+	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
+	__syncthreads();
+	return fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
+}
+
+// One workgroup per row: [post-norm + residual (+ residual out)] + pre-norm.  The normalised row goes out as fp32
+// (out != nullptr) and/or straight as the int8 digit planes + row factors of the MFMA GEMM that consumes it
+// (apack != nullptr): the same bits the stand-alone quantising pre-pass would produce from the fp32 row.
 __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *w_pre, const float *w_post,
-                                                        const float *resid, float *resid_out, int dim) {
-	__shared__ float xs[1152];
+                                                        const float *resid, float *resid_out, int dim, int8_t *apack, float *rowfac,
+                                                        int Mpad) {
+	__shared__ __attribute__((aligned(16))) float xs[1152];
 	__shared__ float sred[4];
 	const int s = blockIdx.x, tid = threadIdx.x;
 	const float eps = 1e-06f;
@@ -67,9 +79,31 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 		}
 		ss = bsum(s2, sred);
 	}
-	if (out != nullptr) {
+	if (out != nullptr || apack != nullptr) {
 		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
-		for (int d = tid; d < dim; d += RNT) out[(size_t)s * dim + d] = (xs[d] * irms) * (w_pre[d] + 1.0f);
+		float amax = 0.0f;
+		for (int d = tid; d < dim; d += RNT) {
+			const float y = (xs[d] * irms) * (w_pre[d] + 1.0f);
+			if (out != nullptr) out[(size_t)s * dim + d] = y;
+			xs[d] = y;  // each thread rewrites only what it read
+			amax = fmaxf(amax, fabsf(y));
+		}
+		if (apack != nullptr) {
+			amax = bmax(amax, sred);  // its barriers also publish xs
+			float mul, inv;
+			tg_row_factors(amax, mul, inv);
+			if (tid == 0) {
+				rowfac[s] = mul;
+				rowfac[Mpad + s] = inv;
+			}
+			for (int g = tid; g < (dim >> 4); g += RNT) {
+				tg_i32x4 pl[3];
+				tg_quant16(&xs[16 * g], mul, pl);
+				tg_i32x4 *dst = tg_plane_dst(apack, s, 16 * g, dim);
+#pragma unroll
+				for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
+			}
+		}
 	}
 }
 
@@ -170,8 +204,10 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 }
 
 void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
-                         int S, int dim, hipStream_t s) {
-	hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, out, in, w_pre, w_post, resid, resid_out, dim);
+                         int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
+	const int Mpad = (int)tg_gemm_mfma_rows(S);
+	hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, out, in, w_pre, w_post, resid, resid_out, dim, apack, rowfac,
+	                   Mpad);
 }
 
 // Wp/scales: GEMV tiling of the matrix (ntiles tiles of Ct columns); C gets ntiles * Ct columns, or half of that for GEGLU
