@@ -14,7 +14,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libtinygemma_hip.so")
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip"]
+SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip", "tg_repack.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
                # leading scalar kernel arguments are preloaded into SGPRs by the dispatcher (no s_load round trip)

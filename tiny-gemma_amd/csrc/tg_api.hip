@@ -1,10 +1,13 @@
 // C ABI of libtinygemma_hip.so (declared in include/tinygemma_hip.h): library state, weight
 // upload / re-tiling, sessions, and the kernel sequences of forward_prefill / forward_decode.
 
+#include <fcntl.h>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <chrono>
@@ -62,98 +65,59 @@ int choose_tile_cols(int N, int min_c) {
 	return C;
 }
 
-// host: [K][N] row-major -> tiles of C columns, each [K/4][C][4]
-void pack_host(int8_t *dst, const int8_t *src, int K, int N, int C) {
-	const int kgs = K / 4;
-	for (int t = 0; t < N / C; t++) {
-		for (int kg = 0; kg < kgs; kg++) {
-			const int8_t *r0 = src + (size_t)(4 * kg) * N + (size_t)t * C;
-			const int8_t *r1 = r0 + N, *r2 = r1 + N, *r3 = r2 + N;
-			int8_t *d = dst + ((size_t)t * kgs + kg) * C * 4;
-			for (int c = 0; c < C; c++) {
-				d[4 * c + 0] = r0[c];
-				d[4 * c + 1] = r1[c];
-				d[4 * c + 2] = r2[c];
-				d[4 * c + 3] = r3[c];
-			}
-		}
-	}
+TgColMap plain_map(const int8_t *W, const float *scales, int N) {
+	TgColMap m;
+	memset(&m, 0, sizeof(m));
+	m.src[0] = W;
+	m.scales[0] = scales;
+	m.n[0] = N;
+	return m;
 }
 
-// host: [K][N] row-major -> tiles of 128 columns, each [K/16][128][16 consecutive k] (MFMA B-operand order)
-void pack_host_mfma(int8_t *dst, const int8_t *src, int K, int N) {
-	const int k16s = K / 16;
-	for (int t = 0; t < N / TG_CT; t++) {
-		for (int kb = 0; kb < k16s; kb++) {
-			int8_t *d = dst + ((size_t)t * k16s + kb) * TG_CT * 16;
-			for (int j = 0; j < 16; j++) {
-				const int8_t *r = src + (size_t)(16 * kb + j) * N + (size_t)t * TG_CT;
-				for (int c = 0; c < TG_CT; c++) d[16 * c + j] = r[c];
-			}
-		}
-	}
-}
+void free_packed(PackedMat *p);
 
-// C > 0: GEMV tiling of C columns; C = 0: MFMA tiling
-int upload_tiles(int8_t **Wd, float **sd, const int8_t *host_rowmajor, const float *host_scales, int K, int N, int C) {
-	std::vector<int8_t> tmp((size_t)K * N);
-	if (C > 0) pack_host(tmp.data(), host_rowmajor, K, N, C);
-	else pack_host_mfma(tmp.data(), host_rowmajor, K, N);
-	TG_HIP(hipMalloc((void **)Wd, (size_t)K * N));
-	TG_HIP(hipMalloc((void **)sd, (size_t)N * sizeof(float)));
-	TG_HIP(hipMemcpy(*Wd, tmp.data(), (size_t)K * N, hipMemcpyHostToDevice));
-	TG_HIP(hipMemcpy(*sd, host_scales, (size_t)N * sizeof(float), hipMemcpyHostToDevice));
-	return TG_OK;
-}
-
-// Plain matrix [K][N] (reference layout) -> GEMV tiles, and GEMM tiles if with_gemm.
-int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_scales, int K, int N, bool with_gemm) {
+// Builds the device layouts of one matrix from sources already on the device (reference layout; see TgColMap):
+// GEMV tiles always, MFMA tiles if with_gemm.  min_c: smallest GEMV tile width allowed.  For an interleaved
+// map (up|gate) `m.half` is ignored on entry and set per layout: half a tile of each.
+int build_packed(PackedMat *p, TgColMap m, int K, int N, int min_c, bool with_gemm) {
+	const bool interleave = m.half != 0;
 	p->K = K;
 	p->N = N;
-	p->C = choose_tile_cols(N, 4);
+	p->C = choose_tile_cols(N, min_c);
 	p->lc_shift = 0;
 	while ((4 << p->lc_shift) < p->C) p->lc_shift++;
 	p->ntiles = N / p->C;
-	if (int rc = upload_tiles(&p->W, &p->scales, host_rowmajor, host_scales, K, N, p->C)) return rc;
+	TG_HIP(hipMalloc((void **)&p->W, (size_t)K * N));
+	TG_HIP(hipMalloc((void **)&p->scales, (size_t)N * sizeof(float)));
+	if (interleave) m.half = p->C / 2;
+	tg_launch_retile_gemv(p->W, p->scales, m, K, N, p->C, g_stream);
 	if (with_gemm) {
 		p->ntiles_g = N / TG_CT;
-		if (int rc = upload_tiles(&p->Wg, &p->scales_g, host_rowmajor, host_scales, K, N, 0)) return rc;
+		TG_HIP(hipMalloc((void **)&p->Wg, (size_t)K * N));
+		TG_HIP(hipMalloc((void **)&p->scales_g, (size_t)N * sizeof(float)));
+		if (interleave) m.half = TG_CT / 2;
+		tg_launch_retile_mfma(p->Wg, p->scales_g, m, K, N, g_stream);
 	}
+	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
 
-// up [K][f] and gate [K][f] -> one matrix of 2f virtual columns whose tiles of C columns hold
-// C/2 up columns followed by the same C/2 gate columns (so gelu(gate)*up never leaves a workgroup).
-void fuse_up_gate(std::vector<int8_t> &cat, std::vector<float> &catsc, const int8_t *up, const float *ups, const int8_t *gate,
-                  const float *gates, int K, int f, int C) {
-	const int C2 = C / 2;
-	cat.assign((size_t)K * 2 * f, 0);
-	catsc.assign((size_t)2 * f, 0.0f);
-	for (int t = 0; t < f / C2; t++) {
-		for (int r = 0; r < K; r++) {
-			memcpy(&cat[(size_t)r * 2 * f + (size_t)t * C], &up[(size_t)r * f + (size_t)t * C2], (size_t)C2);
-			memcpy(&cat[(size_t)r * 2 * f + (size_t)t * C + C2], &gate[(size_t)r * f + (size_t)t * C2], (size_t)C2);
-		}
-		memcpy(&catsc[(size_t)t * C], &ups[(size_t)t * C2], sizeof(float) * (size_t)C2);
-		memcpy(&catsc[(size_t)t * C + C2], &gates[(size_t)t * C2], sizeof(float) * (size_t)C2);
-	}
-}
-
-int upload_up_gate(PackedMat *p, const int8_t *up, const float *ups, const int8_t *gate, const float *gates, int K, int f) {
-	std::vector<int8_t> cat;
-	std::vector<float> catsc;
-	p->K = K;
-	p->N = 2 * f;
-	p->C = choose_tile_cols(2 * f, 8);
-	p->lc_shift = 0;
-	while ((4 << p->lc_shift) < p->C) p->lc_shift++;
-	p->ntiles = p->N / p->C;
-	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, p->C);
-	if (int rc = upload_tiles(&p->W, &p->scales, cat.data(), catsc.data(), K, 2 * f, p->C)) return rc;
-	// MFMA layout: 128-column tiles of 64 up columns followed by the same 64 gate columns
-	p->ntiles_g = p->N / TG_CT;
-	fuse_up_gate(cat, catsc, up, ups, gate, gates, K, f, TG_CT);
-	return upload_tiles(&p->Wg, &p->scales_g, cat.data(), catsc.data(), K, 2 * f, 0);
+// Plain host matrix [K][N] (reference layout): staged on the device, then re-tiled there.
+int upload_packed(PackedMat *p, const int8_t *host_rowmajor, const float *host_scales, int K, int N, bool with_gemm) {
+	int8_t *raw = nullptr;
+	float *rs = nullptr;
+	auto done = [&](int rc) {
+		(void)hipStreamSynchronize(g_stream);
+		if (raw) (void)hipFree(raw);
+		if (rs) (void)hipFree(rs);
+		return rc;
+	};
+	if (hipMalloc((void **)&raw, (size_t)K * N) != hipSuccess || hipMalloc((void **)&rs, (size_t)N * sizeof(float)) != hipSuccess)
+		return done(tg_fail(TG_ERR_HIP, "hipMalloc of the staging copy failed"));
+	if (hipMemcpyAsync(raw, host_rowmajor, (size_t)K * N, hipMemcpyHostToDevice, g_stream) != hipSuccess ||
+	    hipMemcpyAsync(rs, host_scales, (size_t)N * sizeof(float), hipMemcpyHostToDevice, g_stream) != hipSuccess)
+		return done(tg_fail(TG_ERR_HIP, "upload of the staging copy failed"));
+	return done(build_packed(p, plain_map(raw, rs, N), K, N, 4, with_gemm));
 }
 
 void free_packed(PackedMat *p) {
@@ -534,84 +498,145 @@ void tg_model_destroy(tg_model *m) {
 
 }  // extern "C"
 
-// Walks the flat file in the order of transformer.hpp:122-160 through `rd`.
-template <typename Reader>
-static int load_weights_impl(tg_model *m, Reader rd) {
+// The file goes to the device as it is (the reference layout, transformer.hpp:122-160), in chunks through two
+// pinned staging buffers so that producing a chunk (file read or memcpy) overlaps the DMA of the previous one.
+// fill(dst, off, len) must produce bytes [off, off + len) of the file at dst.
+template <typename Fill>
+static int stage_image(uint8_t *d_raw, size_t n, Fill fill) {
+	constexpr size_t CHUNK = (size_t)32 << 20;
+	void *pin[2] = {nullptr, nullptr};
+	hipEvent_t ev[2] = {nullptr, nullptr};
+	bool used[2] = {false, false};
+	int rc = TG_OK;
+	for (int i = 0; i < 2 && rc == TG_OK; i++) {
+		if (hipHostMalloc(&pin[i], std::min(CHUNK, n), hipHostMallocDefault) != hipSuccess || hipEventCreate(&ev[i]) != hipSuccess)
+			rc = tg_fail(TG_ERR_HIP, "pinned staging buffer allocation failed");
+	}
+	int i = 0;
+	for (size_t off = 0; off < n && rc == TG_OK; off += CHUNK, i ^= 1) {
+		const size_t len = std::min(CHUNK, n - off);
+		if (used[i] && hipEventSynchronize(ev[i]) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipEventSynchronize failed");
+		if (rc == TG_OK) rc = fill(pin[i], off, len);
+		if (rc == TG_OK && (hipMemcpyAsync(d_raw + off, pin[i], len, hipMemcpyHostToDevice, g_stream) != hipSuccess ||
+		                    hipEventRecord(ev[i], g_stream) != hipSuccess))
+			rc = tg_fail(TG_ERR_HIP, "upload of a weight chunk failed");
+		used[i] = true;
+	}
+	(void)hipStreamSynchronize(g_stream);
+	for (int k = 0; k < 2; k++) {
+		if (ev[k]) (void)hipEventDestroy(ev[k]);
+		if (pin[k]) (void)hipHostFree(pin[k]);
+	}
+	return rc;
+}
+
+// Walks the device image of the file in the order of transformer.hpp:122-160 and builds the device layouts
+// with the re-tiling kernels; small fp32 vectors get their own allocations.
+static int build_from_image(tg_model *m, const uint8_t *d_raw) {
 	const tg_config &c = m->cfg;
-	const int h = c.hidden_size, f = c.intermediate_size, V = c.n_vocab, hd = c.head_dim;
-	const int qo = c.n_head * hd, kv = c.n_kv * hd;
-	model_free_weights(m);
-	std::vector<int8_t> buf, buf2, cat;
-	std::vector<float> sc, sc2, catsc, fl;
-	int rc;
-	auto read_i8 = [&](std::vector<int8_t> &v, size_t n) { v.resize(n); return rd(v.data(), n); };
-	auto read_f = [&](std::vector<float> &v, size_t n) { v.resize(n); return rd(v.data(), n * 4); };
-	auto read_dev_f = [&](float **dst, size_t n) -> int {
-		if (int r = read_f(fl, n)) return r;
-		return upload_floats(dst, fl.data(), n);
+	const size_t h = (size_t)c.hidden_size, f = (size_t)c.intermediate_size, V = (size_t)c.n_vocab, hd = (size_t)c.head_dim;
+	const size_t qo = (size_t)c.n_head * hd, kv = (size_t)c.n_kv * hd;
+	size_t off = 0;
+	auto take = [&](size_t bytes) {
+		const uint8_t *p = d_raw + off;
+		off += bytes;
+		return p;
 	};
-	// wte + scales, final norm
-	if ((rc = read_i8(buf, (size_t)V * h))) return rc;
-	TG_HIP(hipMalloc((void **)&m->wte, (size_t)V * h));
-	TG_HIP(hipMemcpy(m->wte, buf.data(), (size_t)V * h, hipMemcpyHostToDevice));
-	if ((rc = read_dev_f(&m->wte_scales, (size_t)h))) return rc;
-	if ((rc = read_dev_f(&m->rmsw, (size_t)h))) return rc;
+	auto take_w = [&](size_t n) { return (const int8_t *)take(n); };
+	auto take_f = [&](size_t n) { return (const float *)take(4 * n); };
+	auto own_f = [&](float **dst, size_t n) -> int {
+		const float *src = take_f(n);
+		TG_HIP(hipMalloc((void **)dst, n * sizeof(float)));
+		TG_HIP(hipMemcpyAsync(*dst, src, n * sizeof(float), hipMemcpyDeviceToDevice, g_stream));
+		return TG_OK;
+	};
+	int rc;
+	// wte stays in the reference layout: its rows are gathered, never streamed
+	const int8_t *wte = take_w(V * h);
+	TG_HIP(hipMalloc((void **)&m->wte, V * h));
+	TG_HIP(hipMemcpyAsync(m->wte, wte, V * h, hipMemcpyDeviceToDevice, g_stream));
+	if ((rc = own_f(&m->wte_scales, h))) return rc;
+	if ((rc = own_f(&m->rmsw, h))) return rc;
 	for (int l = 0; l < c.n_layers; l++) {
 		LayerDev &L = m->L[(size_t)l];
-		// Q | K | V fused along the output dimension: [h][qo + 2 kv]
-		const int nq = qo + 2 * kv;
-		cat.assign((size_t)h * nq, 0);
-		catsc.assign((size_t)nq, 0.0f);
-		int col = 0;
+		// Q | K | V side by side along the output dimension: [h][qo + 2 kv]
+		TgColMap qkv;
+		memset(&qkv, 0, sizeof(qkv));
 		for (int part = 0; part < 3; part++) {
-			const int n = part == 0 ? qo : kv;
-			if ((rc = read_i8(buf, (size_t)h * n))) return rc;
-			if ((rc = read_f(sc, (size_t)n))) return rc;
-			for (int r = 0; r < h; r++) memcpy(&cat[(size_t)r * nq + col], &buf[(size_t)r * n], (size_t)n);
-			memcpy(&catsc[(size_t)col], sc.data(), sizeof(float) * (size_t)n);
-			col += n;
+			const size_t n = part == 0 ? qo : kv;
+			qkv.src[part] = take_w(h * n);
+			qkv.scales[part] = take_f(n);
+			qkv.n[part] = (int)n;
 		}
-		if ((rc = upload_packed(&L.qkv, cat.data(), catsc.data(), h, nq, true))) return rc;
-		// O
-		if ((rc = read_i8(buf, (size_t)qo * h))) return rc;
-		if ((rc = read_f(sc, (size_t)h))) return rc;
-		if ((rc = upload_packed(&L.o, buf.data(), sc.data(), qo, h, true))) return rc;
-		if ((rc = read_dev_f(&L.rms_q, (size_t)hd))) return rc;
-		if ((rc = read_dev_f(&L.rms_k, (size_t)hd))) return rc;
-		if ((rc = read_dev_f(&L.apre, (size_t)h))) return rc;
-		if ((rc = read_dev_f(&L.apost, (size_t)h))) return rc;
-		// up | gate fused tile by tile
-		if ((rc = read_i8(buf, (size_t)h * f))) return rc;
-		if ((rc = read_f(sc, (size_t)f))) return rc;
-		if ((rc = read_i8(buf2, (size_t)h * f))) return rc;
-		if ((rc = read_f(sc2, (size_t)f))) return rc;
-		if ((rc = upload_up_gate(&L.ug, buf.data(), sc.data(), buf2.data(), sc2.data(), h, f))) return rc;
-		// down
-		if ((rc = read_i8(buf, (size_t)f * h))) return rc;
-		if ((rc = read_f(sc, (size_t)h))) return rc;
-		if ((rc = upload_packed(&L.d, buf.data(), sc.data(), f, h, true))) return rc;
-		if ((rc = read_dev_f(&L.mpre, (size_t)h))) return rc;
-		if ((rc = read_dev_f(&L.mpost, (size_t)h))) return rc;
+		if ((rc = build_packed(&L.qkv, qkv, (int)h, (int)(qo + 2 * kv), 4, true))) return rc;
+		const int8_t *o = take_w(qo * h);
+		const float *os = take_f(h);
+		if ((rc = build_packed(&L.o, plain_map(o, os, (int)h), (int)qo, (int)h, 4, true))) return rc;
+		if ((rc = own_f(&L.rms_q, hd))) return rc;
+		if ((rc = own_f(&L.rms_k, hd))) return rc;
+		if ((rc = own_f(&L.apre, h))) return rc;
+		if ((rc = own_f(&L.apost, h))) return rc;
+		// up | gate: every tile holds half a tile of up columns followed by the same gate columns, so that
+		// gelu(gate) * up never leaves a workgroup
+		TgColMap ug;
+		memset(&ug, 0, sizeof(ug));
+		for (int part = 0; part < 2; part++) {
+			ug.src[part] = take_w(h * f);
+			ug.scales[part] = take_f(f);
+			ug.n[part] = (int)f;
+		}
+		ug.half = 1;
+		if ((rc = build_packed(&L.ug, ug, (int)h, (int)(2 * f), 8, true))) return rc;
+		const int8_t *d = take_w(f * h);
+		const float *ds = take_f(h);
+		if ((rc = build_packed(&L.d, plain_map(d, ds, (int)h), (int)f, (int)h, 4, true))) return rc;
+		if ((rc = own_f(&L.mpre, h))) return rc;
+		if ((rc = own_f(&L.mpost, h))) return rc;
 	}
-	if ((rc = read_i8(buf, (size_t)h * V))) return rc;
-	if ((rc = read_f(sc, (size_t)V))) return rc;
-	if ((rc = upload_packed(&m->lm, buf.data(), sc.data(), h, V, false))) return rc;
+	const int8_t *lm = take_w(h * V);
+	const float *lms = take_f(V);
+	if ((rc = build_packed(&m->lm, plain_map(lm, lms, (int)V), (int)h, (int)V, 4, false))) return rc;
+	TG_HIP(hipStreamSynchronize(g_stream));
 	m->loaded = true;
 	return TG_OK;
+}
+
+template <typename Fill>
+static int load_weights_impl(tg_model *m, Fill fill) {
+	model_free_weights(m);
+	const size_t n = tg_weight_file_bytes(&m->cfg);
+	uint8_t *d_raw = nullptr;
+	if (hipMalloc((void **)&d_raw, n) != hipSuccess) return tg_fail(TG_ERR_HIP, "hipMalloc of the file image failed");
+	int rc = stage_image(d_raw, n, fill);
+	if (rc == TG_OK) rc = build_from_image(m, d_raw);
+	(void)hipStreamSynchronize(g_stream);
+	(void)hipFree(d_raw);
+	if (rc != TG_OK) model_free_weights(m);
+	return rc;
 }
 
 extern "C" {
 
 int tg_model_load_weights(tg_model *m, const char *path) {
 	if (!m || !path) return tg_fail(TG_ERR_BAD_ARG, "null argument");
-	FILE *fp = fopen(path, "rb");
-	if (!fp) return tg_fail(TG_ERR_FILE_OPEN, "Could not open file.");  // transformer.hpp:163
-	int rc = load_weights_impl(m, [&](void *dst, size_t n) -> int {
-		if (fread(dst, 1, n, fp) != n) return tg_fail(TG_ERR_FILE_SHORT, "weight file is shorter than the configuration requires");
+	const int fd = open(path, O_RDONLY);
+	if (fd < 0) return tg_fail(TG_ERR_FILE_OPEN, "Could not open file.");  // transformer.hpp:163
+	struct stat st;
+	if (fstat(fd, &st) != 0 || (size_t)st.st_size < tg_weight_file_bytes(&m->cfg)) {
+		close(fd);
+		return tg_fail(TG_ERR_FILE_SHORT, "weight file is shorter than the configuration requires");
+	}
+	(void)posix_fadvise(fd, 0, 0, POSIX_FADV_SEQUENTIAL);
+	int rc = load_weights_impl(m, [&](void *dst, size_t off, size_t len) -> int {
+		size_t got = 0;
+		while (got < len) {
+			const ssize_t r = pread(fd, (char *)dst + got, len - got, (off_t)(off + got));
+			if (r <= 0) return tg_fail(TG_ERR_FILE_SHORT, "weight file is shorter than the configuration requires");
+			got += (size_t)r;
+		}
 		return TG_OK;
 	});
-	fclose(fp);
-	if (rc != TG_OK) model_free_weights(m);
+	close(fd);
 	return rc;
 }
 
@@ -619,15 +644,10 @@ int tg_model_load_weights_mem(tg_model *m, const void *image, size_t n) {
 	if (!m || !image) return tg_fail(TG_ERR_BAD_ARG, "null argument");
 	if (n != tg_weight_file_bytes(&m->cfg)) return tg_fail(TG_ERR_FILE_SHORT, "image size does not match the configuration");
 	const uint8_t *p = (const uint8_t *)image;
-	size_t off = 0;
-	int rc = load_weights_impl(m, [&](void *dst, size_t k) -> int {
-		if (off + k > n) return tg_fail(TG_ERR_FILE_SHORT, "image too short");
-		memcpy(dst, p + off, k);
-		off += k;
+	return load_weights_impl(m, [&](void *dst, size_t off, size_t len) -> int {
+		memcpy(dst, p + off, len);
 		return TG_OK;
 	});
-	if (rc != TG_OK) model_free_weights(m);
-	return rc;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -169,6 +169,20 @@ void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *sca
 
 void tg_launch_copy(void *dst, const void *src, size_t bytes, hipStream_t s);
 
+// Load-time re-tiling on the device.  A matrix of N virtual columns is assembled from up to three
+// row-major int8 sources (device pointers, reference layout [K][n[i]], scales[i] per source column):
+//   half == 0: the sources side by side (n[0] + n[1] + n[2] == N);
+//   half  > 0: tiles of 2*half virtual columns = half columns of source 0 followed by the same half
+//              columns of source 1 (both n[0] columns wide).
+struct TgColMap {
+	const int8_t *src[3];
+	const float *scales[3];
+	int n[3];
+	int half;
+};
+void tg_launch_retile_gemv(int8_t *dst, float *dst_scales, const TgColMap &m, int K, int N, int C, hipStream_t s);
+void tg_launch_retile_mfma(int8_t *dst, float *dst_scales, const TgColMap &m, int K, int N, hipStream_t s);
+
 // int8 MFMA prefill GEMM (tg_gemm_mfma.hip): A is first quantised per row into three int8 digit planes in operand order
 size_t tg_gemm_mfma_apack_bytes(int M, int K);
 size_t tg_gemm_mfma_rows(int M);  // rowfac scratch holds twice this many floats
