@@ -70,6 +70,11 @@ int tg_qgemv(float *C, const float *A, const int8_t *B, const float *scales, int
 int tg_qgemv_logits(float *C, const float *A, const int8_t *B, const float *scales, int inDim, int outDim);
 /* gemm::launch_qgemm (linalg.hpp:298): C[m][outDim] is overwritten. */
 int tg_qgemm(float *C, const float *A, const int8_t *B, const float *scales, int m, int inDim, int outDim);
+/* ops::attention_prefill (ops.hpp:377-526), host pointers in the reference's layouts: q and o [4][S][256]
+ * (heads outermost, as activation [1,4,S,256]), k and v [S][256].  q is taken as it reaches the reference's
+ * op: normalised and rotated, not yet scaled by 1/sqrt(256).  is_sw: keys qs - sw_context .. qs
+ * (ops.hpp:437-443), else causal. */
+int tg_attention_prefill(float *o, const float *q, const float *k, const float *v, int S, int is_sw, int sw_context);
 
 /* ---- kernel level: device-resident operands (what the forward uses; for timing) ----------- */
 typedef struct tg_qweight tg_qweight;
@@ -139,6 +144,9 @@ int tg_generate(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode
                 int32_t *out_ids, double *s_prefill, double *s_decode);
 /* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
 int tg_set_graphs(int enable);
+/* Debug taps of tg_forward_prefill (a copy of the residual stream after every block, for prompts of up to 1024
+ * tokens, read back with tg_session_tap): off by default, they cost one device copy per block. */
+int tg_set_taps(int enable);
 /* prefill GEMM: 1 (default) = int8 matrix cores on three int8 digit planes of the row-scaled activations
  * (exact integer accumulation, fp32-rounding-level accuracy),
  * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */

@@ -47,6 +47,7 @@ def tg():
     """The package, with the GPU initialised.  Fails loudly when the HIP library is not built."""
     mod = ge.load_package()
     mod.init(0)
+    mod.lib().tg_set_taps(1)  # the model tests compare the residual stream block by block
     return mod
 
 

@@ -210,3 +210,43 @@ def test_full_size_properties(tg):
     assert np.array_equal(outs[0] + outs[1], outs[2])  # exact on integer data
     colsum = W.astype(np.int64).sum(axis=1)            # sum_c y[c] = s * sum_r x[r] * rowsum(W)[r]
     assert float(outs[0].astype(np.float64).sum()) == float((xa.astype(np.int64) * colsum).sum()) * 2.0 ** -9
+
+
+# ---- prefill attention (ops::attention_prefill, ops.hpp:377-526) through the op-level entry point ----
+
+def _dense_rows(q, k, v, rows, is_sw, ctx):
+    """float64 softmax(q.k/16).v for the given query rows, keys qs-ctx..qs (local) or 0..qs (causal)."""
+    out = np.zeros((q.shape[0], len(rows), 256), np.float64)
+    k64, v64 = k.astype(np.float64), v.astype(np.float64)
+    for n, i in enumerate(rows):
+        lo = max(0, i - ctx) if is_sw else 0
+        sc = (q[:, i, :].astype(np.float64) @ k64[lo:i + 1].T) / 16.0
+        p = np.exp(sc - sc.max(axis=1, keepdims=True))
+        out[:, n, :] = (p / p.sum(axis=1, keepdims=True)) @ v64[lo:i + 1]
+    return out
+
+
+@pytest.mark.parametrize("name", list(gi.ATTN_PREFILL_CASES))
+def test_attention_prefill_vs_fixture_and_checker(tg, oracle, golden, name):
+    S, sw, ctx, seed = gi.ATTN_PREFILL_CASES[name]
+    q, k, v = gi.attn_prefill_inputs(S, seed)
+    o = tg.attention_prefill(q, k, v, sw, ctx)
+    # fp32 throughout; only the summation order differs from the reference's per-key scan
+    assert normrel(o[:, gi.attn_rows(S), :], golden[f"attn_prefill/{name}"]) < 2e-6
+    assert normrel(o, oracle.attention_prefill(q, k, v, sw, ctx)) < 2e-6
+
+
+@pytest.mark.parametrize("S", [1500, 4099])
+def test_attention_prefill_split_key_ranges(tg, oracle, S):
+    """Causal layers long enough for the key ranges to be cut into chunks and merged (S > 512); 4099 is ragged
+    against both the 16-query and the 32-key tiling."""
+    q, k, v = gi.attn_prefill_inputs(S, 410 + S)
+    o = tg.attention_prefill(q, k, v, False, 512)
+    rows = np.unique(np.concatenate([np.arange(0, S, 97), np.arange(505, 530), np.arange(S - 20, S)]))
+    assert normrel(o[:, rows, :], _dense_rows(q, k, v, rows, False, 512)) < 2e-6
+    if S <= 2000:
+        assert normrel(o, oracle.attention_prefill(q, k, v, False, 512)) < 2e-6
+    # the same tokens through a local layer: 513-key window, never split
+    ol = tg.attention_prefill(q, k, v, True, 512)
+    assert normrel(ol[:, rows, :], _dense_rows(q, k, v, rows, True, 512)) < 2e-6
+    assert np.array_equal(ol[:, :513, :], o[:, :513, :]) or normrel(ol[:, :513, :], o[:, :513, :]) < 2e-6

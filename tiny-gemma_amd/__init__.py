@@ -94,6 +94,7 @@ def lib():
     L.tg_forward_decode.argtypes = [C.c_void_p, C.c_int32, c_f32p, c_i32p]
     L.tg_generate_greedy.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_int, c_i32p, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.tg_decode_enqueue.argtypes = [C.c_void_p, C.c_int]
+    L.tg_attention_prefill.argtypes = [c_f32p, c_f32p, c_f32p, c_f32p, C.c_int, C.c_int, C.c_int]
     L.tg_minp_logits.argtypes = [c_f32p, C.c_int, C.c_float, C.c_float, C.c_float, c_i32p]
     L.tg_decode_enqueue_sampled.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_float, c_f32p]
     L.tg_generate.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_int, C.c_float, C.c_float, c_f32p, c_i32p,
@@ -136,6 +137,18 @@ def launch_qgemv(Cv, A, B, scales, inDim, outDim, logits=False):
 
 def launch_qgemm(Cm, A, B, scales, m, inDim, outDim):
     check(lib().tg_qgemm(_f(Cm), _f(A), B.ctypes.data_as(c_i8p), _f(scales), m, inDim, outDim))
+
+
+def attention_prefill(q, k, v, is_sw, sw_context=512):
+    """ops::attention_prefill on the device: q [4][S][256], k, v [S][256] -> o [4][S][256]."""
+    q = np.ascontiguousarray(q, np.float32)
+    k = np.ascontiguousarray(k, np.float32)
+    v = np.ascontiguousarray(v, np.float32)
+    S = k.shape[0]
+    assert q.shape == (4, S, 256) and k.shape == (S, 256) and v.shape == (S, 256)
+    o = np.empty_like(q)
+    check(lib().tg_attention_prefill(_f(o), _f(q), _f(k), _f(v), S, int(bool(is_sw)), int(sw_context)))
+    return o
 
 
 def minp_logits(logits, minp, temp, randf):

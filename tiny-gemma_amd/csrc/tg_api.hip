@@ -34,6 +34,8 @@ bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GP
 int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
+int g_n_cu = 256;
+bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 
 bool legal_in(int d) { return d == 640 || d == 2048 || d == 1024 || d == 256 || d == 1152 || d == 6912; }            // static_switch.hpp:7-30
 bool legal_out(int d) { return d == 640 || d == 262144 || d == 2048 || d == 256 || d == 1024 || d == 1152 || d == 6912; }  // :32-58
@@ -196,6 +198,47 @@ struct tg_model {
 	std::vector<LayerDev> L;
 };
 
+namespace {
+// Device copy of the balanced work list of causal prefill layers of S tokens, with its scratch.
+struct AttnPlanDev {
+	TgAttnPrefillPlan p;
+	bool use = false;
+	int S = -1;  // token count the lists were built for
+	void *bufs[4] = {nullptr, nullptr, nullptr, nullptr};
+	std::vector<int4> items, split;  // host copies stay alive until the uploads have completed
+	int build(int n_tokens) {
+		if (n_tokens == S) return TG_OK;
+		release();
+		int nslots = 0;
+		use = tg_attn_prefill_plan(n_tokens, g_n_cu, items, split, nslots);
+		S = n_tokens;
+		if (!use) return TG_OK;
+		TG_HIP(hipMalloc(&bufs[0], items.size() * sizeof(int4)));
+		TG_HIP(hipMalloc(&bufs[1], split.size() * sizeof(int4)));
+		TG_HIP(hipMalloc(&bufs[2], tg_attn_prefill_part_floats(nslots) * sizeof(float)));
+		TG_HIP(hipMalloc(&bufs[3], tg_attn_prefill_ml_floats(nslots) * sizeof(float)));
+		TG_HIP(hipMemcpyAsync(bufs[0], items.data(), items.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
+		TG_HIP(hipMemcpyAsync(bufs[1], split.data(), split.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
+		p.items = (const int4 *)bufs[0];
+		p.split = (const int4 *)bufs[1];
+		p.nitems = (int)items.size();
+		p.nsplit = (int)split.size();
+		p.part_o = (float *)bufs[2];
+		p.part_ml = (float *)bufs[3];
+		return TG_OK;
+	}
+	const TgAttnPrefillPlan *get() const { return use ? &p : nullptr; }
+	void release() {
+		for (void *&b : bufs) {
+			if (b) (void)hipFree(b);
+			b = nullptr;
+		}
+		use = false;
+		S = -1;
+	}
+};
+}  // namespace
+
 struct tg_session {
 	tg_model *m = nullptr;
 	float *cos_g = nullptr, *sin_g = nullptr, *cos_l = nullptr, *sin_l = nullptr;  // [n_pos][head_dim/2]
@@ -223,6 +266,11 @@ struct tg_session {
 	bool sampling = false;  // decode steps enqueued now draw their token instead of taking the argmax
 	float s_minp = 1.0f, s_temp = 1.0f;
 	int rand_base = 0;      // token-log index of the token that uses randf[0]
+	// prefill workspace (the reference's PrefillState, decode.hpp:281-351): one arena, grown on demand, kept until the
+	// session is destroyed, and the work lists of the causal layers for the last prompt length
+	void *pf_ws = nullptr;
+	size_t pf_ws_bytes = 0;
+	AttnPlanDev pf_plan;
 };
 
 namespace {
@@ -263,6 +311,7 @@ int tg_init(int device) {
 	hipDeviceProp_t prop;
 	TG_HIP(hipGetDeviceProperties(&prop, device));
 	snprintf(g_devname, sizeof(g_devname), "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+	g_n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	TG_HIP(hipStreamCreate(&g_stream));
 	g_device = device;
 	g_inited = true;
@@ -686,9 +735,10 @@ void tg_session_destroy(tg_session *s) {
 	s->graphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
-	              s->tok_log, s->taps, s->probs, s->seg, s->bsum, s->bmax, s->randf};
+	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf};
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
+	s->pf_plan.release();
 	for (float *p : s->kc)
 		if (p) (void)hipFree(p);
 	for (float *p : s->vc)
@@ -779,7 +829,6 @@ int tg_session_reset(tg_session *s) {
 	TG_HIP(hipDeviceSynchronize());
 	s->pos = s->bp_local = s->bp_global = s->steps = 0;
 	if (s->taps) {
-		TG_HIP(hipFree(s->taps));
 		s->taps = nullptr;
 	}
 	s->tap_rows = 0;
@@ -969,7 +1018,6 @@ int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax)
 	TG_HIP(hipStreamSynchronize(g_stream));
 	if (argmax) *argmax = tok;
 	if (s->taps) {  // taps now describe the decode step
-		(void)hipFree(s->taps);
 		s->taps = nullptr;
 		s->tap_rows = 0;
 	}
@@ -1024,7 +1072,6 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 	}
 	if (s->taps) {
 		TG_HIP(hipStreamSynchronize(g_stream));
-		(void)hipFree(s->taps);
 		s->taps = nullptr;
 		s->tap_rows = 0;
 	}
@@ -1036,6 +1083,11 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
 		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	StepOnly only{kernel_class, kernel_class == TG_KC_LMHEAD ? 0 : layer, repeat};
 	return enqueue_decode_step(s, nullptr, false, &only);
+}
+
+int tg_set_taps(int enable) {
+	g_keep_taps = enable != 0;
+	return TG_OK;
 }
 
 int tg_set_gemm_mode(int mfma) {
@@ -1106,6 +1158,47 @@ int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out) {
 // ---------------------------------------------------------------------------------------------
 // forward_prefill
 // ---------------------------------------------------------------------------------------------
+}  // extern "C"
+
+
+extern "C" {
+
+int tg_attention_prefill(float *o, const float *q, const float *k, const float *v, int S, int is_sw, int sw_context) {
+	if (int rc = ensure_init()) return rc;
+	if (!o || !q || !k || !v || S < 1 || sw_context < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	constexpr int NH = 4, HD = 256;
+	const size_t rows = (size_t)S;
+	std::vector<float> qr(rows * NH * HD), orow(rows * NH * HD);
+	for (int hh = 0; hh < NH; hh++)
+		for (size_t t = 0; t < rows; t++) memcpy(&qr[(t * NH + hh) * HD], &q[((size_t)hh * rows + t) * HD], sizeof(float) * HD);
+	float *dq = nullptr, *dk = nullptr, *dv = nullptr, *dout = nullptr;
+	AttnPlanDev plan;
+	auto done = [&](int rc) {
+		(void)hipStreamSynchronize(g_stream);
+		void *ps[] = {dq, dk, dv, dout};
+		for (void *p : ps)
+			if (p) (void)hipFree(p);
+		plan.release();
+		return rc;
+	};
+	int rc = tg_dev_alloc((void **)&dq, sizeof(float) * rows * NH * HD);
+	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dout, sizeof(float) * rows * NH * HD);
+	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dk, sizeof(float) * rows * HD);
+	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dv, sizeof(float) * rows * HD);
+	if (rc == TG_OK) rc = tg_copy_h2d(dq, qr.data(), sizeof(float) * rows * NH * HD);
+	if (rc == TG_OK) rc = tg_copy_h2d(dk, k, sizeof(float) * rows * HD);
+	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
+	if (rc == TG_OK && !is_sw) rc = plan.build(S);
+	if (rc != TG_OK) return done(rc);
+	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), g_stream);
+	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
+	rc = tg_copy_d2h(orow.data(), dout, sizeof(float) * rows * NH * HD);
+	if (rc != TG_OK) return done(rc);
+	for (int hh = 0; hh < NH; hh++)
+		for (size_t t = 0; t < rows; t++) memcpy(&o[((size_t)hh * rows + t) * HD], &orow[(t * NH + hh) * HD], sizeof(float) * HD);
+	return done(TG_OK);
+}
+
 int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, int32_t *argmax) {
 	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
 	tg_model *m = s->m;
@@ -1116,14 +1209,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	const int L = c.n_layers, h = c.hidden_size, f = c.intermediate_size, hd = c.head_dim;
 	const int qo = c.n_head * hd, nq = qo + 2 * hd;
 	const size_t S = (size_t)n;
-	int *d_ids = nullptr;
-	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr;
-	int8_t *apack = nullptr;
-	auto cleanup = [&]() {
-		void *ps[] = {d_ids, x, xn, qkv, ao, t, hb, rowscale, apack};
-		for (void *p : ps)
-			if (p) (void)hipFree(p);
-	};
+	auto cleanup = [&]() {};  // the workspace belongs to the session
 #define TG_TRY(expr)                                                                             \
 	do {                                                                                         \
 		hipError_t e_ = (expr);                                                                  \
@@ -1132,27 +1218,37 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 			return tg_fail(TG_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));       \
 		}                                                                                        \
 	} while (0)
-	TG_TRY(hipMalloc((void **)&d_ids, sizeof(int) * S));
-	TG_TRY(hipMalloc((void **)&x, sizeof(float) * S * h));
-	TG_TRY(hipMalloc((void **)&xn, sizeof(float) * S * h));
-	TG_TRY(hipMalloc((void **)&qkv, sizeof(float) * S * nq));
-	TG_TRY(hipMalloc((void **)&ao, sizeof(float) * S * qo));
-	TG_TRY(hipMalloc((void **)&t, sizeof(float) * S * h));
-	TG_TRY(hipMalloc((void **)&hb, sizeof(float) * S * f));
-	if (g_gemm_mfma) {
-		TG_TRY(hipMalloc((void **)&apack, tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h))));
-		TG_TRY(hipMalloc((void **)&rowscale, sizeof(float) * 2 * tg_gemm_mfma_rows(n)));
+	// PrefillState (decode.hpp:281-351): carved out of one arena the session keeps (hipMalloc/hipFree of a few hundred
+	// MB per call cost milliseconds), 256-byte aligned pieces
+	const bool keep_taps = g_keep_taps && n <= PREFILL_TAP_MAX_ROWS;
+	size_t need = 0;
+	auto carve = [&](size_t bytes) {
+		const size_t off = need;
+		need += (bytes + 255) & ~(size_t)255;
+		return off;
+	};
+	const size_t o_ids = carve(sizeof(int) * S), o_x = carve(sizeof(float) * S * h), o_xn = carve(sizeof(float) * S * h),
+	             o_qkv = carve(sizeof(float) * S * nq), o_ao = carve(sizeof(float) * S * qo), o_t = carve(sizeof(float) * S * h),
+	             o_hb = carve(sizeof(float) * S * f),
+	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
+	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
+	             o_taps = carve(keep_taps ? sizeof(float) * (size_t)(2 * L + 1) * S * h : 0);
+	if (need > s->pf_ws_bytes) {
+		if (s->pf_ws) (void)hipFree(s->pf_ws);
+		s->pf_ws = nullptr;
+		s->pf_ws_bytes = 0;
+		TG_TRY(hipMalloc(&s->pf_ws, need));
+		s->pf_ws_bytes = need;
 	}
-	const bool keep_taps = n <= PREFILL_TAP_MAX_ROWS;
-	if (s->taps) {
-		(void)hipFree(s->taps);
-		s->taps = nullptr;
-		s->tap_rows = 0;
-	}
-	if (keep_taps) {
-		TG_TRY(hipMalloc((void **)&s->taps, sizeof(float) * (size_t)(2 * L + 1) * S * h));
-		s->tap_rows = n;
-	}
+	uint8_t *ws = (uint8_t *)s->pf_ws;
+	int *d_ids = (int *)(ws + o_ids);
+	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
+	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
+	int8_t *apack = (int8_t *)(ws + o_apack);
+	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
+	s->tap_rows = keep_taps ? n : 0;
+	AttnPlanDev &plan = s->pf_plan;
+	if (int rc = plan.build(n)) return rc;
 	auto tap = [&](int b) -> hipError_t {
 		if (!keep_taps) return hipSuccess;
 		return hipMemcpyAsync(s->taps + (size_t)b * S * h, x, sizeof(float) * S * h, hipMemcpyDeviceToDevice, g_stream);
@@ -1174,7 +1270,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
 		                            g_stream);
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, g_stream);
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, plan.get(), g_stream);
 		// O (modules.hpp:127-128)
 		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
@@ -1214,7 +1310,6 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	TG_TRY(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
 	TG_TRY(hipStreamSynchronize(g_stream));
 	if (argmax) *argmax = tok;
-	cleanup();
 #undef TG_TRY
 	return TG_OK;
 }
@@ -1303,7 +1398,6 @@ int tg_decode_enqueue_sampled(tg_session *s, int n_steps, float minp, float temp
 	s->sampling = false;
 	if (rc == TG_OK && s->taps) {
 		TG_HIP(hipStreamSynchronize(g_stream));
-		(void)hipFree(s->taps);
 		s->taps = nullptr;
 		s->tap_rows = 0;
 	}

@@ -17,8 +17,18 @@
 // rows of a read hit 16 different groups of 4 banks (scores) and the 4 rows of a V read are 16 banks
 // apart.  Keys outside a query's range (causal; local layers: qs-window .. qs, ops.hpp:437-443) get a
 // score of -inf.
+//
+// Balance.  A causal layer gives query tile i about i/2 key tiles of work, and at a few thousand tokens there
+// is only about one query tile per compute unit, so the last tile would set the pace at twice the mean.  Long
+// key ranges are therefore cut into chunks of at most `chunk` key tiles: a work item = (query tile, chunk),
+// listed by the host heaviest first.  An item of a split query tile leaves its un-normalised output rows with
+// their running maximum and sum in scratch, and attn_prefill_merge_kernel folds the chunks of a row together
+// (the flash-decoding merge: weights exp(m_c - max m) / sum).
 
 #include "tg_internal.h"
+
+#include <algorithm>
+#include <vector>
 
 namespace {
 
@@ -31,18 +41,33 @@ constexpr int TK = 32;     // keys per LDS tile
 constexpr int LDS_LD = 260;
 constexpr int PNT = 256;
 
+// items == nullptr: workgroup b owns query tile gridDim.x - 1 - b and all its keys.
+// items != nullptr (causal layers only): items[b] = {query tile, first key tile, end key tile, slot}; slot < 0: the
+// item is the whole key range of its query tile and writes o; else it writes part_o[slot][16][NH][HD] (un-normalised)
+// and part_ml[slot][16][NH][2] (running maximum, running sum).
 __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
-                                                               int ldkv, int ldo, int is_sw, int window) {
+                                                               int ldkv, int ldo, int is_sw, int window, const int4 *items,
+                                                               float *part_o, float *part_ml) {
 	__shared__ __attribute__((aligned(16))) float Ks[TK][LDS_LD];
 	__shared__ __attribute__((aligned(16))) float Vs[TK][LDS_LD];
 
 	const int tid = threadIdx.x, lane = tid & 63, head = tid >> 6, c = lane & 15, g = lane >> 4;
 	// late query tiles of a causal layer see the most keys: start them first
-	const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ;
+	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ, slot = -1;
+	int4 item = int4{0, 0, 0, -1};
+	if (items != nullptr) {
+		item = items[blockIdx.x];
+		q0 = item.x * TQ;
+		slot = item.w;
+	}
 	const int qpos = q0 + c;                         // the query whose scores this lane holds
 	const int qrow = qpos < S ? qpos : S - 1;
-	const int kb = (is_sw && q0 > window) ? q0 - window : 0;
-	const int ke = (q0 + TQ < S) ? q0 + TQ : S;      // exclusive
+	int kb = (is_sw && q0 > window) ? q0 - window : 0;
+	int ke = (q0 + TQ < S) ? q0 + TQ : S;            // exclusive
+	if (items != nullptr) {
+		kb = item.y * TK;
+		ke = min(ke, item.z * TK);
+	}
 	const int ntiles = (ke - kb + TK - 1) / TK;
 	const int klo = is_sw ? qpos - window : 0;       // this query's first key (may be negative)
 
@@ -146,6 +171,21 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 		}
 	}
 
+	if (slot >= 0) {  // one chunk of a split query tile: un-normalised rows + (m, l) per (query, head)
+		float *po = part_o + (size_t)slot * TQ * NH * HD;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			float *op = po + ((size_t)(4 * g + i) * NH + head) * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i];
+		}
+		if (g == 0) {
+			float *pm = part_ml + (((size_t)slot * TQ + c) * NH + head) * 2;
+			pm[0] = m_run;
+			pm[1] = l_run;
+		}
+		return;
+	}
 	float lr[4];
 #pragma unroll
 	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
@@ -160,13 +200,74 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 	}
 }
 
+// One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
+// split[b] = {query tile, first slot, number of chunks}.
+__global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
+                                                                const float *part_ml) {
+	const int4 sp = split[blockIdx.x / TQ];
+	const int qi = blockIdx.x % TQ, qpos = sp.x * TQ + qi;
+	if (qpos >= S) return;
+	const int lane = threadIdx.x & 63, head = threadIdx.x >> 6;
+	float M = -INFINITY;
+	for (int ch = 0; ch < sp.z; ch++) M = fmaxf(M, part_ml[(((size_t)(sp.y + ch) * TQ + qi) * NH + head) * 2]);
+	float L = 0.0f;
+	f32x4 acc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+	for (int ch = 0; ch < sp.z; ch++) {
+		const size_t row = ((size_t)(sp.y + ch) * TQ + qi) * NH + head;
+		const float wgt = expf(part_ml[row * 2] - M);
+		L = fmaf(part_ml[row * 2 + 1], wgt, L);
+		const f32x4 x = *reinterpret_cast<const f32x4 *>(part_o + row * HD + 4 * lane);
+		acc += x * wgt;
+	}
+	*reinterpret_cast<f32x4 *>(o + (size_t)qpos * ldo + head * HD + 4 * lane) = acc / L;
+}
+
 }  // namespace
+
+// Work list of a causal layer of S tokens, for tg_launch_attn_prefill.  Returns false when no query tile needs
+// splitting (then the plain launch is already balanced).  items: one int4 per workgroup, heaviest first;
+// split: one int4 per split query tile; nslots: chunks that go through scratch.
+bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
+	const int nq = (S + TQ - 1) / TQ;
+	auto ntiles_of = [&](int qt) { return (std::min(qt * TQ + TQ, S) + TK - 1) / TK; };
+	long total = 0;
+	for (int qt = 0; qt < nq; qt++) total += ntiles_of(qt);
+	// about 8 items per compute unit, and never chunks below 16 key tiles (512 keys)
+	const int chunk = (int)std::max<long>(16, total / ((long)n_cu * 8));
+	items.clear();
+	split.clear();
+	nslots = 0;
+	for (int qt = 0; qt < nq; qt++) {
+		const int nt = ntiles_of(qt), nc = (nt + chunk - 1) / chunk;
+		if (nc == 1) {
+			items.push_back(int4{qt, 0, nt, -1});
+			continue;
+		}
+		split.push_back(int4{qt, nslots, nc, 0});
+		for (int ch = 0; ch < nc; ch++) {  // equal chunks
+			const int tb = (int)((long)nt * ch / nc), te = (int)((long)nt * (ch + 1) / nc);
+			items.push_back(int4{qt, tb, te, nslots++});
+		}
+	}
+	if (split.empty()) return false;
+	std::stable_sort(items.begin(), items.end(), [](const int4 &a, const int4 &b) { return a.z - a.y > b.z - b.y; });
+	return true;
+}
+size_t tg_attn_prefill_part_floats(int nslots) { return (size_t)nslots * TQ * NH * HD; }
+size_t tg_attn_prefill_ml_floats(int nslots) { return (size_t)nslots * TQ * NH * 2; }
 
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, hipStream_t s) {
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, hipStream_t s) {
 	(void)n_head;
 	(void)hd;
-	hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)((S + TQ - 1) / TQ)), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
-	                   window);
+	if (plan == nullptr || is_sw) {
+		hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)((S + TQ - 1) / TQ)), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo,
+		                   is_sw, window, (const int4 *)nullptr, (float *)nullptr, (float *)nullptr);
+		return;
+	}
+	hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)plan->nitems), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, 0, window,
+	                   plan->items, plan->part_o, plan->part_ml);
+	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * TQ)), dim3(PNT), 0, s, o, S, ldo, plan->split,
+	                   plan->part_o, plan->part_ml);
 }

@@ -161,8 +161,18 @@ void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const 
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
                                  const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
                                  hipStream_t s);
+// Balanced work list of a causal prefill layer (device copies of what tg_attn_prefill_plan returns) + scratch.
+struct TgAttnPrefillPlan {
+	const int4 *items;  // [nitems] {query tile, first key tile, end key tile, slot or -1}
+	const int4 *split;  // [nsplit] {query tile, first slot, chunks}
+	int nitems, nsplit;
+	float *part_o, *part_ml;
+};
+bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
+size_t tg_attn_prefill_part_floats(int nslots);
+size_t tg_attn_prefill_ml_floats(int nslots);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, hipStream_t s);
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, hipStream_t s);
 // exact-order GEMM on the GEMV tiling (ntiles tiles of Ct columns): C[m][N] = (A[m][K] . W) * scales; epi GEGLU writes C[m][N/2]
 void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);

@@ -42,68 +42,111 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 	for (int d = threadIdx.x; d < hidden; d += RNT) x[(size_t)s * hidden + d] = scales[d] * (emb_scale * (float)row[d]);
 }
 
-__device__ __forceinline__ float bmax(float v, float *sred) {
-	v = tg_wave_max(v);
-	__syncthreads();
-	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
-	__syncthreads();
-	return fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
-}
-
-// One workgroup per row: [post-norm + residual (+ residual out)] + pre-norm.  The normalised row goes out as fp32
-// (out != nullptr) and/or straight as the int8 digit planes + row factors of the MFMA GEMM that consumes it
-// (apack != nullptr): the same bits the stand-alone quantising pre-pass would produce from the fp32 row.
+// One wave per row, the row held in registers (16 consecutive elements per lane and round; ROUNDS = 2 covers rows of
+// up to 2048 elements), wave reductions only: [post-norm + residual (+ residual out)] + pre-norm.  The normalised row
+// goes out as fp32 (out != nullptr) and/or straight as the int8 digit planes + row factors of the MFMA GEMM that
+// consumes it (apack != nullptr): the same bits the stand-alone quantising pre-pass would produce from the fp32 row.
+template <int ROUNDS>
 __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *w_pre, const float *w_post,
-                                                        const float *resid, float *resid_out, int dim, int8_t *apack, float *rowfac,
-                                                        int Mpad) {
-	__shared__ __attribute__((aligned(16))) float xs[1152];
-	__shared__ float sred[4];
-	const int s = blockIdx.x, tid = threadIdx.x;
+                                                        const float *resid, float *resid_out, int S, int dim, int8_t *apack,
+                                                        float *rowfac, int Mpad) {
+	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	const int lane = threadIdx.x & 63, s = blockIdx.x * (RNT / 64) + (threadIdx.x >> 6);
+	if (s >= S) return;  // uniform over the wave
 	const float eps = 1e-06f;
-	const float *row = in + (size_t)s * dim;
-	float ss = 0.0f;
-	for (int d = tid; d < dim; d += RNT) {
-		float p = row[d];
-		xs[d] = p;
-		ss = fmaf(p, p, ss);
+	const int npieces = dim >> 4;
+	bool act[ROUNDS];
+	size_t off[ROUNDS];  // element offset of this lane's piece inside a row (clamped to piece 0 when the lane idles)
+	f32x4 v[ROUNDS][4], rs[ROUNDS][4], wpo[ROUNDS][4], wpr[ROUNDS][4];
+	// every load of the row is requested before the first use
+#pragma unroll
+	for (int r = 0; r < ROUNDS; r++) {
+		const int piece = lane + 64 * r;
+		act[r] = piece < npieces;
+		off[r] = act[r] ? (size_t)piece * 16 : 0;
+#pragma unroll
+		for (int q = 0; q < 4; q++) v[r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)s * dim + off[r] + 4 * q);
 	}
-	ss = bsum(ss, sred);
+	if (resid != nullptr) {
+#pragma unroll
+		for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				rs[r][q] = *reinterpret_cast<const f32x4 *>(resid + (size_t)s * dim + off[r] + 4 * q);
+				wpo[r][q] = *reinterpret_cast<const f32x4 *>(w_post + off[r] + 4 * q);
+			}
+	}
+	if (w_pre != nullptr) {
+#pragma unroll
+		for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+			for (int q = 0; q < 4; q++) wpr[r][q] = *reinterpret_cast<const f32x4 *>(w_pre + off[r] + 4 * q);
+	}
+	float ss = 0.0f;
+#pragma unroll
+	for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+		for (int q = 0; q < 4; q++) {
+			if (!act[r]) v[r][q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+			for (int e = 0; e < 4; e++) ss = fmaf(v[r][q][e], v[r][q][e], ss);
+		}
+	ss = tg_wave_sum(ss);
 	if (resid != nullptr) {
 		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
 		float s2 = 0.0f;
-		for (int d = tid; d < dim; d += RNT) {
-			float t = (xs[d] * irms) * (w_post[d] + 1.0f) + resid[(size_t)s * dim + d];
-			xs[d] = t;
-			resid_out[(size_t)s * dim + d] = t;
-			s2 = fmaf(t, t, s2);
-		}
-		ss = bsum(s2, sred);
-	}
-	if (out != nullptr || apack != nullptr) {
-		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
-		float amax = 0.0f;
-		for (int d = tid; d < dim; d += RNT) {
-			const float y = (xs[d] * irms) * (w_pre[d] + 1.0f);
-			if (out != nullptr) out[(size_t)s * dim + d] = y;
-			xs[d] = y;  // each thread rewrites only what it read
-			amax = fmaxf(amax, fabsf(y));
-		}
-		if (apack != nullptr) {
-			amax = bmax(amax, sred);  // its barriers also publish xs
-			float mul, inv;
-			tg_row_factors(amax, mul, inv);
-			if (tid == 0) {
-				rowfac[s] = mul;
-				rowfac[Mpad + s] = inv;
-			}
-			for (int g = tid; g < (dim >> 4); g += RNT) {
-				tg_i32x4 pl[3];
-				tg_quant16(&xs[16 * g], mul, pl);
-				tg_i32x4 *dst = tg_plane_dst(apack, s, 16 * g, dim);
 #pragma unroll
-				for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
+		for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				f32x4 t;
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					t[e] = act[r] ? (v[r][q][e] * irms) * (wpo[r][q][e] + 1.0f) + rs[r][q][e] : 0.0f;
+					s2 = fmaf(t[e], t[e], s2);
+				}
+				v[r][q] = t;
+				if (act[r]) *reinterpret_cast<f32x4 *>(resid_out + (size_t)s * dim + off[r] + 4 * q) = t;
 			}
+		ss = tg_wave_sum(s2);
+	}
+	if (out == nullptr && apack == nullptr) return;
+	const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
+	float amax = 0.0f;
+#pragma unroll
+	for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+		for (int q = 0; q < 4; q++) {
+			f32x4 y;
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				y[e] = act[r] ? (v[r][q][e] * irms) * (wpr[r][q][e] + 1.0f) : 0.0f;
+				amax = fmaxf(amax, fabsf(y[e]));
+			}
+			v[r][q] = y;
+			if (out != nullptr && act[r]) *reinterpret_cast<f32x4 *>(out + (size_t)s * dim + off[r] + 4 * q) = y;
 		}
+	if (apack == nullptr) return;
+	amax = tg_wave_max(amax);
+	float mul, inv;
+	tg_row_factors(amax, mul, inv);
+	if (lane == 0) {
+		rowfac[s] = mul;
+		rowfac[Mpad + s] = inv;
+	}
+#pragma unroll
+	for (int r = 0; r < ROUNDS; r++) {
+		if (!act[r]) continue;
+		float y[16];
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+#pragma unroll
+			for (int e = 0; e < 4; e++) y[4 * q + e] = v[r][q][e];
+		tg_i32x4 pl[3];
+		tg_quant16(y, mul, pl);
+		tg_i32x4 *dst = tg_plane_dst(apack, s, (int)off[r], dim);
+#pragma unroll
+		for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
 	}
 }
 
@@ -206,8 +249,12 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
                          int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(S);
-	hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, out, in, w_pre, w_post, resid, resid_out, dim, apack, rowfac,
-	                   Mpad);
+	const dim3 grid((unsigned)((S + RNT / 64 - 1) / (RNT / 64))), block(RNT);
+	// dim is a legal row dimension: a multiple of 16, at most 2048 where a norm is applied (hidden sizes 640 and 1152)
+	if (dim <= 1024)
+		hipLaunchKernelGGL(norm_rows_kernel<1>, grid, block, 0, s, out, in, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac, Mpad);
+	else
+		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac, Mpad);
 }
 
 // Wp/scales: GEMV tiling of the matrix (ntiles tiles of Ct columns); C gets ntiles * Ct columns, or half of that for GEGLU
