@@ -47,7 +47,7 @@ constexpr int PNT = 256;
 // and part_ml[slot][16][NH][2] (running maximum, running sum).
 __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
                                                                int ldkv, int ldo, int is_sw, int window, const int4 *items,
-                                                               float *part_o, float *part_ml) {
+                                                               float *part_o, float *part_ml, float *rowmax_part, int Mpad) {
 	__shared__ __attribute__((aligned(16))) float Ks[TK][LDS_LD];
 	__shared__ __attribute__((aligned(16))) float Vs[TK][LDS_LD];
 
@@ -192,10 +192,20 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0 + 4 * g + i;
+		float omax = 0.0f;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+			for (int dt = 0; dt < HD / 16; dt++) {
+				const float val = oacc[dt][i] / lr[i];
+				op[16 * dt] = val;
+				omax = fmaxf(omax, fabsf(val));
+			}
+		}
+		// the output projection quantises these rows next: leave max|row| over this head's columns for it
+		if (rowmax_part != nullptr) {
+			omax = tg_row16_max(omax);
+			if (c == 0 && qo < S) rowmax_part[(size_t)head * Mpad + qo] = omax;
 		}
 	}
 }
@@ -203,7 +213,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
-                                                                const float *part_ml) {
+                                                                const float *part_ml, float *rowmax_part, int Mpad) {
 	const int4 sp = split[blockIdx.x / TQ];
 	const int qi = blockIdx.x % TQ, qpos = sp.x * TQ + qi;
 	if (qpos >= S) return;
@@ -219,7 +229,12 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 		const f32x4 x = *reinterpret_cast<const f32x4 *>(part_o + row * HD + 4 * lane);
 		acc += x * wgt;
 	}
-	*reinterpret_cast<f32x4 *>(o + (size_t)qpos * ldo + head * HD + 4 * lane) = acc / L;
+	const f32x4 res = acc / L;
+	*reinterpret_cast<f32x4 *>(o + (size_t)qpos * ldo + head * HD + 4 * lane) = res;
+	if (rowmax_part != nullptr) {
+		const float omax = tg_wave_max(fmaxf(fmaxf(fabsf(res[0]), fabsf(res[1])), fmaxf(fabsf(res[2]), fabsf(res[3]))));
+		if (lane == 0) rowmax_part[(size_t)head * Mpad + qpos] = omax;
+	}
 }
 
 }  // namespace
@@ -258,16 +273,17 @@ size_t tg_attn_prefill_ml_floats(int nslots) { return (size_t)nslots * TQ * NH *
 
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, hipStream_t s) {
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, hipStream_t s) {
 	(void)n_head;
 	(void)hd;
+	const int Mpad = (int)tg_gemm_mfma_rows(S);  // rowmax_part (may be null): [4 heads][Mpad], max|o[row][head's columns]|
 	if (plan == nullptr || is_sw) {
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)((S + TQ - 1) / TQ)), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo,
-		                   is_sw, window, (const int4 *)nullptr, (float *)nullptr, (float *)nullptr);
+		                   is_sw, window, (const int4 *)nullptr, (float *)nullptr, (float *)nullptr, rowmax_part, Mpad);
 		return;
 	}
 	hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)plan->nitems), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, 0, window,
-	                   plan->items, plan->part_o, plan->part_ml);
+	                   plan->items, plan->part_o, plan->part_ml, rowmax_part, Mpad);
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * TQ)), dim3(PNT), 0, s, o, S, ldo, plan->split,
-	                   plan->part_o, plan->part_ml);
+	                   plan->part_o, plan->part_ml, rowmax_part, Mpad);
 }

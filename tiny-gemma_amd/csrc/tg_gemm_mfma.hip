@@ -73,6 +73,33 @@ __global__ __launch_bounds__(GNT) void row_scale_kernel(const float *A, int lda,
 	}
 }
 
+// The same factors from partial row maxima the producer of A left behind: rowmax_part[p][Mpad] = max|A[m][columns of
+// part p]| (the GeGLU epilogue writes one part per column tile, prefill attention one per head), so A is not read.
+// Workgroup = 32 rows; thread (r, kq) folds the parts p = kq, kq + 8, ...; the 8 partial maxima of a row meet in LDS.
+__global__ __launch_bounds__(GNT) void row_scale_parts_kernel(const float *rowmax_part, int nparts, int M, float *mul, float *inv,
+                                                              int Mpad) {
+	__shared__ float pmax[8][32];
+	const int tid = threadIdx.x, r = tid & 31, kq = tid >> 5, m = blockIdx.x * 32 + r;
+	float a0 = 0.0f, a1 = 0.0f;
+	int p = kq;
+	for (; p + 8 < nparts; p += 16) {
+		a0 = fmaxf(a0, rowmax_part[(size_t)p * Mpad + m]);
+		a1 = fmaxf(a1, rowmax_part[(size_t)(p + 8) * Mpad + m]);
+	}
+	if (p < nparts) a0 = fmaxf(a0, rowmax_part[(size_t)p * Mpad + m]);
+	pmax[kq][r] = fmaxf(a0, a1);
+	__syncthreads();
+	if (kq == 0) {
+		float amax = pmax[0][r];
+#pragma unroll
+		for (int i = 1; i < 8; i++) amax = fmaxf(amax, pmax[i][r]);
+		float s, rcp;
+		tg_row_factors(m < M ? amax : 0.0f, s, rcp);  // rows of the padding were never written
+		mul[m] = s;
+		inv[m] = rcp;
+	}
+}
+
 // A [M][lda] fp32 -> digit planes in A-operand order.  Workgroup = 32 rows x 128 k; thread = one lane's 16
 // bytes of one (k step, half): row r = tid % 32, k = 128 blockIdx.y + 16 (tid / 32) .. + 15.
 __global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda, int M, int K, const float *mul, int8_t *Apack) {
@@ -100,7 +127,7 @@ __global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda
 template <bool GEGLU, bool LUTLDS>
 __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
                                                       const float *scales, int M, int K, int ldc, const float *lut, float gmin,
-                                                      float geps, float ginv, int lut_size) {
+                                                      float geps, float ginv, int lut_size, float *rowmax_part, int Mpad) {
 	// B operands of one stage: [k / 16][column][16 bytes], double buffered
 	__shared__ __attribute__((aligned(16))) i32x4 Bs[2][KSTAGE / 16][TG_CT];
 	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
@@ -234,6 +261,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 		const float v = fmaf((float)acc[2][j][i], 65536.0f, fmaf((float)acc[1][j][i], 256.0f, (float)acc[0][j][i]));
 		return (v * rs) * sc[j][i >> 2][i & 3];
 	};
+	float omax = 0.0f;  // GEGLU: largest magnitude this lane writes (its row, 32 of the tile's 64 columns)
 	if (m < M) {
 		float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 4 * hb;
 #pragma unroll
@@ -248,6 +276,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 						const float gate = value(j + 2, i);
 						o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
 						       value(j, i);
+						omax = fmaxf(omax, fabsf(o[e]));
 					} else {
 						o[e] = value(j, i);
 					}
@@ -255,6 +284,11 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 				*reinterpret_cast<f32x4 *>(crow + 32 * j + 8 * q) = o;
 			}
 		}
+	}
+	if (GEGLU && rowmax_part != nullptr) {
+		// the consumer quantises these rows next: leave max|row| over this tile's columns for it
+		omax = fmaxf(omax, tg_red_partner<32>(omax));
+		if (hb == 0) rowmax_part[(size_t)tile * Mpad + m] = omax;
 	}
 }
 
@@ -264,29 +298,38 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 size_t tg_gemm_mfma_apack_bytes(int M, int K) { return (size_t)((M + 127) / 128) * 128 * (size_t)K * 3; }
 size_t tg_gemm_mfma_rows(int M) { return (size_t)((M + 127) / 128) * 128; }
 
-// A [M][lda] fp32 -> digit planes + row factors; rowfac holds 2 * tg_gemm_mfma_rows(M) floats (multipliers, then inverses)
-void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, hipStream_t s) {
+// A [M][lda] fp32 -> digit planes + row factors; rowfac holds 2 * tg_gemm_mfma_rows(M) floats (multipliers, then inverses).
+// rowmax_part != nullptr: [nparts][tg_gemm_mfma_rows(M)] partial row maxima left by the producer of A (no pass over A for them).
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax_part, int nparts,
+                          hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(M);
-	hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)(Mpad / 4)), dim3(GNT), 0, s, A, lda, M, K, rowfac, rowfac + Mpad, Mpad);
+	if (rowmax_part != nullptr)
+		hipLaunchKernelGGL(row_scale_parts_kernel, dim3((unsigned)(Mpad / 32)), dim3(GNT), 0, s, rowmax_part, nparts, M, rowfac, rowfac + Mpad,
+		                   Mpad);
+	else
+		hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)(Mpad / 4)), dim3(GNT), 0, s, A, lda, M, K, rowfac, rowfac + Mpad, Mpad);
 	hipLaunchKernelGGL(quant_pack_kernel, dim3((unsigned)(Mpad / 32), (unsigned)(K / 128)), dim3(GNT), 0, s, A, lda, M, K, rowfac, apack);
 }
 
-// ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns
+// ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns;
+// rowmax_part (GEGLU only, may be null): [ntiles][tg_gemm_mfma_rows(M)] floats, max|C[m][tile's columns]|
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
-                         int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, hipStream_t s) {
+                         int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
+                         hipStream_t s) {
 	const unsigned mblocks = (unsigned)((M + 127) / 128);
-	const float *rowinv = rowfac + tg_gemm_mfma_rows(M);
+	const int Mpad = (int)tg_gemm_mfma_rows(M);
+	const float *rowinv = rowfac + Mpad;
 	const dim3 grid((unsigned)ntiles, mblocks), block(GNT);
 	int e = 0;
 	const float ginv = (epi == TG_EPI_GEGLU && geps > 0.0f && frexpf(geps, &e) == 0.5f && e > -100 && e < 100) ? 1.0f / geps : 0.0f;
 	if (epi == TG_EPI_GEGLU && lut_size <= LUT_LDS_MAX) {
 		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
-		                   gmin, geps, ginv, lut_size);
+		                   gmin, geps, ginv, lut_size, rowmax_part, Mpad);
 	} else if (epi == TG_EPI_GEGLU) {
 		hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
-		                   gmin, geps, ginv, lut_size);
+		                   gmin, geps, ginv, lut_size, rowmax_part, Mpad);
 	} else {
 		hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * TG_CT, lut, gmin,
-		                   geps, ginv, lut_size);
+		                   geps, ginv, lut_size, (float *)nullptr, Mpad);
 	}
 }

@@ -172,7 +172,7 @@ bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector
 size_t tg_attn_prefill_part_floats(int nslots);
 size_t tg_attn_prefill_ml_floats(int nslots);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, hipStream_t s);
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, hipStream_t s);
 // exact-order GEMM on the GEMV tiling (ntiles tiles of Ct columns): C[m][N] = (A[m][K] . W) * scales; epi GEGLU writes C[m][N/2]
 void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
@@ -196,9 +196,11 @@ void tg_launch_retile_mfma(int8_t *dst, float *dst_scales, const TgColMap &m, in
 // int8 MFMA prefill GEMM (tg_gemm_mfma.hip): A is first quantised per row into three int8 digit planes in operand order
 size_t tg_gemm_mfma_apack_bytes(int M, int K);
 size_t tg_gemm_mfma_rows(int M);  // rowfac scratch holds twice this many floats
-void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, hipStream_t s);
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax_part, int nparts,
+                          hipStream_t s);
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
-                         int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
+                         int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
+                         hipStream_t s);
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global load of the wave (its fence covers all address spaces), which would drain a software pipeline
