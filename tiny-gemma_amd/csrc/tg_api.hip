@@ -35,6 +35,7 @@ int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
 int g_n_cu = 256;
+int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 
 bool legal_in(int d) { return d == 640 || d == 2048 || d == 1024 || d == 256 || d == 1152 || d == 6912; }            // static_switch.hpp:7-30
@@ -844,13 +845,16 @@ int tg_session_position(const tg_session *s) { return s ? s->pos : -1; }
 // ---------------------------------------------------------------------------------------------
 // forward_decode: 5 launches per layer + 1 for the head
 // ---------------------------------------------------------------------------------------------
-// Keys per attention workgroup.  Up to 4096 keys the chunk is sized so that at most
-// TG_ATTN_MERGE_MAX partials result, which the output projection merges in its prologue;
-// beyond that 128-key chunks are used and a merge launch folds the partials first.
+// Keys per attention workgroup.  While TG_ATTN_MERGE_MAX workgroups of at most g_attn_merge_chunk keys cover the
+// context, the output projection merges their partials in its prologue.  Longer contexts are bound by how long one
+// workgroup walks its keys, so they are spread over up to TG_ATTN_MAX_BLOCKS workgroups (32 keys each or more) and a
+// merge launch folds the partials first: the extra launch costs less than a few dozen keys per workgroup.
 static int attn_chunk_for(int valid, bool *needs_merge) {
-	int c = ((valid + TG_ATTN_MERGE_MAX - 1) / TG_ATTN_MERGE_MAX + 15) / 16 * 16;
-	*needs_merge = c > 256;
-	return *needs_merge ? 128 : c;
+	auto up16 = [](int x) { return (x + 15) / 16 * 16; };
+	const int c = up16((valid + TG_ATTN_MERGE_MAX - 1) / TG_ATTN_MERGE_MAX);
+	*needs_merge = c > g_attn_merge_chunk;
+	if (!*needs_merge) return c;
+	return std::max(32, up16((valid + TG_ATTN_MAX_BLOCKS - 1) / TG_ATTN_MAX_BLOCKS));
 }
 
 // Event pool for tg_decode_profile: one event before every launch of a step plus one at the end.
@@ -941,7 +945,7 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		TG_MARK(TG_KC_ATTN);
 		// a captured step is replayed at later positions with the same chunk: launch the largest grid that
 		// chunk can need (workgroups past the valid keys exit at once)
-		const int nblk = full_grid ? (needs_merge ? (a.max_pos + a.chunk - 1) / a.chunk : TG_ATTN_MERGE_MAX)
+		const int nblk = full_grid ? (needs_merge ? std::min(TG_ATTN_MAX_BLOCKS, (a.max_pos + a.chunk - 1) / a.chunk) : TG_ATTN_MERGE_MAX)
 		                           : (valid + a.chunk - 1) / a.chunk;
 		TG_DO(TG_KC_ATTN, l, tg_launch_attn_decode(a, nblk, g_stream); if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream));
 		// --- merge of the attention partials + O projection (modules.hpp:161-164)
@@ -1087,6 +1091,12 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
 		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	StepOnly only{kernel_class, kernel_class == TG_KC_LMHEAD ? 0 : layer, repeat};
 	return enqueue_decode_step(s, nullptr, false, &only);
+}
+
+int tg_set_attn_merge_chunk(int keys) {
+	if (keys < 32 || keys > 256 || keys % 16) return tg_fail(TG_ERR_BAD_ARG, "keys per workgroup: a multiple of 16 in 32..256");
+	g_attn_merge_chunk = keys;
+	return TG_OK;
 }
 
 int tg_set_taps(int enable) {

@@ -277,14 +277,24 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, cons
 }
 
 // Long contexts only: folds more than TG_ATTN_MERGE_MAX partials into one (max 0, sum 1, normalised
-// output) so that the consumer's merge stays small.  One workgroup per head.
+// output) so that the consumer's merge stays small.  Workgroup = (head, 64 of its 256 dims); lane = dim, the
+// four waves share the partials round-robin and meet in LDS.
 __global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, float *merged_acc, float *merged_ml) {
 	__shared__ float wg[TG_ATTN_MAX_BLOCKS];
 	__shared__ float sred[4];
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x;
+	__shared__ float osum[4][64];
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x, d = 64 * (int)blockIdx.y + lane;
 	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;
 	const int nb = (valid + a.chunk - 1) / a.chunk;
+	// the first partials of this wave are requested before the weights are known
+	constexpr int U = 8;
+	float v[U];
+#pragma unroll
+	for (int u = 0; u < U; u++) {
+		const int b = w + 4 * u;
+		v[u] = a.part_acc[((size_t)(b < nb ? b : 0) * NH + h) * HD + d];
+	}
 	const bool ok = tid < nb;
 	const float m = ok ? a.part_ml[((size_t)tid * NH + h) * 2] : -INFINITY;
 	const float l = ok ? a.part_ml[((size_t)tid * NH + h) * 2 + 1] : 0.0f;
@@ -298,20 +308,31 @@ __global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, f
 	if (lane == 0) sred[w] = L;
 	__syncthreads();
 	L = (sred[0] + sred[1]) + (sred[2] + sred[3]);
-	wg[tid] = e / L;
+	wg[tid] = e / L;  // 0 beyond nb
 	__syncthreads();
 	float o = 0.0f;
-	for (int b0 = 0; b0 < nb; b0 += 8) {
-		float v[8];
+	for (int b0 = w; b0 < nb; b0 += 4 * U) {
+		float nx[U];
 #pragma unroll
-		for (int u = 0; u < 8; u++) v[u] = (b0 + u < nb) ? a.part_acc[((size_t)(b0 + u) * NH + h) * HD + tid] : 0.0f;
+		for (int u = 0; u < U; u++) {
+			const int b = b0 + 4 * (U + u);
+			nx[u] = a.part_acc[((size_t)(b < nb ? b : 0) * NH + h) * HD + d];
+		}
 #pragma unroll
-		for (int u = 0; u < 8; u++) o = fmaf(v[u], wg[(b0 + u < nb) ? b0 + u : 0], o);
+		for (int u = 0; u < U; u++) {
+			const int b = b0 + 4 * u;
+			o = fmaf(v[u], b < nb ? wg[b] : 0.0f, o);
+			v[u] = nx[u];
+		}
 	}
-	merged_acc[h * HD + tid] = o;
-	if (tid == 0) {
-		merged_ml[h * 2 + 0] = 0.0f;
-		merged_ml[h * 2 + 1] = 1.0f;
+	osum[w][lane] = o;
+	__syncthreads();
+	if (w == 0) {
+		merged_acc[h * HD + d] = (osum[0][lane] + osum[1][lane]) + (osum[2][lane] + osum[3][lane]);
+		if (lane == 0 && blockIdx.y == 0) {
+			merged_ml[h * 2 + 0] = 0.0f;
+			merged_ml[h * 2 + 1] = 1.0f;
+		}
 	}
 }
 
@@ -358,7 +379,7 @@ void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t
 }
 
 void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s) {
-	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH), dim3(ANT), 0, s, a, merged_acc, merged_ml);
+	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, HD / 64), dim3(ANT), 0, s, a, merged_acc, merged_ml);
 }
 
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
