@@ -161,7 +161,7 @@ int tg_set_prefetch_blocks(int n);
  * (q|k|v touches o and up|gate, attention touches down). */
 int tg_set_prefetch_plan(int plan);
 /* tuning knob: decode attention gives a workgroup at most this many keys (multiple of 16 in 32..256, default 48) while 16
- * workgroups cover the context; longer contexts use up to 256 workgroups and one extra merge launch. */
+ * workgroups cover the context; longer contexts use up to 1024 workgroups of 32 keys and one extra merge launch. */
 int tg_set_attn_merge_chunk(int keys);
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out);
 

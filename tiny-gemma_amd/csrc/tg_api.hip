@@ -255,7 +255,7 @@ struct tg_session {
 	float *xr = nullptr;      // [(2L+1)][hidden] residual stream after every block of the last decode
 	float *qkv = nullptr, *attn_out = nullptr, *o_out = nullptr, *hbuf = nullptr, *d_out = nullptr, *logits = nullptr;
 	float *part_acc = nullptr, *part_ml = nullptr;      // attention partials [nb][4][256], [nb][4][2]
-	float *merged_acc = nullptr, *merged_ml = nullptr;  // long contexts: partials folded into one
+	float *merged_acc = nullptr, *merged_ml = nullptr;  // long contexts: every TG_ATTN_FOLD partials folded into one
 	float *blk_val = nullptr;
 	int *blk_idx = nullptr;
 	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token
@@ -808,8 +808,8 @@ int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin,
 	TG_ALLOC(s->logits, sizeof(float) * (size_t)c.n_vocab);
 	TG_ALLOC(s->part_acc, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * hd);
 	TG_ALLOC(s->part_ml, sizeof(float) * (size_t)ATTN_MAX_BLOCKS * c.n_head * 2);
-	TG_ALLOC(s->merged_acc, sizeof(float) * (size_t)c.n_head * hd);
-	TG_ALLOC(s->merged_ml, sizeof(float) * (size_t)c.n_head * 2);
+	TG_ALLOC(s->merged_acc, sizeof(float) * (size_t)TG_ATTN_MERGE_MAX * c.n_head * hd);
+	TG_ALLOC(s->merged_ml, sizeof(float) * (size_t)TG_ATTN_MERGE_MAX * c.n_head * 2);
 	TG_ALLOC(s->blk_val, sizeof(float) * (size_t)m->lm.ntiles);
 	TG_ALLOC(s->blk_idx, sizeof(int) * (size_t)m->lm.ntiles);
 	TG_ALLOC(s->ctr, sizeof(int) * 8);
@@ -848,7 +848,7 @@ int tg_session_position(const tg_session *s) { return s ? s->pos : -1; }
 // Keys per attention workgroup.  While TG_ATTN_MERGE_MAX workgroups of at most g_attn_merge_chunk keys cover the
 // context, the output projection merges their partials in its prologue.  Longer contexts are bound by how long one
 // workgroup walks its keys, so they are spread over up to TG_ATTN_MAX_BLOCKS workgroups (32 keys each or more) and a
-// merge launch folds the partials first: the extra launch costs less than a few dozen keys per workgroup.
+// merge launch folds every TG_ATTN_FOLD partials into one first: the extra launch costs less than a few dozen keys per workgroup.
 static int attn_chunk_for(int valid, bool *needs_merge) {
 	auto up16 = [](int x) { return (x + 15) / 16 * 16; };
 	const int c = up16((valid + TG_ATTN_MERGE_MAX - 1) / TG_ATTN_MERGE_MAX);
@@ -947,13 +947,13 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		// chunk can need (workgroups past the valid keys exit at once)
 		const int nblk = full_grid ? (needs_merge ? std::min(TG_ATTN_MAX_BLOCKS, (a.max_pos + a.chunk - 1) / a.chunk) : TG_ATTN_MERGE_MAX)
 		                           : (valid + a.chunk - 1) / a.chunk;
-		TG_DO(TG_KC_ATTN, l, tg_launch_attn_decode(a, nblk, g_stream); if (needs_merge) tg_launch_attn_merge(a, s->merged_acc, s->merged_ml, g_stream));
+		TG_DO(TG_KC_ATTN, l, tg_launch_attn_decode(a, nblk, g_stream); if (needs_merge) tg_launch_attn_merge(a, nblk, s->merged_acc, s->merged_ml, g_stream));
 		// --- merge of the attention partials + O projection (modules.hpp:161-164)
 		g = gemv_base(Ld.o);
 		g.pos = s->ctr;
 		g.host_pos = a.host_pos;
 		g.attn_max_pos = a.max_pos;
-		g.attn_chunk = needs_merge ? a.max_pos : a.chunk;  // merged: a single partial
+		g.attn_chunk = needs_merge ? TG_ATTN_FOLD * a.chunk : a.chunk;  // folded: one partial per TG_ATTN_FOLD workgroups
 		g.part_acc = needs_merge ? s->merged_acc : s->part_acc;
 		g.part_ml = needs_merge ? s->merged_ml : s->part_ml;
 		g.y = s->o_out;

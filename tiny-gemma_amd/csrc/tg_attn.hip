@@ -276,62 +276,52 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, cons
 	}
 }
 
-// Long contexts only: folds more than TG_ATTN_MERGE_MAX partials into one (max 0, sum 1, normalised
-// output) so that the consumer's merge stays small.  Workgroup = (head, 64 of its 256 dims); lane = dim, the
-// four waves share the partials round-robin and meet in LDS.
+// Long contexts only: folds every TG_ATTN_FOLD consecutive partials into one partial of the same form (maximum, sum,
+// un-normalised output relative to that maximum), so that the consumer's merge stays at TG_ATTN_MERGE_MAX partials of
+// TG_ATTN_FOLD * chunk keys each.  Workgroup = (head, 64 of its 256 dims, group of partials); lane = dim, the four waves
+// share the group's partials round-robin and meet in LDS.
 __global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, float *merged_acc, float *merged_ml) {
-	__shared__ float wg[TG_ATTN_MAX_BLOCKS];
-	__shared__ float sred[4];
+	__shared__ float wg[TG_ATTN_FOLD];
 	__shared__ float osum[4][64];
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x, d = 64 * (int)blockIdx.y + lane;
+	__shared__ float s_ml[2];
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, h = blockIdx.x, d = 64 * (int)blockIdx.y + lane, grp = blockIdx.z;
 	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;
-	const int nb = (valid + a.chunk - 1) / a.chunk;
-	// the first partials of this wave are requested before the weights are known
-	constexpr int U = 8;
+	const int b_lo = grp * TG_ATTN_FOLD;
+	const int nb = min((valid + a.chunk - 1) / a.chunk - b_lo, TG_ATTN_FOLD);  // partials of this group
+	if (nb <= 0) return;  // uniform over the workgroup: a fixed-size grid launched for a longer context
+	// the wave's partials are requested before their weights are known: wave w takes b_lo + w, + 4, ...
+	constexpr int U = TG_ATTN_FOLD / 4;
 	float v[U];
 #pragma unroll
 	for (int u = 0; u < U; u++) {
 		const int b = w + 4 * u;
-		v[u] = a.part_acc[((size_t)(b < nb ? b : 0) * NH + h) * HD + d];
+		v[u] = a.part_acc[((size_t)(b_lo + (b < nb ? b : 0)) * NH + h) * HD + d];
 	}
-	const bool ok = tid < nb;
-	const float m = ok ? a.part_ml[((size_t)tid * NH + h) * 2] : -INFINITY;
-	const float l = ok ? a.part_ml[((size_t)tid * NH + h) * 2 + 1] : 0.0f;
-	float M = wmax(m);
-	if (lane == 0) sred[w] = M;
-	__syncthreads();
-	M = fmaxf(fmaxf(sred[0], sred[1]), fmaxf(sred[2], sred[3]));
-	__syncthreads();
-	const float e = ok ? expf(m - M) : 0.0f;
-	float L = wsum(l * e);
-	if (lane == 0) sred[w] = L;
-	__syncthreads();
-	L = (sred[0] + sred[1]) + (sred[2] + sred[3]);
-	wg[tid] = e / L;  // 0 beyond nb
+	if (w == 0) {
+		const bool ok = lane < nb;  // TG_ATTN_FOLD == 64: one partial per lane
+		const float m = ok ? a.part_ml[((size_t)(b_lo + lane) * NH + h) * 2] : -INFINITY;
+		const float l = ok ? a.part_ml[((size_t)(b_lo + lane) * NH + h) * 2 + 1] : 0.0f;
+		const float M = wmax(m);
+		const float e = ok ? expf(m - M) : 0.0f;
+		const float L = wsum(l * e);
+		wg[lane] = e;
+		if (lane == 0) {
+			s_ml[0] = M;
+			s_ml[1] = L;
+		}
+	}
 	__syncthreads();
 	float o = 0.0f;
-	for (int b0 = w; b0 < nb; b0 += 4 * U) {
-		float nx[U];
 #pragma unroll
-		for (int u = 0; u < U; u++) {
-			const int b = b0 + 4 * (U + u);
-			nx[u] = a.part_acc[((size_t)(b < nb ? b : 0) * NH + h) * HD + d];
-		}
-#pragma unroll
-		for (int u = 0; u < U; u++) {
-			const int b = b0 + 4 * u;
-			o = fmaf(v[u], b < nb ? wg[b] : 0.0f, o);
-			v[u] = nx[u];
-		}
-	}
+	for (int u = 0; u < U; u++) o = fmaf(v[u], wg[w + 4 * u], o);  // weight 0 beyond nb
 	osum[w][lane] = o;
 	__syncthreads();
 	if (w == 0) {
-		merged_acc[h * HD + d] = (osum[0][lane] + osum[1][lane]) + (osum[2][lane] + osum[3][lane]);
+		merged_acc[((size_t)grp * NH + h) * HD + d] = (osum[0][lane] + osum[1][lane]) + (osum[2][lane] + osum[3][lane]);
 		if (lane == 0 && blockIdx.y == 0) {
-			merged_ml[h * 2 + 0] = 0.0f;
-			merged_ml[h * 2 + 1] = 1.0f;
+			merged_ml[((size_t)grp * NH + h) * 2 + 0] = s_ml[0];
+			merged_ml[((size_t)grp * NH + h) * 2 + 1] = s_ml[1];
 		}
 	}
 }
@@ -378,8 +368,11 @@ void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t
 	                   a.rms_k, a.cos_t, a.sin_t, a.host_pos, a.host_bp, a);
 }
 
-void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s) {
-	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, HD / 64), dim3(ANT), 0, s, a, merged_acc, merged_ml);
+// nblk: workgroups of the attention launch whose partials are folded
+void tg_launch_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, hipStream_t s) {
+	static_assert(TG_ATTN_FOLD == 64 && TG_ATTN_MAX_BLOCKS == TG_ATTN_FOLD * TG_ATTN_MERGE_MAX, "one partial per lane; the consumer merges the rest");
+	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, HD / 64, (unsigned)((nblk + TG_ATTN_FOLD - 1) / TG_ATTN_FOLD)), dim3(ANT), 0, s, a,
+	                   merged_acc, merged_ml);
 }
 
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,

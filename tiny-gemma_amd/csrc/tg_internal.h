@@ -31,7 +31,8 @@
 #define TG_MAX_K 6912        // largest reduction length (1B down projection)
 #define TG_MAX_HIDDEN 1152   // largest residual-stream width
 #define TG_ATTN_MERGE_MAX 16 // attention partials the output projection merges in its prologue
-#define TG_ATTN_MAX_BLOCKS 256  // attention workgroups per launch, upper bound
+#define TG_ATTN_MAX_BLOCKS 1024 // attention workgroups per launch, upper bound
+#define TG_ATTN_FOLD 64         // partials the merge launch folds into one
 
 // ---- weight prefetch riding along with a launch ------------------------------------------------
 // Batch-1 decode is a chain of ~130 dependent, latency-bound launches per token during which HBM
@@ -140,7 +141,7 @@ enum { TG_ROLE_PLAIN = 0, TG_ROLE_QKV_EMBED, TG_ROLE_QKV, TG_ROLE_OPROJ, TG_ROLE
        TG_ROLE_LMHEAD_PLAIN };
 void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s);
 void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s);
-void tg_launch_attn_merge(const TgAttnDecode &a, float *merged_acc, float *merged_ml, hipStream_t s);
+void tg_launch_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, hipStream_t s);
 void tg_launch_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log, int advance, hipStream_t s);
 // min-p sampling (tg_sample.hip): n a multiple of 1024; scratch probs[n], seg[tg_minp_segments(n)], bsum/bmax[tg_minp_blocks(n)];
 // mode 0 = decode step (append + advance), 1 = replace the token written last, 2 = out_tok only;
