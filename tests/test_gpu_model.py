@@ -253,8 +253,10 @@ def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
             assert np.array_equal(a, b)
 
 
-def test_long_context_merge_path(tg, oracle, weight_images, tables):
-    """More than 4096 keys on a global layer: 128-key chunks plus the merge launch."""
+@pytest.mark.parametrize("n_prompt", [1000, 4100])
+def test_long_context_merge_path(tg, oracle, weight_images, tables, n_prompt):
+    """More than 768 keys on a global layer: 32-key workgroups plus the merge launch, which folds groups of 64
+    partials (1000 keys: one partly filled group; 4100 keys: two full groups and a group of one)."""
     cfg_o = gi.oracle_config("270m", 2)
     cfg_o.pattern = 2  # layer 0 local, layer 1 global
     image = oracle.generate_weights(cfg_o, 21)
@@ -265,7 +267,7 @@ def test_long_context_merge_path(tg, oracle, weight_images, tables):
     table = oracle.gelu_table(-4.0, 4.0, 1 << 20)
     sess = model.session(rope=tables[0], rope_sw=tables[1], gelu_table=table)
     osess = oracle.model(cfg_o, image=image).session(-4.0, 4.0, 1 << 20)
-    prompt = gi.prompt_ids(21, 4100)
+    prompt = gi.prompt_ids(21, n_prompt)
     tok, logits = sess.prefill(prompt)
     otok, ologits, _ = osess.prefill(prompt)
     assert tok == otok and normrel(logits, ologits) < 5e-5
