@@ -339,6 +339,12 @@ class Ref:
         L.ref_prefill.argtypes = [C.c_void_p, c_i32p, C.c_int, c_f32p, c_i32p, c_f32p]
         L.ref_decode.argtypes = [C.c_void_p, C.c_int, c_f32p, c_i32p, c_f32p]
         L.ref_kv_read.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
+        L.ref_tok_create.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.ref_tok_create.restype = C.c_void_p
+        L.ref_tok_destroy.argtypes = [C.c_void_p]
+        L.ref_tok_encode.argtypes = [C.c_void_p, C.c_char_p, C.c_int, c_i32p, C.c_int]
+        L.ref_tok_decode_piece.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.c_int]
+        L.ref_tok_decode.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_char_p, C.c_int]
 
     def qgemv(self, x, W, s, logits=False):
         inn, out = W.shape
@@ -413,6 +419,9 @@ class Ref:
         idx = self.L.ref_minp_logits(_f(p), minp, temp, randf)
         return idx, p
 
+    def tokenizer(self, path, bos_id, eos_id, vocab_size, chat_format):
+        return _RefTokenizer(self, path, bos_id, eos_id, vocab_size, chat_format)
+
     def model(self, cfg, path):
         return _RefModel(self, cfg, path)
 
@@ -457,4 +466,44 @@ class _RefSession(_Session):
     def __del__(self):
         if getattr(self, "h", None):
             self.L.ref_session_destroy(self.h)
+            self.h = None
+
+
+class _RefTokenizer:
+    """sentencepiece::Tokenizer of the reference (tokenizer.hpp), bytes in / bytes out."""
+
+    def __init__(self, ref, path, bos_id, eos_id, vocab_size, chat_format):
+        self.L = ref.L
+        self.h = self.L.ref_tok_create(str(path).encode(), bos_id, eos_id, vocab_size, int(bool(chat_format)))
+        if not self.h:
+            raise RuntimeError("Cannot open model file: " + str(path))
+
+    def encode(self, text):
+        cap = 16 + 4 * len(text)
+        ids = np.empty(cap, np.int32)
+        n = self.L.ref_tok_encode(self.h, text, len(text), _i(ids), cap)
+        assert n <= cap
+        return ids[:n].copy()
+
+    def decode_piece(self, token, prev_token):
+        buf = C.create_string_buffer(4096)
+        n = self.L.ref_tok_decode_piece(self.h, int(token), int(prev_token), buf, 4096)
+        if n == -2:
+            raise ValueError("the reference threw std::invalid_argument")
+        assert n >= 0
+        return buf.raw[:n]
+
+    def decode(self, ids):
+        ids = np.ascontiguousarray(ids, np.int32)
+        cap = 1 << 20
+        buf = C.create_string_buffer(cap)
+        n = self.L.ref_tok_decode(self.h, _i(ids), ids.size, buf, cap)
+        if n == -2:
+            raise ValueError("the reference threw std::invalid_argument")
+        assert 0 <= n <= cap
+        return buf.raw[:n]
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.ref_tok_destroy(self.h)
             self.h = None

@@ -12,6 +12,7 @@
 //
 // Every entry point names the reference function it forwards to.
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -20,6 +21,7 @@
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "transformer.hpp"  // pulls in linalg/tensor/ops/decode/modules/config/tokenizer
 
@@ -311,6 +313,48 @@ int ref_kv_read(void *sp, int layer, float *keys, float *values, int *position_p
 	if (buffer_ptr) *buffer_ptr = kv->buffer_ptr;
 	if (max_pos) *max_pos = kv->max_pos;
 	return 0;
+}
+
+// ---- sentencepiece::Tokenizer (tokenizer.hpp:14-239) ----
+void *ref_tok_create(const char *path, int bos_id, int eos_id, int vocab_size, int chat_format) {
+	try {
+		return new sentencepiece::Tokenizer(path, bos_id, eos_id, vocab_size, chat_format != 0);
+	} catch (const std::exception &) {
+		return nullptr;
+	}
+}
+void ref_tok_destroy(void *tp) { delete static_cast<sentencepiece::Tokenizer *>(tp); }
+// Tokenizer::encode (tokenizer.hpp:113-201); text is n bytes (may hold any byte but is passed on as a std::string).
+// Returns the number of ids; writes at most cap of them.
+int ref_tok_encode(void *tp, const char *text, int n, int *ids, int cap) {
+	std::vector<int> v = static_cast<sentencepiece::Tokenizer *>(tp)->encode(std::string(text, (size_t)n));
+	for (int i = 0; i < (int)v.size() && i < cap; i++) ids[i] = v[i];
+	return (int)v.size();
+}
+// Tokenizer::decode(token, prev_token) (tokenizer.hpp:203-218).  Returns the piece length; writes at most cap bytes.
+// -2: the reference threw std::invalid_argument, -3: another exception.
+int ref_tok_decode_piece(void *tp, int token, int prev_token, char *out, int cap) {
+	try {
+		std::string piece = static_cast<sentencepiece::Tokenizer *>(tp)->decode(token, prev_token);
+		std::memcpy(out, piece.data(), std::min((size_t)cap, piece.size()));
+		return (int)piece.size();
+	} catch (const std::invalid_argument &) {
+		return -2;
+	} catch (const std::exception &) {
+		return -3;
+	}
+}
+// Tokenizer::decode(tokens) (tokenizer.hpp:220-233)
+int ref_tok_decode(void *tp, const int *ids, int n, char *out, int cap) {
+	try {
+		std::string text = static_cast<sentencepiece::Tokenizer *>(tp)->decode(std::vector<int>(ids, ids + n));
+		std::memcpy(out, text.data(), std::min((size_t)cap, text.size()));
+		return (int)text.size();
+	} catch (const std::invalid_argument &) {
+		return -2;
+	} catch (const std::exception &) {
+		return -3;
+	}
 }
 
 }  // extern "C"

@@ -153,3 +153,86 @@ def prompt_ids(seed, n):
 def oracle_config(shape, n_layers):
     from oracle.oracle import named_config
     return named_config(shape, n_layers)
+
+
+# ---- tokenizer (tokenizer.hpp; file format of py/convert.py:83-113) ----
+TOKENIZER_VOCAB = 5000
+TOKENIZER_SEED = 77
+
+
+def tokenizer_vocab(seed=TOKENIZER_SEED, vocab_size=TOKENIZER_VOCAB):
+    """A synthetic vocabulary laid out like Gemma's: specials, <start_of_turn>/<end_of_turn>/newline at 105-107,
+    byte tokens <0x00>..<0xFF> at 238..493, "user" at 2364, "model" at 4368, unique pieces elsewhere.
+    Returns (pieces: list of bytes, scores: float32 array); scores are multiples of 0.5 so that ties occur."""
+    rng = np.random.default_rng(seed)
+    pieces = [None] * vocab_size
+    fixed = {0: b"<pad>", 1: b"<eos>", 2: b"<bos>", 3: b"<unk>", 4: b"<mask>", 105: b"<start_of_turn>", 106: b"<end_of_turn>",
+             107: b"\n", 2364: b"user", 4368: b"model"}
+    for i in range(256):
+        fixed[238 + i] = ("<0x%02X>" % i).encode()
+    fixed[494] = b"<0xabc>"   # three hex digits: still matches the reference's byte pattern
+    fixed[495] = b" <0x41>"   # becomes a byte piece once its leading space is stripped
+    for i, p in fixed.items():
+        pieces[i] = p
+    used = set(fixed.values())
+    letters = "abcdefghijklmnopqrstuvwxyzABCDEFGH0123456789.,;:!?-'\"()"
+    cands = [c.encode() for c in letters] + [b" "]
+    cands += ["é".encode(), "ü".encode(), "ñ".encode(), "日".encode(), "本".encode(), "語".encode(),
+              "\U0001F600".encode(), b"\xf0\x9f\x98\x80\x80"]
+    cands += [(" " + c).encode() for c in "abcdefghijklmnopqrstuvwxyz"]
+    small = "abcdefghij "
+    for a in small:
+        for b in small:
+            cands.append((a + b).encode())
+    while len(cands) < 3 * vocab_size:
+        n = int(rng.integers(3, 9))
+        w = "".join(small[int(k)] for k in rng.integers(0, len(small), n))
+        cands.append(w.encode())
+    it = iter(cands)
+    for i in range(vocab_size):
+        if pieces[i] is None:
+            p = next(it)
+            while p in used:
+                p = next(it)
+            used.add(p)
+            pieces[i] = p
+    scores = (-np.round(rng.uniform(0.0, 20.0, vocab_size) * 2.0) / 2.0).astype(np.float32)
+    for i in fixed:
+        scores[i] = 0.0
+    return pieces, scores
+
+
+def write_tokenizer_file(path, pieces, scores):
+    import struct
+    with open(path, "wb") as f:
+        f.write(struct.pack("I", max(len(p) for p in pieces)))
+        for p, s in zip(pieces, scores):
+            f.write(struct.pack("fI", float(s), len(p)))
+            f.write(p)
+
+
+def tokenizer_texts(seed=TOKENIZER_SEED):
+    """Byte strings to encode: vocabulary words, random letters, UTF-8 (1-4 byte code points), malformed UTF-8."""
+    rng = np.random.default_rng(seed + 1)
+    pieces, _ = tokenizer_vocab()
+    small = "abcdefghij "
+    texts = [b"", b" ", b"a", b"hello world", b"user model\n", "café 日本語 \U0001F600!".encode(),
+             b"\x80\x80\x80", b"a\xc3", b"\xf0\x9f\x98\x80\x80\x80\x80 b", b"\xff\xfe abc", b"<0x41> <bos>"]
+    for _ in range(24):
+        n = int(rng.integers(1, 60))
+        texts.append("".join(small[int(k)] for k in rng.integers(0, len(small), n)).encode())
+    for _ in range(12):
+        words = [pieces[int(k)] for k in rng.integers(496, TOKENIZER_VOCAB, int(rng.integers(2, 12)))]
+        texts.append(b" ".join(words))
+    texts.append("".join(small[int(k)] for k in rng.integers(0, len(small), 1500)).encode())
+    return texts
+
+
+def tokenizer_vocab_full(n=262144):
+    """A full-size vocabulary for the command line front end (it always loads 262144 entries): the 5000 pieces of
+    tokenizer_vocab() followed by unique filler pieces '~' + base-10 digits written with the letters k..t."""
+    pieces, scores = tokenizer_vocab()
+    tr = bytes.maketrans(b"0123456789", b"klmnopqrst")
+    pieces = pieces + [b"~" + str(i).encode().translate(tr) for i in range(len(pieces), n)]
+    scores = np.concatenate([scores, np.full(n - scores.size, -30.0, np.float32)])
+    return pieces, scores

@@ -1,0 +1,194 @@
+"""CPU: the host tokenizer (tiny-gemma_amd/host/tokenizer.hpp) against the reference's sentencepiece::Tokenizer
+(csrc/include/tokenizer.hpp:14-239).
+
+Two checkers: the fixture tests/golden/tokenizer.npz, written by tests/golden/make_tokenizer_golden.py from the
+compiled reference on the synthetic vocabulary of tests/golden_inputs.py, and — where oracle/_ref/libtg_ref.so
+is present — the compiled reference itself, called side by side on further random inputs.  Token ids and bytes
+must be identical, including the cases where the reference throws (byte tokens).  Independent of both, the
+merge rule is checked by brute force on a tiny vocabulary.
+"""
+import ctypes as C
+import hashlib
+import os
+
+import numpy as np
+import pytest
+
+import golden_inputs as gi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHIM = os.path.join(ROOT, "tests", "host", "libtokenizer_shim.so")
+c_i32p = C.POINTER(C.c_int32)
+
+
+class Tok:
+    def __init__(self, path, bos, eos, vocab, chat):
+        if not os.path.exists(SHIM):
+            pytest.fail("tests/host/libtokenizer_shim.so is not built: run __graft_entry__.build()")
+        L = self.L = C.CDLL(SHIM)
+        L.tok_create.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.tok_create.restype = C.c_void_p
+        L.tok_destroy.argtypes = [C.c_void_p]
+        L.tok_encode.argtypes = [C.c_void_p, C.c_char_p, C.c_int, c_i32p, C.c_int]
+        L.tok_decode_piece.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_char_p, C.c_int]
+        L.tok_decode.argtypes = [C.c_void_p, c_i32p, C.c_int, C.c_char_p, C.c_int]
+        L.tok_byte_of.argtypes = [C.c_void_p, C.c_int]
+        self.h = L.tok_create(str(path).encode(), bos, eos, vocab, int(chat))
+        if not self.h:
+            raise RuntimeError("Cannot open model file")
+
+    def encode(self, text):
+        cap = 16 + 4 * len(text)
+        ids = np.empty(cap, np.int32)
+        n = self.L.tok_encode(self.h, text, len(text), ids.ctypes.data_as(c_i32p), cap)
+        assert n <= cap
+        return ids[:n].copy()
+
+    def decode_piece(self, tok, prev):
+        buf = C.create_string_buffer(4096)
+        n = self.L.tok_decode_piece(self.h, int(tok), int(prev), buf, 4096)
+        if n == -2:
+            raise ValueError("std::invalid_argument")
+        assert n >= 0
+        return buf.raw[:n]
+
+    def decode(self, ids):
+        ids = np.ascontiguousarray(ids, np.int32)
+        buf = C.create_string_buffer(1 << 20)
+        n = self.L.tok_decode(self.h, ids.ctypes.data_as(c_i32p), ids.size, buf, 1 << 20)
+        if n == -2:
+            raise ValueError("std::invalid_argument")
+        assert n >= 0
+        return buf.raw[:n]
+
+    def byte_of(self, tok):
+        return self.L.tok_byte_of(self.h, int(tok))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.tok_destroy(self.h)
+
+
+@pytest.fixture(scope="module")
+def tokfile(tmp_path_factory):
+    path = tmp_path_factory.mktemp("tok") / "tok.bin"
+    pieces, scores = gi.tokenizer_vocab()
+    gi.write_tokenizer_file(path, pieces, scores)
+    return path
+
+
+@pytest.fixture(scope="module")
+def tgold():
+    return np.load(os.path.join(ROOT, "tests", "golden", "tokenizer.npz"))
+
+
+@pytest.mark.parametrize("chat", [0, 1])
+def test_encode_and_decode_equal_the_fixture(tokfile, tgold, chat):
+    t = Tok(tokfile, 2, 1, gi.TOKENIZER_VOCAB, chat)
+    offs, ids_all = tgold[f"chat{chat}/offsets"], tgold[f"chat{chat}/ids"]
+    dec_len, dec_all = tgold[f"chat{chat}/decoded_len"], tgold[f"chat{chat}/decoded"].tobytes()
+    dpos = 0
+    for n, text in enumerate(gi.tokenizer_texts()):
+        want = ids_all[offs[n]:offs[n + 1]]
+        got = t.encode(text)
+        assert np.array_equal(got, want), (text[:40], got[:20], want[:20])
+        if dec_len[n] == -2:   # a byte token among the ids: the reference throws std::invalid_argument
+            with pytest.raises(ValueError):
+                t.decode(got)
+        else:
+            assert t.decode(got) == dec_all[dpos:dpos + dec_len[n]]
+            dpos += int(dec_len[n])
+    assert dpos == len(dec_all)
+    if chat:   # <bos> <start_of_turn> user \n ... <end_of_turn> \n <start_of_turn> model \n  (tokenizer.hpp:117-119, 196-198)
+        ids = t.encode(b"")
+        assert ids.tolist() == [2, 105, 2364, 107, 106, 107, 105, 4368, 107]
+
+
+@pytest.mark.parametrize("prev", [1, 5])
+def test_every_piece_decodes_like_the_fixture(tokfile, tgold, prev):
+    t = Tok(tokfile, 2, 1, gi.TOKENIZER_VOCAB, 0)
+    lens, h = [], hashlib.sha256()
+    for tok in range(gi.TOKENIZER_VOCAB):
+        try:
+            p = t.decode_piece(tok, prev)
+            lens.append(len(p))
+            h.update(p)
+        except ValueError:
+            lens.append(-2)
+    assert np.array_equal(np.array(lens, np.int32), tgold[f"piece_len/prev{prev}"])
+    assert h.hexdigest() == str(tgold[f"piece_sha/prev{prev}"])
+    # byte tokens are where the reference throws; byte_of names the byte
+    assert lens[238 + 0x41] == -2 and t.byte_of(238 + 0x41) == 0x41 and t.byte_of(300 + 300) == -1
+    # a leading space is dropped only after token id 1 (tokenizer.hpp:206-208)
+    sp = next(i for i, p in enumerate(gi.tokenizer_vocab()[0]) if p.startswith(b" ") and len(p) > 1 and i > 495)
+    assert (t.decode_piece(sp, 1) == gi.tokenizer_vocab()[0][sp][1:]) and (t.decode_piece(sp, 5) == gi.tokenizer_vocab()[0][sp])
+
+
+def test_side_by_side_with_the_compiled_reference(tokfile, orc):
+    if not orc.Ref.available():
+        pytest.skip("oracle/_ref/libtg_ref.so is not present (no reference checkout at build time)")
+    ref = orc.Ref()
+    rng = np.random.default_rng(5)
+    alphabet = [c.encode() for c in "abcdefghij  \n.,"] + ["é".encode(), "日".encode(), "\U0001F600".encode(), b"\x80", b"\xc3", b"\xf0"]
+    for chat in (0, 1):
+        mine, theirs = Tok(tokfile, 2, 1, gi.TOKENIZER_VOCAB, chat), ref.tokenizer(tokfile, 2, 1, gi.TOKENIZER_VOCAB, chat)
+        for _ in range(150):
+            text = b"".join(alphabet[int(k)] for k in rng.integers(0, len(alphabet), int(rng.integers(0, 80))))
+            a, b = mine.encode(text), theirs.encode(text)
+            assert np.array_equal(a, b), text
+            try:
+                want = theirs.decode(b)
+            except ValueError:
+                with pytest.raises(ValueError):
+                    mine.decode(a)
+            else:
+                assert mine.decode(a) == want
+
+
+def brute_force_encode(pieces, scores, text):
+    """The reference's rule, restated from its description: code points, byte fallback + 3, then repeatedly merge the
+    leftmost best-scored adjacent pair whose concatenation is a vocabulary entry."""
+    idx = {p: i for i, p in reversed(list(enumerate(pieces)))}
+    toks, i = [2], 0
+    while i < len(text):
+        j = i + 1
+        while j < len(text) and (text[j] & 0xC0) == 0x80 and j - i < 4:
+            j += 1
+        cp = text[i:j]
+        toks += [idx[cp]] if cp in idx else [b + 3 for b in cp]
+        i = j
+    while True:
+        best = None
+        for k in range(len(toks) - 1):
+            m = pieces[toks[k]] + pieces[toks[k + 1]]
+            if m in idx and scores[idx[m]] > -1e10 and (best is None or scores[idx[m]] > best[0]):
+                best = (scores[idx[m]], k, idx[m])
+        if best is None:
+            return toks
+        toks[best[1]:best[1] + 2] = [best[2]]
+
+
+def test_merge_rule_by_brute_force(tmp_path):
+    # ties (ab and bc score alike: the left pair wins), a chain (ab + c -> abc only when it outranks bc), fallback bytes
+    pieces = [b"<pad>", b"<eos>", b"<bos>"] + [bytes([i]) + b"?" for i in range(256)] + [b"a", b"b", b"c", b"ab", b"bc", b"abc", b"abcb", b"ca"]
+    scores = np.zeros(len(pieces), np.float32)
+    scores[-5:] = [-1.0, -1.0, -0.5, -3.0, -2.0]
+    path = tmp_path / "t.bin"
+    gi.write_tokenizer_file(path, pieces, scores)
+    t = Tok(path, 2, 1, len(pieces), 0)
+    rng = np.random.default_rng(3)
+    for _ in range(300):
+        text = bytes(rng.choice(list(b"abcx"), int(rng.integers(0, 14))).astype(np.uint8))
+        assert t.encode(text).tolist() == brute_force_encode(pieces, scores, text), text
+    a, b, c, ab, bc = 259, 260, 261, 262, 263
+    assert t.encode(b"abc").tolist() == [2, ab, c] or t.encode(b"abc").tolist() == [2, 264]  # ab first (leftmost tie), then ab+c -> abc
+    assert t.encode(b"abc").tolist() == [2, 264]
+
+
+def test_missing_file_and_short_file(tmp_path):
+    with pytest.raises(RuntimeError):
+        Tok(tmp_path / "nope.bin", 2, 1, 10, 0)
+    pieces, scores = gi.tokenizer_vocab()
+    gi.write_tokenizer_file(tmp_path / "short.bin", pieces[:100], scores[:100])
+    with pytest.raises(RuntimeError):
+        Tok(tmp_path / "short.bin", 2, 1, 5000, 0)

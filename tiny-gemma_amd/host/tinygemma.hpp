@@ -13,6 +13,8 @@
 //   gemma::forward_prefill, forward_decode        transformer.hpp:22-165
 //   ops::argmax_logits, ops::minp_logits          ops.hpp:744, 762
 //   gemma::generate_greedy, gemma::generate_ids   transformer.hpp:167-258 on token ids (argmax / min-p branch)
+//   gemma::generate                               transformer.hpp:167-258 on text, streaming (with tokenizer.hpp)
+//   sentencepiece::Tokenizer                      tokenizer.hpp:14-239 (in host/tokenizer.hpp)
 //
 // Errors: the reference throws std::runtime_error for an unknown dimension ("Unsupported ROW/COL
 // dimension: N") and an unopenable weight file ("Could not open file."), and assert()s on shape
@@ -22,7 +24,11 @@
 
 #include <cmath>
 #include <cstdint>
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
 #include <cstring>
+#include <iostream>
 #include <memory>
 #include <random>
 #include <stdexcept>
@@ -32,6 +38,7 @@
 #include <vector>
 
 #include "../../include/tinygemma_hip.h"
+#include "tokenizer.hpp"
 
 namespace tinygemma {
 
@@ -231,6 +238,86 @@ inline std::tuple<int, std::vector<int>, float, float> generate_ids(const std::v
 	double sp = 0, sd = 0;
 	check(tg_generate(d.session, prompt.data(), (int)prompt.size(), n_decode, minp, temp, randf.data(), ids.data(), &sp, &sd));
 	return {n_decode, ids, (float)sp, (float)sd};
+}
+
+// gemma::generate (transformer.hpp:167-258): tokenize, print the prompt, prefill, then up to n_decode steps, every
+// token printed as it is produced; returns {decode steps completed, generated text, prefill seconds, decode seconds}
+// with the reference's timing boundaries (tokenizing and the first token belong to the prefill time).  minp >= 1 is
+// greedy, else every token is drawn with ops::minp_logits and a uniform number from a std::mt19937 seeded from
+// std::random_device, as in the reference.  The decode loop runs on the device in bursts of `burst` tokens (the ids
+// come back once per burst, so text appears burst by burst; 1 = token by token); with terminate_on_end the text
+// stops before the first <end_of_turn> and the count is that of the steps before it, as in the reference.
+// Where the reference's tokenizer throws on a byte token (see tokenizer.hpp) the byte itself is printed.
+inline std::tuple<int, std::string, float, float> generate(std::string prompt, int n_decode, sentencepiece::Tokenizer *tokenizer,
+                                                           Transformer *t, const float minp, const float temp,
+                                                           const bool terminate_on_end, int burst = 16) {
+	using clk = std::chrono::high_resolution_clock;
+	auto t_prefill_s = clk::now();
+	std::random_device rd;
+	std::mt19937 gen(rd());
+	std::uniform_real_distribution<float> unif(0.0, 1.0);
+	const bool sampling = minp < 1;
+
+	std::vector<int> ids = tokenizer->encode(prompt);
+	const size_t prompt_len = ids.size();
+	std::string decoded;
+	decoded.reserve((size_t)std::max(n_decode, 0));
+	printf("Prompt length: %lu\n", (unsigned long)prompt_len);
+	std::cout << tokenizer->decode(ids);
+
+	auto piece_of = [&](int token, int prev) -> std::string {
+		try {
+			return tokenizer->decode(token, prev);
+		} catch (const std::invalid_argument &) {
+			const int b = tokenizer->byte_of(token);
+			return b >= 0 ? std::string(1, (char)b) : std::string();
+		}
+	};
+
+	decode::RoPE rope(&t->cfg, false), rope_sw(&t->cfg, true);
+	lut::GeLUTable table{-4.0, 4.0, 1024};  // transformer.hpp:197
+	decode::DecodeState d(1, &t->cfg);
+	bind_session(t, &d, &rope, &rope_sw, &table);
+
+	std::vector<float> randf((size_t)std::max(n_decode, 0) + 1, 0.0f);
+	if (sampling)
+		for (float &r : randf) r = unif(gen);
+	std::vector<int> out((size_t)std::max(n_decode, 0) + 1);
+	// prefill and the first token (from the prefill logits)
+	check(tg_generate(d.session, ids.data(), (int)prompt_len, 0, minp, temp, randf.data(), out.data(), nullptr, nullptr));
+	int prev_token = ids[ids.size() - 1];
+	std::cout << piece_of(out[0], prev_token) << std::flush;
+	prev_token = out[0];
+	auto t_prefill_e = clk::now();
+
+	auto t_decode_s = clk::now();
+	int done = 0;
+	bool stop = false;
+	if (burst < 1) burst = 1;
+	while (done < n_decode && !stop) {
+		const int n = std::min(burst, n_decode - done);
+		if (sampling) check(tg_decode_enqueue_sampled(d.session, n, minp, temp, randf.data() + 1 + done));
+		else check(tg_decode_enqueue(d.session, n));
+		int got = 0;
+		check(tg_session_read_ids(d.session, out.data(), done + 1 + n, &got));
+		if (got != done + 1 + n) throw std::runtime_error("token log incomplete");
+		for (int i = 0; i < n; i++) {
+			const int tok = out[(size_t)done + 1];
+			if (terminate_on_end && tok == tokenizer->get_eot_id()) {
+				stop = true;
+				break;
+			}
+			const std::string piece = piece_of(tok, prev_token);
+			decoded.append(piece);
+			std::cout << piece << std::flush;
+			prev_token = tok;
+			done++;
+		}
+	}
+	auto t_decode_e = clk::now();
+	const double s_prefill = std::chrono::duration<double>(t_prefill_e - t_prefill_s).count();
+	const double s_decode = std::chrono::duration<double>(t_decode_e - t_decode_s).count();
+	return {done, decoded, (float)s_prefill, (float)s_decode};
 }
 }  // namespace gemma
 
