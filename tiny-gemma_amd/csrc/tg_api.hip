@@ -1099,6 +1099,11 @@ int tg_set_attn_merge_chunk(int keys) {
 	return TG_OK;
 }
 
+int tg_set_attn_prefill_mode(int bf16x3) {
+	g_attn_prefill_bf16x3 = bf16x3 != 0;
+	return TG_OK;
+}
+
 int tg_set_taps(int enable) {
 	g_keep_taps = enable != 0;
 	return TG_OK;

@@ -210,6 +210,266 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 	}
 }
 
+// ---- the same computation on the bf16 matrix cores, fp32-accurate -------------------------------------------
+// An fp32 number is the sum of three bf16 numbers (8 + 8 + 8 significant bits): x = h + m + l with h = bf16(x),
+// m = bf16(x - h), l = bf16(x - h - m), the two differences exact.  A product of two such sums keeps fp32 accuracy
+// with six of the nine cross terms (hh, hm, mh, mm, hl, lh; the dropped ones are below 2^-24 of the product), every
+// bf16 x bf16 product is exact in fp32 and the matrix core accumulates in fp32: measured error of a 32-term dot
+// product 5e-8 of the sum of magnitudes, against 1.3e-7 for an fp32 fused chain.  v_mfma_f32_16x16x32_bf16 does 8
+// times the work of v_mfma_f32_16x16x4_f32 in half the cycles, so six of them per product still run 2.7 times
+// faster than the fp32 matrix path.
+//
+// Layout of v_mfma_f32_16x16x32_bf16: lane (r = lane % 16, g = lane / 16) holds A[r][8g..8g+7], B[8g..8g+7][r] and
+// C[4g..4g+3][r].  As above only the pairing of A and B slots matters, so
+//   scores:  A = K tile, lane holds dims 32t + 8g .. + 7 of key r (+16 for the second half), B = Q likewise:
+//            C[4g+i][c] = S^T[key 4g+i][query c]: lane again holds 4 keys of query c per half;
+//   output:  A = P, lane's 8 slots = its 8 scores: keys 4g..4g+3 and 16+4g..16+4g+3; B = V with the same key order,
+//            so V is stored in LDS dim-major with those 8 keys of a group adjacent (one 16-byte read per operand).
+// K and V tiles are split into their three planes once per workgroup when they are staged (shared by the 4 heads
+// and 16 queries); Q is split once, P once per tile and wave.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+struct Planes {
+	bf16x8 h, m, l;
+};
+__device__ __forceinline__ Planes split8(const float *x) {
+	Planes o;
+#pragma unroll
+	for (int i = 0; i < 8; i += 2) {
+		const f32x2 v = {x[i], x[i + 1]};
+		const bf16x2 a = __builtin_convertvector(v, bf16x2);  // round to nearest even
+		const f32x2 r1 = v - __builtin_convertvector(a, f32x2);
+		const bf16x2 b = __builtin_convertvector(r1, bf16x2);
+		const f32x2 r2 = r1 - __builtin_convertvector(b, f32x2);
+		const bf16x2 c = __builtin_convertvector(r2, bf16x2);
+		o.h[i] = a[0];
+		o.h[i + 1] = a[1];
+		o.m[i] = b[0];
+		o.m[i + 1] = b[1];
+		o.l[i] = c[0];
+		o.l[i + 1] = c[1];
+	}
+	return o;
+}
+// acc += a . b with the six significant cross terms, smallest first
+__device__ __forceinline__ f32x4 mfma6(const Planes &a, const Planes &b, f32x4 acc) {
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.l, b.h, acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.l, acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.m, b.m, acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.m, b.h, acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.m, acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.h, acc, 0, 0, 0);
+	return acc;
+}
+
+constexpr int NT32 = HD / 32;  // k steps of a score product
+
+// Same arguments, work items and outputs as attn_prefill_mfma_kernel.
+__global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
+                                                                 int ldkv, int ldo, int is_sw, int window, const int4 *items,
+                                                                 float *part_o, float *part_ml, float *rowmax_part, int Mpad) {
+	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+	// Kb[plane][t][key][g]: dims 32t + 8g .. + 7 of a key; Vb[plane][g][dim]: the 8 keys of group g at one dim
+	bf16x8(*Kb)[NT32][TK][4] = reinterpret_cast<bf16x8(*)[NT32][TK][4]>(smem);
+	bf16x8(*Vb)[4][HD] = reinterpret_cast<bf16x8(*)[4][HD]>(smem + sizeof(bf16x8) * 3 * NT32 * TK * 4);
+
+	const int tid = threadIdx.x, lane = tid & 63, head = tid >> 6, c = lane & 15, g = lane >> 4;
+	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ, slot = -1;
+	int4 item = int4{0, 0, 0, -1};
+	if (items != nullptr) {
+		item = items[blockIdx.x];
+		q0 = item.x * TQ;
+		slot = item.w;
+	}
+	const int qpos = q0 + c;
+	const int qrow = qpos < S ? qpos : S - 1;
+	int kb = (is_sw && q0 > window) ? q0 - window : 0;
+	int ke = (q0 + TQ < S) ? q0 + TQ : S;  // exclusive
+	if (items != nullptr) {
+		kb = item.y * TK;
+		ke = min(ke, item.z * TK);
+	}
+	const int ntiles = (ke - kb + TK - 1) / TK;
+	const int klo = is_sw ? qpos - window : 0;
+
+	// staging.  K: thread = (key, g) of k steps t = tid / 128 + 2u: 8 consecutive dims, two 16-byte loads.
+	// V: thread = (dim 64u + lane, group tid / 64): the group's 8 keys at one dim, 4-byte loads (a wave reads 256
+	// contiguous bytes of a key row).
+	const int sk_g = tid & 3, sk_key = (tid >> 2) & 31, sk_t0 = tid >> 7;
+	const int sv_g = tid >> 6;
+	f32x4 kpre[4][2];
+	float vpre[4][8];
+	auto key_row = [&](int tile, int key) {
+		int j = kb + tile * TK + key;
+		return (size_t)(j < ke ? j : ke - 1) * ldkv;
+	};
+	auto fetch = [&](int tile) {
+		const float *kp = k + key_row(tile, sk_key) + 8 * sk_g;
+#pragma unroll
+		for (int u = 0; u < 4; u++) {
+			kpre[u][0] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * u));
+			kpre[u][1] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * u) + 4);
+		}
+#pragma unroll
+		for (int sl = 0; sl < 8; sl++) {
+			const float *vp = v + key_row(tile, (sl < 4 ? 4 * sv_g + sl : 12 + 4 * sv_g + sl)) + lane;
+#pragma unroll
+			for (int u = 0; u < 4; u++) vpre[u][sl] = vp[64 * u];
+		}
+	};
+	fetch(0);
+
+	// Q planes: qp[t] = dims 32t + 8g .. + 7 of query c, scaled by 1/sqrt(hd) (a power of two: commutes with the split)
+	Planes qp[NT32];
+	{
+		const float *qsrc = q + (size_t)qrow * ldq + head * HD + 8 * g;
+#pragma unroll
+		for (int t = 0; t < NT32; t++) {
+			const f32x4 x0 = *reinterpret_cast<const f32x4 *>(qsrc + 32 * t), x1 = *reinterpret_cast<const f32x4 *>(qsrc + 32 * t + 4);
+			float x[8];
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				x[e] = x0[e] * 0.0625f;
+				x[4 + e] = x1[e] * 0.0625f;
+			}
+			qp[t] = split8(x);
+		}
+	}
+
+	f32x4 oacc[HD / 16];  // oacc[dt][i] = O[query 4 g + i][16 dt + c]
+#pragma unroll
+	for (int dt = 0; dt < HD / 16; dt++) oacc[dt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+	float m_run = -INFINITY, l_run = 0.0f;
+
+	for (int tile = 0; tile < ntiles; tile++) {
+		tg_lds_barrier();  // everyone is done with the previous tile
+#pragma unroll
+		for (int u = 0; u < 4; u++) {
+			float x[8];
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				x[e] = kpre[u][0][e];
+				x[4 + e] = kpre[u][1][e];
+			}
+			const Planes pl = split8(x);
+			const int t = sk_t0 + 2 * u;
+			Kb[0][t][sk_key][sk_g] = pl.h;
+			Kb[1][t][sk_key][sk_g] = pl.m;
+			Kb[2][t][sk_key][sk_g] = pl.l;
+		}
+#pragma unroll
+		for (int u = 0; u < 4; u++) {
+			const Planes pl = split8(vpre[u]);
+			Vb[0][sv_g][64 * u + lane] = pl.h;
+			Vb[1][sv_g][64 * u + lane] = pl.m;
+			Vb[2][sv_g][64 * u + lane] = pl.l;
+		}
+		tg_lds_barrier();
+		if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during the products
+
+		// ---- scores of the tile's two groups of 16 keys; even and odd k steps in separate accumulators ----
+		f32x4 sa[2][2];
+#pragma unroll
+		for (int hf = 0; hf < 2; hf++) sa[hf][0] = sa[hf][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+		for (int t = 0; t < NT32; t++) {
+#pragma unroll
+			for (int hf = 0; hf < 2; hf++) {
+				Planes kf;
+				kf.h = Kb[0][t][16 * hf + c][g];
+				kf.m = Kb[1][t][16 * hf + c][g];
+				kf.l = Kb[2][t][16 * hf + c][g];
+				sa[hf][t & 1] = mfma6(kf, qp[t], sa[hf][t & 1]);
+			}
+		}
+		f32x4 s0 = sa[0][0] + sa[0][1], s1 = sa[1][0] + sa[1][1];
+		// ---- mask + online softmax for query c ----
+		const int j0 = kb + tile * TK + 4 * g;
+		float tmax = -INFINITY;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int ja = j0 + i, jb = j0 + 16 + i;
+			if (ja > qpos || ja < klo) s0[i] = -INFINITY;
+			if (jb > qpos || jb < klo) s1[i] = -INFINITY;
+			tmax = fmaxf(tmax, fmaxf(s0[i], s1[i]));
+		}
+		tmax = fmaxf(tmax, tg_red_partner<16>(tmax));
+		tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
+		const float m_new = fmaxf(m_run, tmax);
+		const float alpha = expf(m_run - m_new);
+		float psum = 0.0f;
+		float pv[8];  // the lane's 8 key slots: keys 4g + i, then 16 + 4g + i
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			pv[i] = expf(s0[i] - m_new);
+			pv[4 + i] = expf(s1[i] - m_new);
+			psum += pv[i] + pv[4 + i];
+		}
+		psum += tg_red_partner<16>(psum);
+		psum += tg_red_partner<32>(psum);
+		l_run = fmaf(l_run, alpha, psum);
+		m_run = m_new;
+		float ar[4];
+#pragma unroll
+		for (int i = 0; i < 4; i++) ar[i] = __shfl(alpha, 4 * g + i, 64);
+#pragma unroll
+		for (int dt = 0; dt < HD / 16; dt++) {
+#pragma unroll
+			for (int i = 0; i < 4; i++) oacc[dt][i] *= ar[i];
+		}
+		// ---- O += P V ----
+		const Planes pp = split8(pv);
+#pragma unroll
+		for (int dt = 0; dt < HD / 16; dt++) {
+			Planes vf;
+			vf.h = Vb[0][g][16 * dt + c];
+			vf.m = Vb[1][g][16 * dt + c];
+			vf.l = Vb[2][g][16 * dt + c];
+			oacc[dt] = mfma6(pp, vf, oacc[dt]);
+		}
+	}
+
+	if (slot >= 0) {
+		float *po = part_o + (size_t)slot * TQ * NH * HD;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			float *op = po + ((size_t)(4 * g + i) * NH + head) * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i];
+		}
+		if (g == 0) {
+			float *pm = part_ml + (((size_t)slot * TQ + c) * NH + head) * 2;
+			pm[0] = m_run;
+			pm[1] = l_run;
+		}
+		return;
+	}
+	float lr[4];
+#pragma unroll
+	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int qo = q0 + 4 * g + i;
+		float omax = 0.0f;
+		if (qo < S) {
+			float *op = o + (size_t)qo * ldo + head * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) {
+				const float val = oacc[dt][i] / lr[i];
+				op[16 * dt] = val;
+				omax = fmaxf(omax, fabsf(val));
+			}
+		}
+		if (rowmax_part != nullptr) {
+			omax = tg_row16_max(omax);
+			if (c == 0 && qo < S) rowmax_part[(size_t)head * Mpad + qo] = omax;
+		}
+	}
+}
+constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD);  // 96 KB
+
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
@@ -238,6 +498,8 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 }
 
 }  // namespace
+
+int g_attn_prefill_bf16x3 = 1;  // 1: split-bf16 matrix path (default), 0: fp32 matrix path
 
 // Work list of a causal layer of S tokens, for tg_launch_attn_prefill.  Returns false when no query tile needs
 // splitting (then the plain launch is already balanced).  items: one int4 per workgroup, heaviest first;
@@ -277,13 +539,23 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	(void)n_head;
 	(void)hd;
 	const int Mpad = (int)tg_gemm_mfma_rows(S);  // rowmax_part (may be null): [4 heads][Mpad], max|o[row][head's columns]|
-	if (plan == nullptr || is_sw) {
-		hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)((S + TQ - 1) / TQ)), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo,
-		                   is_sw, window, (const int4 *)nullptr, (float *)nullptr, (float *)nullptr, rowmax_part, Mpad);
-		return;
+	static bool lds_set = false;
+	if (g_attn_prefill_bf16x3 && !lds_set) {  // 96 KB of dynamic LDS needs the opt-in
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+		                          (int)BF_LDS_BYTES);
+		lds_set = true;
 	}
-	hipLaunchKernelGGL(attn_prefill_mfma_kernel, dim3((unsigned)plan->nitems), dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, 0, window,
-	                   plan->items, plan->part_o, plan->part_ml, rowmax_part, Mpad);
+	const bool whole = plan == nullptr || is_sw;
+	const dim3 grid(whole ? (unsigned)((S + TQ - 1) / TQ) : (unsigned)plan->nitems);
+	const int4 *items = whole ? nullptr : plan->items;
+	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
+	if (g_attn_prefill_bf16x3)
+		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel, grid, dim3(PNT), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
+		                   window, items, po, pml, rowmax_part, Mpad);
+	else
+		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0, window, items,
+		                   po, pml, rowmax_part, Mpad);
+	if (whole) return;
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * TQ)), dim3(PNT), 0, s, o, S, ldo, plan->split,
 	                   plan->part_o, plan->part_ml, rowmax_part, Mpad);
 }

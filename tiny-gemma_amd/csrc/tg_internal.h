@@ -169,6 +169,7 @@ struct TgAttnPrefillPlan {
 	int nitems, nsplit;
 	float *part_o, *part_ml;
 };
+extern int g_attn_prefill_bf16x3;  // prefill attention: 1 = split-bf16 matrix path, 0 = fp32 matrix path
 bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
 size_t tg_attn_prefill_part_floats(int nslots);
 size_t tg_attn_prefill_ml_floats(int nslots);
