@@ -152,8 +152,10 @@ int tg_set_taps(int enable);
  * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */
 int tg_set_gemm_mode(int mfma);
 /* prefill attention: 1 (default) = bf16 matrix cores on three bf16 planes of every fp32 operand (six cross terms per
- * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), 0 = fp32 matrix cores */
-int tg_set_attn_prefill_mode(int bf16x3);
+ * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), workgroups of 32 query positions
+ * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;
+ * 0 = fp32 matrix cores, workgroups of 16 */
+int tg_set_attn_prefill_mode(int mode);
 /* tuning knob: a GEMV launch uses at most n workgroups, which then loop over column tiles (0: one per tile) */
 int tg_set_gemv_max_blocks(int n);
 /* tuning knob: extra workgroups per decode launch that pull the NEXT launch's weights out of HBM into

@@ -226,8 +226,17 @@ def _dense_rows(q, k, v, rows, is_sw, ctx):
     return out
 
 
+@pytest.fixture(params=[0, 1, 2], ids=["fp32_mfma", "bf16x3", "bf16x3_32q"])
+def attn_mode(tg, request):
+    """The fp32 matrix path, the split-bf16 path as launched by default, and the latter with 32-query workgroups
+    forced (what long prompts get)."""
+    tg.check(tg.lib().tg_set_attn_prefill_mode(request.param))
+    yield request.param
+    tg.check(tg.lib().tg_set_attn_prefill_mode(1))
+
+
 @pytest.mark.parametrize("name", list(gi.ATTN_PREFILL_CASES))
-def test_attention_prefill_vs_fixture_and_checker(tg, oracle, golden, name):
+def test_attention_prefill_vs_fixture_and_checker(tg, oracle, golden, attn_mode, name):
     S, sw, ctx, seed = gi.ATTN_PREFILL_CASES[name]
     q, k, v = gi.attn_prefill_inputs(S, seed)
     o = tg.attention_prefill(q, k, v, sw, ctx)
@@ -237,7 +246,7 @@ def test_attention_prefill_vs_fixture_and_checker(tg, oracle, golden, name):
 
 
 @pytest.mark.parametrize("S", [1500, 4099])
-def test_attention_prefill_split_key_ranges(tg, oracle, S):
+def test_attention_prefill_split_key_ranges(tg, oracle, attn_mode, S):
     """Causal layers long enough for the key ranges to be cut into chunks and merged (S > 512); 4099 is ragged
     against both the 16-query and the 32-key tiling."""
     q, k, v = gi.attn_prefill_inputs(S, 410 + S)

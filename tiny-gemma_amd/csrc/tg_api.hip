@@ -208,20 +208,22 @@ namespace {
 struct AttnPlanDev {
 	TgAttnPrefillPlan p;
 	bool use = false;
-	int S = -1;  // token count the lists were built for
+	int S = -1, tq = 0;  // token count and query tile size the lists were built for
 	void *bufs[4] = {nullptr, nullptr, nullptr, nullptr};
 	std::vector<int4> items, split;  // host copies stay alive until the uploads have completed
 	int build(int n_tokens) {
-		if (n_tokens == S) return TG_OK;
+		const int tile = tg_attn_prefill_query_tile(n_tokens, g_n_cu);
+		if (n_tokens == S && tile == tq) return TG_OK;
 		release();
 		int nslots = 0;
-		use = tg_attn_prefill_plan(n_tokens, g_n_cu, items, split, nslots);
+		use = tg_attn_prefill_plan(n_tokens, g_n_cu, tile, items, split, nslots);
 		S = n_tokens;
+		tq = tile;
 		if (!use) return TG_OK;
 		TG_HIP(hipMalloc(&bufs[0], items.size() * sizeof(int4)));
 		TG_HIP(hipMalloc(&bufs[1], split.size() * sizeof(int4)));
-		TG_HIP(hipMalloc(&bufs[2], tg_attn_prefill_part_floats(nslots) * sizeof(float)));
-		TG_HIP(hipMalloc(&bufs[3], tg_attn_prefill_ml_floats(nslots) * sizeof(float)));
+		TG_HIP(hipMalloc(&bufs[2], tg_attn_prefill_part_floats(nslots, tile) * sizeof(float)));
+		TG_HIP(hipMalloc(&bufs[3], tg_attn_prefill_ml_floats(nslots, tile) * sizeof(float)));
 		TG_HIP(hipMemcpyAsync(bufs[0], items.data(), items.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
 		TG_HIP(hipMemcpyAsync(bufs[1], split.data(), split.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
 		p.items = (const int4 *)bufs[0];
@@ -240,6 +242,7 @@ struct AttnPlanDev {
 		}
 		use = false;
 		S = -1;
+		tq = 0;
 	}
 };
 }  // namespace
@@ -1099,8 +1102,9 @@ int tg_set_attn_merge_chunk(int keys) {
 	return TG_OK;
 }
 
-int tg_set_attn_prefill_mode(int bf16x3) {
-	g_attn_prefill_bf16x3 = bf16x3 != 0;
+int tg_set_attn_prefill_mode(int mode) {
+	if (mode < 0 || mode > 2) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1 or 2");
+	g_attn_prefill_bf16x3 = mode;
 	return TG_OK;
 }
 
@@ -1209,7 +1213,7 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
 	if (rc == TG_OK && !is_sw) rc = plan.build(S);
 	if (rc != TG_OK) return done(rc);
-	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), nullptr, g_stream);
+	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), nullptr, g_n_cu, g_stream);
 	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
 	rc = tg_copy_d2h(orow.data(), dout, sizeof(float) * rows * NH * HD);
 	if (rc != TG_OK) return done(rc);
@@ -1291,7 +1295,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
 		                            g_stream);
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, plan.get(), amax, g_stream);
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, plan.get(), amax, g_n_cu, g_stream);
 		// O (modules.hpp:127-128)
 		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)

@@ -266,27 +266,34 @@ __device__ __forceinline__ f32x4 mfma6(const Planes &a, const Planes &b, f32x4 a
 
 constexpr int NT32 = HD / 32;  // k steps of a score product
 
-// Same arguments, work items and outputs as attn_prefill_mfma_kernel.
-__global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
+// Same arguments and outputs as attn_prefill_mfma_kernel.  QG = groups of 16 query positions per workgroup, each
+// with its own four waves (heads).  QG = 2: a K/V tile is fetched, split and staged once for 32 queries x 4 heads,
+// and the two waves a SIMD then holds overlap each other's LDS reads, matrix and vector work; the launcher takes it
+// for prompts long enough to keep the compute units busy with such workgroups, else QG = 1.
+template <int QG>
+__global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
                                                                  int ldkv, int ldo, int is_sw, int window, const int4 *items,
                                                                  float *part_o, float *part_ml, float *rowmax_part, int Mpad) {
 	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 	// Kb[plane][t][key][g]: dims 32t + 8g .. + 7 of a key; Vb[plane][g][dim]: the 8 keys of group g at one dim
 	bf16x8(*Kb)[NT32][TK][4] = reinterpret_cast<bf16x8(*)[NT32][TK][4]>(smem);
 	bf16x8(*Vb)[4][HD] = reinterpret_cast<bf16x8(*)[4][HD]>(smem + sizeof(bf16x8) * 3 * NT32 * TK * 4);
+	constexpr int BQ = 16 * QG;   // query positions per workgroup
+	constexpr int SU = 4 / QG;    // staging units per thread and operand
 
-	const int tid = threadIdx.x, lane = tid & 63, head = tid >> 6, c = lane & 15, g = lane >> 4;
-	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ, slot = -1;
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, head = w & 3, qh = w >> 2, c = lane & 15, g = lane >> 4;
+	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * BQ, slot = -1;
 	int4 item = int4{0, 0, 0, -1};
 	if (items != nullptr) {
 		item = items[blockIdx.x];
-		q0 = item.x * TQ;
+		q0 = item.x * BQ;
 		slot = item.w;
 	}
-	const int qpos = q0 + c;
+	const int q0w = q0 + 16 * qh;  // first query of this wave's group
+	const int qpos = q0w + c;
 	const int qrow = qpos < S ? qpos : S - 1;
 	int kb = (is_sw && q0 > window) ? q0 - window : 0;
-	int ke = (q0 + TQ < S) ? q0 + TQ : S;  // exclusive
+	int ke = (q0 + BQ < S) ? q0 + BQ : S;  // exclusive
 	if (items != nullptr) {
 		kb = item.y * TK;
 		ke = min(ke, item.z * TK);
@@ -294,13 +301,13 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 	const int ntiles = (ke - kb + TK - 1) / TK;
 	const int klo = is_sw ? qpos - window : 0;
 
-	// staging.  K: thread = (key, g) of k steps t = tid / 128 + 2u: 8 consecutive dims, two 16-byte loads.
-	// V: thread = (dim 64u + lane, group tid / 64): the group's 8 keys at one dim, 4-byte loads (a wave reads 256
-	// contiguous bytes of a key row).
+	// staging.  K: thread = (key, g) of k steps t = tid / 128 + 2 QG u: 8 consecutive dims, two 16-byte loads.
+	// V: thread = (dim 64 QG u + 64 (w / 4) + lane, group w % 4): the group's 8 keys at one dim, 4-byte loads (a wave
+	// reads 256 contiguous bytes of a key row).
 	const int sk_g = tid & 3, sk_key = (tid >> 2) & 31, sk_t0 = tid >> 7;
-	const int sv_g = tid >> 6;
-	f32x4 kpre[4][2];
-	float vpre[4][8];
+	const int sv_g = w & 3, sv_d = 64 * (w >> 2) + lane;
+	f32x4 kpre[SU][2];
+	float vpre[SU][8];
 	auto key_row = [&](int tile, int key) {
 		int j = kb + tile * TK + key;
 		return (size_t)(j < ke ? j : ke - 1) * ldkv;
@@ -308,15 +315,15 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 	auto fetch = [&](int tile) {
 		const float *kp = k + key_row(tile, sk_key) + 8 * sk_g;
 #pragma unroll
-		for (int u = 0; u < 4; u++) {
-			kpre[u][0] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * u));
-			kpre[u][1] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * u) + 4);
+		for (int u = 0; u < SU; u++) {
+			kpre[u][0] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * QG * u));
+			kpre[u][1] = *reinterpret_cast<const f32x4 *>(kp + 32 * (sk_t0 + 2 * QG * u) + 4);
 		}
 #pragma unroll
 		for (int sl = 0; sl < 8; sl++) {
-			const float *vp = v + key_row(tile, (sl < 4 ? 4 * sv_g + sl : 12 + 4 * sv_g + sl)) + lane;
+			const float *vp = v + key_row(tile, (sl < 4 ? 4 * sv_g + sl : 12 + 4 * sv_g + sl)) + sv_d;
 #pragma unroll
-			for (int u = 0; u < 4; u++) vpre[u][sl] = vp[64 * u];
+			for (int u = 0; u < SU; u++) vpre[u][sl] = vp[64 * QG * u];
 		}
 	};
 	fetch(0);
@@ -346,7 +353,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 	for (int tile = 0; tile < ntiles; tile++) {
 		tg_lds_barrier();  // everyone is done with the previous tile
 #pragma unroll
-		for (int u = 0; u < 4; u++) {
+		for (int u = 0; u < SU; u++) {
 			float x[8];
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
@@ -354,20 +361,22 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 				x[4 + e] = kpre[u][1][e];
 			}
 			const Planes pl = split8(x);
-			const int t = sk_t0 + 2 * u;
+			const int t = sk_t0 + 2 * QG * u;
 			Kb[0][t][sk_key][sk_g] = pl.h;
 			Kb[1][t][sk_key][sk_g] = pl.m;
 			Kb[2][t][sk_key][sk_g] = pl.l;
 		}
 #pragma unroll
-		for (int u = 0; u < 4; u++) {
+		for (int u = 0; u < SU; u++) {
 			const Planes pl = split8(vpre[u]);
-			Vb[0][sv_g][64 * u + lane] = pl.h;
-			Vb[1][sv_g][64 * u + lane] = pl.m;
-			Vb[2][sv_g][64 * u + lane] = pl.l;
+			Vb[0][sv_g][64 * QG * u + sv_d] = pl.h;
+			Vb[1][sv_g][64 * QG * u + sv_d] = pl.m;
+			Vb[2][sv_g][64 * QG * u + sv_d] = pl.l;
 		}
 		tg_lds_barrier();
 		if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during the products
+		// a tile that starts behind this group's last query holds none of its keys (the other group still needs it)
+		if (kb + tile * TK > q0w + 15) continue;
 
 		// ---- scores of the tile's two groups of 16 keys; even and odd k steps in separate accumulators ----
 		f32x4 sa[2][2];
@@ -432,15 +441,15 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 	}
 
 	if (slot >= 0) {
-		float *po = part_o + (size_t)slot * TQ * NH * HD;
+		float *po = part_o + (size_t)slot * BQ * NH * HD;
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
-			float *op = po + ((size_t)(4 * g + i) * NH + head) * HD + c;
+			float *op = po + ((size_t)(16 * qh + 4 * g + i) * NH + head) * HD + c;
 #pragma unroll
 			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i];
 		}
 		if (g == 0) {
-			float *pm = part_ml + (((size_t)slot * TQ + c) * NH + head) * 2;
+			float *pm = part_ml + (((size_t)slot * BQ + 16 * qh + c) * NH + head) * 2;
 			pm[0] = m_run;
 			pm[1] = l_run;
 		}
@@ -451,7 +460,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_bf16x3_kernel(float *o, cons
 	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
-		const int qo = q0 + 4 * g + i;
+		const int qo = q0w + 4 * g + i;
 		float omax = 0.0f;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
@@ -473,17 +482,17 @@ constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
-                                                                const float *part_ml, float *rowmax_part, int Mpad) {
-	const int4 sp = split[blockIdx.x / TQ];
-	const int qi = blockIdx.x % TQ, qpos = sp.x * TQ + qi;
+                                                                const float *part_ml, float *rowmax_part, int Mpad, int tq) {
+	const int4 sp = split[blockIdx.x / tq];
+	const int qi = blockIdx.x % tq, qpos = sp.x * tq + qi;
 	if (qpos >= S) return;
 	const int lane = threadIdx.x & 63, head = threadIdx.x >> 6;
 	float M = -INFINITY;
-	for (int ch = 0; ch < sp.z; ch++) M = fmaxf(M, part_ml[(((size_t)(sp.y + ch) * TQ + qi) * NH + head) * 2]);
+	for (int ch = 0; ch < sp.z; ch++) M = fmaxf(M, part_ml[(((size_t)(sp.y + ch) * tq + qi) * NH + head) * 2]);
 	float L = 0.0f;
 	f32x4 acc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 	for (int ch = 0; ch < sp.z; ch++) {
-		const size_t row = ((size_t)(sp.y + ch) * TQ + qi) * NH + head;
+		const size_t row = ((size_t)(sp.y + ch) * tq + qi) * NH + head;
 		const float wgt = expf(part_ml[row * 2] - M);
 		L = fmaf(part_ml[row * 2 + 1], wgt, L);
 		const f32x4 x = *reinterpret_cast<const f32x4 *>(part_o + row * HD + 4 * lane);
@@ -499,14 +508,20 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 
 }  // namespace
 
-int g_attn_prefill_bf16x3 = 1;  // 1: split-bf16 matrix path (default), 0: fp32 matrix path
+int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
 
 // Work list of a causal layer of S tokens, for tg_launch_attn_prefill.  Returns false when no query tile needs
 // splitting (then the plain launch is already balanced).  items: one int4 per workgroup, heaviest first;
 // split: one int4 per split query tile; nslots: chunks that go through scratch.
-bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
-	const int nq = (S + TQ - 1) / TQ;
-	auto ntiles_of = [&](int qt) { return (std::min(qt * TQ + TQ, S) + TK - 1) / TK; };
+// 32 query positions per workgroup once that leaves a workgroup for every other compute unit (measured crossover:
+// between 2048 and 4096 tokens on 256 compute units)
+int tg_attn_prefill_query_tile(int S, int n_cu) {
+	return (g_attn_prefill_bf16x3 == 2 || (g_attn_prefill_bf16x3 == 1 && (S + 31) / 32 >= n_cu / 2)) ? 32 : TQ;
+}
+
+bool tg_attn_prefill_plan(int S, int n_cu, int tq, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
+	const int nq = (S + tq - 1) / tq;
+	auto ntiles_of = [&](int qt) { return (std::min(qt * tq + tq, S) + TK - 1) / TK; };
 	long total = 0;
 	for (int qt = 0; qt < nq; qt++) total += ntiles_of(qt);
 	// about 8 items per compute unit, and never chunks below 16 key tiles (512 keys)
@@ -530,32 +545,38 @@ bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector
 	std::stable_sort(items.begin(), items.end(), [](const int4 &a, const int4 &b) { return a.z - a.y > b.z - b.y; });
 	return true;
 }
-size_t tg_attn_prefill_part_floats(int nslots) { return (size_t)nslots * TQ * NH * HD; }
-size_t tg_attn_prefill_ml_floats(int nslots) { return (size_t)nslots * TQ * NH * 2; }
+size_t tg_attn_prefill_part_floats(int nslots, int tq) { return (size_t)nslots * tq * NH * HD; }
+size_t tg_attn_prefill_ml_floats(int nslots, int tq) { return (size_t)nslots * tq * NH * 2; }
 
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, hipStream_t s) {
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s) {
 	(void)n_head;
 	(void)hd;
 	const int Mpad = (int)tg_gemm_mfma_rows(S);  // rowmax_part (may be null): [4 heads][Mpad], max|o[row][head's columns]|
 	static bool lds_set = false;
 	if (g_attn_prefill_bf16x3 && !lds_set) {  // 96 KB of dynamic LDS needs the opt-in
-		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
+		                          (int)BF_LDS_BYTES);
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
 		                          (int)BF_LDS_BYTES);
 		lds_set = true;
 	}
 	const bool whole = plan == nullptr || is_sw;
-	const dim3 grid(whole ? (unsigned)((S + TQ - 1) / TQ) : (unsigned)plan->nitems);
+	const int tq = tg_attn_prefill_query_tile(S, n_cu);  // a plan must have been built for this tile size
+	const dim3 grid(whole ? (unsigned)((S + tq - 1) / tq) : (unsigned)plan->nitems);
 	const int4 *items = whole ? nullptr : plan->items;
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
-	if (g_attn_prefill_bf16x3)
-		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel, grid, dim3(PNT), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
+	if (g_attn_prefill_bf16x3 && tq == 32)
+		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
+		                   window, items, po, pml, rowmax_part, Mpad);
+	else if (g_attn_prefill_bf16x3)
+		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<1>, grid, dim3(256), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
 		                   window, items, po, pml, rowmax_part, Mpad);
 	else
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0, window, items,
 		                   po, pml, rowmax_part, Mpad);
 	if (whole) return;
-	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * TQ)), dim3(PNT), 0, s, o, S, ldo, plan->split,
-	                   plan->part_o, plan->part_ml, rowmax_part, Mpad);
+	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * tq)), dim3(PNT), 0, s, o, S, ldo, plan->split,
+	                   plan->part_o, plan->part_ml, rowmax_part, Mpad, tq);
 }

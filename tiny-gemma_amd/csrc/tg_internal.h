@@ -169,12 +169,13 @@ struct TgAttnPrefillPlan {
 	int nitems, nsplit;
 	float *part_o, *part_ml;
 };
-extern int g_attn_prefill_bf16x3;  // prefill attention: 1 = split-bf16 matrix path, 0 = fp32 matrix path
-bool tg_attn_prefill_plan(int S, int n_cu, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
-size_t tg_attn_prefill_part_floats(int nslots);
-size_t tg_attn_prefill_ml_floats(int nslots);
+extern int g_attn_prefill_bf16x3;  // prefill attention: 0 = fp32 matrix path, 1 = split-bf16 matrix path, 2 = the same with 32-query workgroups at any length
+int tg_attn_prefill_query_tile(int S, int n_cu);  // query positions per workgroup of the kernel a launch will take
+bool tg_attn_prefill_plan(int S, int n_cu, int tq, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
+size_t tg_attn_prefill_part_floats(int nslots, int tq);
+size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, hipStream_t s);
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s);
 // exact-order GEMM on the GEMV tiling (ntiles tiles of Ct columns): C[m][N] = (A[m][K] . W) * scales; epi GEGLU writes C[m][N/2]
 void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
