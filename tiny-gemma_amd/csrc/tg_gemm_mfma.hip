@@ -42,6 +42,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GNT = 256;     // threads per workgroup: 4 waves, each owns 32 rows x 128 columns
 constexpr int KSTAGE = 64;   // rows of K per LDS stage
+constexpr int TG_GEMM_SKINNY_ROWS = 256;    // at most this many rows and
+constexpr int TG_GEMM_SKINNY_BLOCKS = 128;  // fewer workgroups than this in the plain tiling: split K over the waves
 constexpr int LUT_LDS_MAX = 4096;  // GeLU tables up to this many entries are staged in LDS (Bs holds 16 KB)
 
 // ginv != 0: the table step is a power of two and ginv its exact reciprocal, so the product equals the quotient
@@ -292,6 +294,147 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 	}
 }
 
+// ---- few rows (a short prompt): the same product with the reduction split over the four waves ----------------
+// With M <= 256 the kernel above has only a handful of workgroups (two row blocks x 9 column tiles for the down
+// projection of the 1B shape) and each walks all of K alone.  Here a workgroup owns 32 rows x 128 columns and its
+// four waves take the K stages round-robin (stage w, w + 4, ...), each with a private register pipeline: no LDS and
+// no barrier in the main loop, weights fetched straight from global memory in operand order (32 lanes x 16 bytes =
+// 512 contiguous bytes per fragment).  The integer partial sums are added through LDS at the end (exact, so the
+// result equals the unsplit one bit for bit) and wave j finishes column block j.
+template <bool GEGLU, bool LUTLDS>
+__global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
+                                                             const float *scales, int M, int K, int ldc, const float *lut, float gmin,
+                                                             float geps, float ginv, int lut_size, float *rowmax_part, int Mpad) {
+	__shared__ __attribute__((aligned(16))) i32x4 red[4][3][4][64];  // [wave][plane][quarter of the 16 registers][lane]
+	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
+	__shared__ float pmax[2][32];
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hb = lane >> 5;
+	const int tile = blockIdx.x, mtile = blockIdx.y;
+	const int nstage = K / KSTAGE, last = nstage - 1;
+	if (GEGLU && LUTLDS) {  // visible after the barriers of the reduction
+		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
+	}
+	const i32x4 *bsrc = reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + hb * TG_CT + c;
+	const i32x4 *asrc = reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane;
+
+	// ring of three stages: loads go to ordinary vector registers only, and 3 x 56 of them is what fits beside the
+	// addresses (the 192 accumulators live in the accumulation registers)
+	i32x4 areg[3][6];  // [ring slot][k step * 3 + plane]
+	i32x4 breg[3][8];  // [ring slot][k step * 4 + column block]
+	auto load = [&](int st, i32x4 *ar, i32x4 *br) {
+		st = st < last ? st : last;  // unconditional loads: surplus ones land in ring slots nobody reads again
+#pragma unroll
+		for (int i = 0; i < 6; i++) ar[i] = asrc[(size_t)(st * 6 + i) * 64];
+#pragma unroll
+		for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+			for (int j = 0; j < 4; j++) br[ks * 4 + j] = bsrc[(size_t)(st * 4 + 2 * ks) * TG_CT + 32 * j];
+	};
+	i32x16 acc[3][4];
+#pragma unroll
+	for (int p = 0; p < 3; p++)
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int i = 0; i < 16; i++) acc[p][j][i] = 0;
+
+	// iteration i of wave w is stage w + 4 i; every wave runs the same number of iterations, a stage beyond K
+	// contributes zeros (its activation fragments are cleared: no branch around the matrix instructions)
+	auto stage = [&](int i, auto uc) {
+		constexpr int u = decltype(uc)::value;
+		load(w + 4 * (i + 2), areg[(u + 2) % 3], breg[(u + 2) % 3]);
+		const bool valid = w + 4 * i < nstage;
+#pragma unroll
+		for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+			for (int p = 0; p < 3; p++) {
+				i32x4 a = areg[u][ks * 3 + p];
+				if (!valid) a = i32x4{0, 0, 0, 0};
+#pragma unroll
+				for (int j = 0; j < 4; j++) acc[p][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(breg[u][ks * 4 + j], a, acc[p][j], 0, 0, 0);
+			}
+	};
+	load(w, areg[0], breg[0]);
+	load(w + 4, areg[1], breg[1]);
+	const int n_it = (nstage + 3) / 4;
+	int i0 = 0;
+	for (; i0 + 3 <= n_it; i0 += 3) {
+		stage(i0, std::integral_constant<int, 0>{});
+		stage(i0 + 1, std::integral_constant<int, 1>{});
+		stage(i0 + 2, std::integral_constant<int, 2>{});
+	}
+	if (i0 < n_it) stage(i0, std::integral_constant<int, 0>{});
+	if (i0 + 1 < n_it) stage(i0 + 1, std::integral_constant<int, 1>{});
+
+	// reduction over the waves, one column block per round; STORE: wave j keeps block j; GEGLU: waves 0 and 1 keep
+	// the up block j and the gate block j + 2
+	i32x16 fin[2][3];
+#pragma unroll
+	for (int j = 0; j < 4; j++) {
+#pragma unroll
+		for (int p = 0; p < 3; p++)
+#pragma unroll
+			for (int qq = 0; qq < 4; qq++)
+				red[w][p][qq][lane] = i32x4{acc[p][j][4 * qq], acc[p][j][4 * qq + 1], acc[p][j][4 * qq + 2], acc[p][j][4 * qq + 3]};
+		__syncthreads();
+		const int owner = GEGLU ? (j & 1) : j;
+		if (w == owner) {
+#pragma unroll
+			for (int p = 0; p < 3; p++)
+#pragma unroll
+				for (int qq = 0; qq < 4; qq++) {
+					const i32x4 t = (red[0][p][qq][lane] + red[1][p][qq][lane]) + (red[2][p][qq][lane] + red[3][p][qq][lane]);
+#pragma unroll
+					for (int e = 0; e < 4; e++) fin[(GEGLU && j >= 2) ? 1 : 0][p][4 * qq + e] = t[e];
+				}
+		}
+		__syncthreads();
+	}
+
+	const int m = mtile * 32 + c;
+	const float rs = rowinv[m];
+	const int jb = w;  // column block this wave finishes (GEGLU: waves 0 and 1 only)
+	auto value = [&](const i32x16 *f, int i, float scale) {
+		const float v = fmaf((float)f[2][i], 65536.0f, fmaf((float)f[1][i], 256.0f, (float)f[0][i]));
+		return (v * rs) * scale;
+	};
+	float omax = 0.0f;
+	if (!GEGLU || w < 2) {
+		f32x4 sc_u[4], sc_g[4];
+#pragma unroll
+		for (int q = 0; q < 4; q++) {
+			sc_u[q] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * jb + 8 * q + 4 * hb);
+			if (GEGLU) sc_g[q] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * (jb + 2) + 8 * q + 4 * hb);
+		}
+		if (m < M) {
+			float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 32 * jb + 4 * hb;
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				f32x4 o;
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int i = 4 * q + e;
+					if (GEGLU) {
+						const float gate = value(fin[1], i, sc_g[q][e]);
+						o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
+						       value(fin[0], i, sc_u[q][e]);
+						omax = fmaxf(omax, fabsf(o[e]));
+					} else {
+						o[e] = value(fin[0], i, sc_u[q][e]);
+					}
+				}
+				*reinterpret_cast<f32x4 *>(crow + 8 * q) = o;
+			}
+		}
+	}
+	if (GEGLU && rowmax_part != nullptr) {
+		omax = fmaxf(omax, tg_red_partner<32>(omax));
+		if (w < 2 && hb == 0) pmax[w][c] = omax;
+		__syncthreads();
+		if (w == 0 && hb == 0) rowmax_part[(size_t)tile * Mpad + m] = fmaxf(pmax[0][c], pmax[1][c]);
+	}
+}
+
 }  // namespace
 
 // scratch sizes for M rows of K: digit planes (bytes) and row factors (floats, two arrays of this length)
@@ -319,17 +462,33 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	const unsigned mblocks = (unsigned)((M + 127) / 128);
 	const int Mpad = (int)tg_gemm_mfma_rows(M);
 	const float *rowinv = rowfac + Mpad;
-	const dim3 grid((unsigned)ntiles, mblocks), block(GNT);
 	int e = 0;
 	const float ginv = (epi == TG_EPI_GEGLU && geps > 0.0f && frexpf(geps, &e) == 0.5f && e > -100 && e < 100) ? 1.0f / geps : 0.0f;
-	if (epi == TG_EPI_GEGLU && lut_size <= LUT_LDS_MAX) {
-		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
-		                   gmin, geps, ginv, lut_size, rowmax_part, Mpad);
-	} else if (epi == TG_EPI_GEGLU) {
-		hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * (TG_CT / 2), lut,
-		                   gmin, geps, ginv, lut_size, rowmax_part, Mpad);
-	} else {
-		hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ntiles * TG_CT, lut, gmin,
-		                   geps, ginv, lut_size, (float *)nullptr, Mpad);
+	const bool geglu = epi == TG_EPI_GEGLU, lutlds = geglu && lut_size <= LUT_LDS_MAX;
+	const int ldc = geglu ? ntiles * (TG_CT / 2) : ntiles * TG_CT;
+	float *rmp = geglu ? rowmax_part : nullptr;
+	// few rows and few column tiles: split K over the waves instead of leaving most compute units idle
+	if (M <= TG_GEMM_SKINNY_ROWS && (int)mblocks * ntiles < TG_GEMM_SKINNY_BLOCKS) {
+		const dim3 grid((unsigned)ntiles, (unsigned)((M + 31) / 32)), block(GNT);
+		if (geglu && lutlds)
+			hipLaunchKernelGGL((gemm_i8_skinny_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, Mpad);
+		else if (geglu)
+			hipLaunchKernelGGL((gemm_i8_skinny_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, Mpad);
+		else
+			hipLaunchKernelGGL((gemm_i8_skinny_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
+			                   geps, ginv, lut_size, rmp, Mpad);
+		return;
 	}
+	const dim3 grid((unsigned)ntiles, mblocks), block(GNT);
+	if (geglu && lutlds)
+		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
+		                   lut_size, rmp, Mpad);
+	else if (geglu)
+		hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
+		                   lut_size, rmp, Mpad);
+	else
+		hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
+		                   lut_size, rmp, Mpad);
 }
