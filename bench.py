@@ -11,8 +11,9 @@ Prints one JSON line.  `roofline` is for the dominant kernel of a step, the LM-h
 (tg_gemv_lmhead_argmax: 1152 x 262144 int8 + scales + x + logits = 304,091,648 algorithmic
 bytes per launch), timed with HIP events on the library's stream during real decode steps.
 Reported beside it: `gemv_lmhead_shape` (the plain GEMV entry point tg_qgemv_dev on the same matrix,
-launched back to back) and `prefill.long_prompt` (a 4096-token prefill of the same model: the
-matrix-matrix path on the int8 matrix cores).
+launched back to back), `gemv_640x2048` (the bare matvec of the first benchmark configuration, warm and
+rotating over 512 MB of distinct copies) and `prefill.long_prompt` (a 4096-token prefill of the same
+model: the matrix-matrix path on the int8 matrix cores).
 `cpu_baseline` times the reference's single-threaded AVX2 path (oracle/_ref, built from the
 reference's own sources) — or, where that library is absent, the scalar C restatement — on
 this machine's host cores over a bounded sample of the same workload.
@@ -217,6 +218,36 @@ def main():
     bare_us = ev.elapsed_ms(e0, e1) * 1e3 / 50
     qw.free()
 
+    # ---- the bare matvec of the first benchmark configuration: 640 x 2048, warm (one matrix, re-launched) and cold
+    # (rotating over distinct copies that together exceed the 256 MB memory-side cache twice over) ----
+    ci, cn = 640, 2048
+    c1_bytes = ci * cn + 4 * cn + 4 * ci + 4 * cn
+    n_copies = (512 << 20) // (ci * cn) + 1
+    crng = np.random.default_rng(101)
+    Wc = crng.integers(-127, 128, (ci, cn), dtype=np.int8)
+    sc = crng.uniform(0.001, 0.02, cn).astype(np.float32)
+    copies = [tg.QWeight(Wc, sc) for _ in range(n_copies)]
+    cx = tg.DeviceBuffer.from_numpy(crng.standard_normal(ci).astype(np.float32))
+    cy = tg.DeviceBuffer(4 * cn)
+    for q_ in copies[:8]:
+        q_.gemv(cy, cx)
+    tg.synchronize()
+    ev.record(e0, stream)
+    for _ in range(200):
+        copies[0].gemv(cy, cx)
+    ev.record(e1, stream)
+    tg.synchronize()
+    c1_warm_us = ev.elapsed_ms(e0, e1) * 1e3 / 200
+    ev.record(e0, stream)
+    for q_ in copies:
+        q_.gemv(cy, cx)
+    ev.record(e1, stream)
+    tg.synchronize()
+    c1_cold_us = ev.elapsed_ms(e0, e1) * 1e3 / n_copies
+    for q_ in copies:
+        q_.free()
+    del copies
+
     # ---- long-prompt prefill (the matrix-matrix path) on a fresh session ----
     long_prefill = None
     if args.long_prefill > 0:
@@ -274,6 +305,15 @@ def main():
             "GBps": lm_bytes / bare_us / 1e3,
             "frac": lm_bytes / bare_us / 1e3 / HBM_PEAK_GBS,
             "timing": "HIP events around 50 back-to-back launches of the plain GEMV (no norm prologue, no argmax epilogue)",
+        },
+        "gemv_640x2048": {
+            "entry": "tg_qgemv_dev",
+            "algorithmic_bytes": c1_bytes,
+            "warm_us_per_launch": c1_warm_us,
+            "cold_us_per_launch": c1_cold_us,
+            "cold_GBps": c1_bytes / c1_cold_us / 1e3,
+            "timing": f"HIP events around 200 launches on one matrix (warm) and one launch on each of {n_copies} distinct copies "
+                      f"({n_copies * ci * cn >> 20} MB, cold); 1.3 MB per launch is launch-latency bound on this machine",
         },
         "decode_step": {
             "gpu_ms_per_step_events": gpu_ms / args.steps,
