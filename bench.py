@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--profile-steps", type=int, default=32)
     ap.add_argument("--long-prefill", type=int, default=4096,
                     help="tokens of the extra long-prompt prefill measurement, reported beside the headline (0 = skip)")
+    ap.add_argument("--no-small-model", action="store_true",
+                    help="skip the extra 270m-shape measurements (64-token prompt + 256 steps; 16384-token prefill + 256 steps)")
     ap.add_argument("--graphs", action="store_true", help="replay captured HIP graphs instead of plain stream launches")
     ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
     ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
@@ -262,6 +264,44 @@ def main():
         long_prefill = {"tokens": args.long_prefill, "ms": 1e3 * dt, "tok_s": args.long_prefill / dt}
         del s2
 
+    # ---- the 270m shape, reported beside the headline: 64-token prompt + 256 greedy steps, and a 16384-token
+    # prefill + 256 greedy steps at that context.  Its layer weights (100 MB) fit the 256 MB memory-side cache. ----
+    small = None
+    if args.model == "1B" and not args.no_small_model:
+        del sess, model
+        scfg = tg.named_config("270m")
+        simg = tgw.random_weight_image(scfg, args.seed + 1)
+        smodel = tg.Transformer(scfg)
+        smodel.read_weights_mem(simg)
+        del simg
+        ss = smodel.session()
+        s_bytes = MODELS["270m"][1]
+
+        def run(n_prompt_s, n_steps):
+            ids = rng.integers(0, scfg.n_vocab, n_prompt_s).astype(np.int32)
+            ss.reset()
+            ss.prefill(ids, want_logits=False)  # allocates the workspace for this length
+            ss.reset()
+            tg.synchronize()
+            t0 = time.perf_counter()
+            ss.prefill(ids, want_logits=False)
+            tp = time.perf_counter() - t0
+            ss.decode_enqueue(16)
+            tg.synchronize()
+            t0 = time.perf_counter()
+            ss.decode_enqueue(n_steps)
+            tg.synchronize()
+            td = time.perf_counter() - t0
+            return {"prompt_tokens": n_prompt_s, "prefill_ms": 1e3 * tp, "prefill_tok_s": n_prompt_s / tp, "decode_steps": n_steps,
+                    "decode_tok_s": n_steps / td, "ms_per_step": 1e3 * td / n_steps}
+
+        short, long_ctx = run(64, 256), run(16384, 256)
+        short["weight_stream_GBps"] = s_bytes * short["decode_tok_s"] / 1e9
+        short["frac_of_hbm_roofline"] = short["weight_stream_GBps"] / HBM_PEAK_GBS
+        small = {"shape": "gemma-3-270m", "weight_bytes_per_token": s_bytes, "prompt64_decode256": short,
+                 "prompt16384_decode256": long_ctx}
+        del ss, smodel
+
     tok_s = args.steps / wall
     out = {
         "metric": "decode_tokens_per_s",
@@ -324,6 +364,7 @@ def main():
         },
         "prefill": {"tokens": n_prompt, "tok_s_forward_only": n_prompt / t_prefill, "ms": 1e3 * t_prefill,
                     "first_call_ms": 1e3 * t_prefill_first, "long_prompt": long_prefill},
+        "gemma3_270m": small,
         "setup_s": {"generate_weights": t_gen, "upload_and_retile": t_load},
         "device": dev,
     }
