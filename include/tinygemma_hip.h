@@ -151,6 +151,9 @@ int tg_set_taps(int enable);
  * (exact integer accumulation, fp32-rounding-level accuracy),
  * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */
 int tg_set_gemm_mode(int mfma);
+/* prefill, int8 matrix path: 1 (default) = the output and down projections run as two half-K copies of their grid
+ * when that fills the last round of workgroups better (the following norm adds the halves); 0 = never */
+int tg_set_gemm_split(int enable);
 /* prefill attention: 1 (default) = bf16 matrix cores on three bf16 planes of every fp32 operand (six cross terms per
  * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), workgroups of 32 query positions
  * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;

@@ -35,6 +35,7 @@ int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
 int g_n_cu = 256;
+bool g_gemm_split = true;       // prefill: products with a badly filled last round of workgroups run as two half-K copies
 int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 
@@ -148,12 +149,15 @@ TgGemv gemv_base(const PackedMat &p) {
 //   prepacked : the producer of A already wrote the digit planes and row factors
 //   amax_in   : partial row maxima of A left by its producer ([amax_parts][rows]; saves the pass over A that finds them)
 //   amax_out  : GEGLU only: where this product leaves the partial row maxima of C, one part per column tile
+//   C_half2   : MFMA path, STORE only, and only where tg_gemm_mfma_wants_split says so: the product runs as two half-K
+//               copies, the second half's partial result goes here and the consumer adds the two
 void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
                  int lut_size, int8_t *apack, float *rowscale, bool prepacked = false, const float *amax_in = nullptr,
-                 int amax_parts = 0, float *amax_out = nullptr) {
+                 int amax_parts = 0, float *amax_out = nullptr, float *C_half2 = nullptr) {
 	if (g_gemm_mfma) {
 		if (!prepacked) tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, amax_in, amax_parts, g_stream);
-		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, amax_out, g_stream);
+		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, amax_out, C_half2,
+		                    g_stream);
 	} else {
 		(void)lda;  // the exact kernel reads dense rows (lda == K at every call site)
 		tg_launch_gemm(C, A, p.W, p.scales, m, p.K, p.ntiles, p.C, epi, lut, gmin, geps, lut_size, g_stream);
@@ -1108,6 +1112,11 @@ int tg_set_attn_prefill_mode(int mode) {
 	return TG_OK;
 }
 
+int tg_set_gemm_split(int enable) {
+	g_gemm_split = enable != 0;
+	return TG_OK;
+}
+
 int tg_set_taps(int enable) {
 	g_keep_taps = enable != 0;
 	return TG_OK;
@@ -1252,7 +1261,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	};
 	const size_t o_ids = carve(sizeof(int) * S), o_x = carve(sizeof(float) * S * h), o_xn = carve(sizeof(float) * S * h),
 	             o_qkv = carve(sizeof(float) * S * nq), o_ao = carve(sizeof(float) * S * qo), o_t = carve(sizeof(float) * S * h),
-	             o_hb = carve(sizeof(float) * S * f),
+	             o_t2 = carve(sizeof(float) * S * h), o_hb = carve(sizeof(float) * S * f),
 	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
 	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
 	             o_amax = carve(g_gemm_mfma ? sizeof(float) * (size_t)std::max(2 * f / TG_CT, c.n_head) * tg_gemm_mfma_rows(n) : 0),
@@ -1267,7 +1276,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	uint8_t *ws = (uint8_t *)s->pf_ws;
 	int *d_ids = (int *)(ws + o_ids);
 	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
-	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
+	      *t = (float *)(ws + o_t), *t2 = (float *)(ws + o_t2), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
 	int8_t *apack = (int8_t *)(ws + o_apack);
 	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // partial row maxima: max|ao| per (head, row), then max|hb| per (up|gate tile, row)
 	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
@@ -1284,7 +1293,12 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	// xn = rmsnorm(x, attn_pre of layer 0)
 	// With the int8 MFMA GEMM the norm writes the GEMM's digit planes itself and the fp32 row is not stored.
 	const bool pk = g_gemm_mfma;
-	tg_launch_norm_rows(pk ? nullptr : xn, x, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale, g_stream);
+	tg_launch_norm_rows(pk ? nullptr : xn, x, nullptr, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale,
+	                    g_stream);
+	// products whose plain grid would leave most compute units idle in its last round run as two half-K copies; the
+	// norm that consumes them adds the halves
+	float *o_h2 = (pk && g_gemm_split && tg_gemm_mfma_wants_split(n, qo, m->L[0].o.ntiles_g, g_n_cu)) ? t2 : nullptr;
+	float *d_h2 = (pk && g_gemm_split && tg_gemm_mfma_wants_split(n, f, m->L[0].d.ntiles_g, g_n_cu)) ? t2 : nullptr;
 	for (int l = 0; l < L; l++) {
 		const LayerDev &Ld = m->L[(size_t)l];
 		const int mp = s->max_pos[(size_t)l];
@@ -1297,18 +1311,18 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
 		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, plan.get(), amax, g_n_cu, g_stream);
 		// O (modules.hpp:127-128)
-		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0);
+		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0, nullptr, o_h2);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
-		tg_launch_norm_rows(pk ? nullptr : xn, t, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
+		tg_launch_norm_rows(pk ? nullptr : xn, t, o_h2, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
 		TG_TRY(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
 		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, 0, amax);
-		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g);
+		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g, nullptr, d_h2);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
 		// the last layer's final norm feeds the LM head GEMV, which reads the fp32 row
 		const bool last = l + 1 == L;
-		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
+		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, d_h2, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
 		                    g_stream);
 		TG_TRY(tap(2 * l + 2));
 	}

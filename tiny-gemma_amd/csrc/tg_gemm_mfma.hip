@@ -129,7 +129,8 @@ __global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda
 template <bool GEGLU, bool LUTLDS>
 __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
                                                       const float *scales, int M, int K, int ldc, const float *lut, float gmin,
-                                                      float geps, float ginv, int lut_size, float *rowmax_part, int Mpad) {
+                                                      float geps, float ginv, int lut_size, float *rowmax_part, int Mpad, int ksplit,
+                                                      size_t csplit) {
 	// B operands of one stage: [k / 16][column][16 bytes], double buffered
 	__shared__ __attribute__((aligned(16))) i32x4 Bs[2][KSTAGE / 16][TG_CT];
 	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
@@ -157,15 +158,22 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 			mblock = (int)blockIdx.y;
 		}
 	}
+	// ksplit == 2: the grid holds every row block twice; copy z walks half z of K and writes its own partial result
+	// (C + z * csplit), which the consumer adds.  Used where the plain grid would leave most compute units idle in
+	// its last round (288 workgroups on 256 compute units).
+	const int mreal = (int)gridDim.y / ksplit, z = mblock / mreal;
+	mblock -= z * mreal;
 	const int mtile = mblock * 4 + w;
-	const int nstage = K / KSTAGE;
+	const int nstage = K / KSTAGE / ksplit;
 	if (GEGLU && LUTLDS) {  // the table is read once per output element; visible after the first barrier
 		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
 	}
+	C += (size_t)z * csplit;
 
 	// a stage of B is 8 KB contiguous: 512 pieces of 16 bytes, two per thread
-	const i32x4 *bsrc = reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + tid;
-	const i32x4 *asrc = reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane;
+	const i32x4 *bsrc = reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + tid + (size_t)z * nstage * 512;
+	const i32x4 *asrc =
+	    reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane + (size_t)z * nstage * 6 * 64;
 	i32x4 *bdst = &Bs[0][0][0] + tid;
 
 	// Software pipeline, all through registers (one wave per SIMD: nothing else hides latency):
@@ -458,7 +466,7 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 // rowmax_part (GEGLU only, may be null): [ntiles][tg_gemm_mfma_rows(M)] floats, max|C[m][tile's columns]|
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
-                         hipStream_t s) {
+                         float *C_half2, hipStream_t s) {
 	const unsigned mblocks = (unsigned)((M + 127) / 128);
 	const int Mpad = (int)tg_gemm_mfma_rows(M);
 	const float *rowinv = rowfac + Mpad;
@@ -481,14 +489,29 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 			                   geps, ginv, lut_size, rmp, Mpad);
 		return;
 	}
-	const dim3 grid((unsigned)ntiles, mblocks), block(GNT);
+	// C_half2 != nullptr (STORE only; see tg_gemm_mfma_wants_split): two half-K copies of the grid, the second writes C_half2
+	const int ksplit = (C_half2 != nullptr && !geglu) ? 2 : 1;
+	const size_t csplit = ksplit == 2 ? (size_t)(C_half2 - C) : 0;
+	const dim3 grid((unsigned)ntiles, mblocks * (unsigned)ksplit), block(GNT);
 	if (geglu && lutlds)
 		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
-		                   lut_size, rmp, Mpad);
+		                   lut_size, rmp, Mpad, 1, (size_t)0);
 	else if (geglu)
 		hipLaunchKernelGGL((gemm_i8_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
-		                   lut_size, rmp, Mpad);
+		                   lut_size, rmp, Mpad, 1, (size_t)0);
 	else
 		hipLaunchKernelGGL((gemm_i8_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
-		                   lut_size, rmp, Mpad);
+		                   lut_size, rmp, Mpad, ksplit, csplit);
 }
+
+// Whether a STORE product of M rows, K deep, ntiles column tiles should run as two half-K copies whose results the
+// consumer adds: when that fills the last round of workgroups noticeably better.  Needs whole pairs of stages per half.
+bool tg_gemm_mfma_wants_split(int M, int K, int ntiles, int n_cu) {
+	if (M <= TG_GEMM_SKINNY_ROWS || (K / KSTAGE) % 4 != 0) return false;
+	const long wgs = (long)((M + 127) / 128) * ntiles;
+	auto eff = [&](long n) { return (double)n / (double)(((n + n_cu - 1) / n_cu) * n_cu); };
+	// measured: worth it only when the last round is nearly empty (288 workgroups on 256 compute units: -2 % prefill time);
+	// at 0.75 or better the second prologue/epilogue and the extra partial result cost more than the idle units
+	return eff(wgs) < 0.6 && eff(2 * wgs) > eff(wgs) + 0.1;
+}
+

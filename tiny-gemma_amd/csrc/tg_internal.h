@@ -157,8 +157,8 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 // out = rmsnorm(in, w); if resid != null first in = rmsnorm(in, w_post) + resid is formed and stored to resid_out
 // apack/rowfac non-null: the normalised rows are also (out == nullptr: only) written as digit planes + row factors for
 // tg_launch_gemm_mfma (rowfac as tg_launch_quant_pack lays it out for S rows)
-void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
-                         int S, int dim, int8_t *apack, float *rowfac, hipStream_t s);
+void tg_launch_norm_rows(float *out, const float *in, const float *in2, const float *w_pre, const float *w_post, const float *resid,
+                         float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s);
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
                                  const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
                                  hipStream_t s);
@@ -203,7 +203,8 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
                           hipStream_t s);
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
-                         hipStream_t s);
+                         float *C_half2, hipStream_t s);
+bool tg_gemm_mfma_wants_split(int M, int K, int ntiles, int n_cu);
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global load of the wave (its fence covers all address spaces), which would drain a software pipeline

@@ -47,9 +47,9 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 // goes out as fp32 (out != nullptr) and/or straight as the int8 digit planes + row factors of the MFMA GEMM that
 // consumes it (apack != nullptr): the same bits the stand-alone quantising pre-pass would produce from the fp32 row.
 template <int ROUNDS>
-__global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *w_pre, const float *w_post,
-                                                        const float *resid, float *resid_out, int S, int dim, int8_t *apack,
-                                                        float *rowfac, int Mpad) {
+__global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *in2, const float *w_pre,
+                                                        const float *w_post, const float *resid, float *resid_out, int S, int dim,
+                                                        int8_t *apack, float *rowfac, int Mpad) {
 	typedef float f32x4 __attribute__((ext_vector_type(4)));
 	const int lane = threadIdx.x & 63, s = blockIdx.x * (RNT / 64) + (threadIdx.x >> 6);
 	if (s >= S) return;  // uniform over the wave
@@ -66,6 +66,12 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 		off[r] = act[r] ? (size_t)piece * 16 : 0;
 #pragma unroll
 		for (int q = 0; q < 4; q++) v[r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)s * dim + off[r] + 4 * q);
+	}
+	if (in2 != nullptr) {  // the row arrives as two addends (a product computed in two halves of K)
+#pragma unroll
+		for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+			for (int q = 0; q < 4; q++) v[r][q] += *reinterpret_cast<const f32x4 *>(in2 + (size_t)s * dim + off[r] + 4 * q);
 	}
 	if (resid != nullptr) {
 #pragma unroll
@@ -246,15 +252,17 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 	hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, x, ids, wte, scales, hidden, vocab, emb_scale);
 }
 
-void tg_launch_norm_rows(float *out, const float *in, const float *w_pre, const float *w_post, const float *resid, float *resid_out,
-                         int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
+void tg_launch_norm_rows(float *out, const float *in, const float *in2, const float *w_pre, const float *w_post, const float *resid,
+                         float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(S);
 	const dim3 grid((unsigned)((S + RNT / 64 - 1) / (RNT / 64))), block(RNT);
 	// dim is a legal row dimension: a multiple of 16, at most 2048 where a norm is applied (hidden sizes 640 and 1152)
 	if (dim <= 1024)
-		hipLaunchKernelGGL(norm_rows_kernel<1>, grid, block, 0, s, out, in, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac, Mpad);
+		hipLaunchKernelGGL(norm_rows_kernel<1>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
+		                   Mpad);
 	else
-		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac, Mpad);
+		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
+		                   Mpad);
 }
 
 // Wp/scales: GEMV tiling of the matrix (ntiles tiles of Ct columns); C gets ntiles * Ct columns, or half of that for GEGLU
