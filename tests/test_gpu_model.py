@@ -301,3 +301,26 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
     with pytest.raises(tg.TgError) as e:
         tg.Transformer(bad)
     assert e.value.code == -1
+
+
+def test_half_k_grid_copies_equal_the_plain_grid(tg, oracle, weight_images, tables):
+    """Prefill with the output/down projections computed as two half-K copies added by the following norm
+    (taken when the plain grid fills its last round badly: here 1000 rows x 5 column tiles) against the
+    same prefill with the plain grid: same ids, logits equal to fp32 rounding of one extra addition."""
+    cfg = tg.named_config("270m", 2)
+    image = oracle.generate_weights(gi.oracle_config("270m", 2), 21)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(image)
+    sess = model.session(gsize=1 << 20)
+    prompt = gi.prompt_ids(33, 1000)
+    out = []
+    try:
+        for split in (1, 0):
+            tg.check(tg.lib().tg_set_gemm_split(split))
+            sess.reset()
+            out.append(sess.prefill(prompt))
+    finally:
+        tg.check(tg.lib().tg_set_gemm_split(1))
+    (tok_a, lg_a), (tok_b, lg_b) = out
+    assert tok_a == tok_b and normrel(lg_a, lg_b) < 2e-5
+    assert not np.array_equal(lg_a, lg_b)   # the two paths really differ (the split was taken)
