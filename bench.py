@@ -104,8 +104,9 @@ def main():
     ap.add_argument("--profile-steps", type=int, default=32)
     ap.add_argument("--long-prefill", type=int, default=4096,
                     help="tokens of the extra long-prompt prefill measurement, reported beside the headline (0 = skip)")
-    ap.add_argument("--no-small-model", action="store_true",
-                    help="skip the extra 270m-shape measurements (64-token prompt + 256 steps; 16384-token prefill + 256 steps)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the extra measurements that launch the same kernels at other shapes (640x2048 matvec; 270m shape), "
+                         "so that a profiler's per-kernel statistics describe the headline workload only")
     ap.add_argument("--graphs", action="store_true", help="replay captured HIP graphs instead of plain stream launches")
     ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
     ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
@@ -224,31 +225,42 @@ def main():
     # (rotating over distinct copies that together exceed the 256 MB memory-side cache twice over) ----
     ci, cn = 640, 2048
     c1_bytes = ci * cn + 4 * cn + 4 * ci + 4 * cn
-    n_copies = (512 << 20) // (ci * cn) + 1
-    crng = np.random.default_rng(101)
-    Wc = crng.integers(-127, 128, (ci, cn), dtype=np.int8)
-    sc = crng.uniform(0.001, 0.02, cn).astype(np.float32)
-    copies = [tg.QWeight(Wc, sc) for _ in range(n_copies)]
-    cx = tg.DeviceBuffer.from_numpy(crng.standard_normal(ci).astype(np.float32))
-    cy = tg.DeviceBuffer(4 * cn)
-    for q_ in copies[:8]:
-        q_.gemv(cy, cx)
-    tg.synchronize()
-    ev.record(e0, stream)
-    for _ in range(200):
-        copies[0].gemv(cy, cx)
-    ev.record(e1, stream)
-    tg.synchronize()
-    c1_warm_us = ev.elapsed_ms(e0, e1) * 1e3 / 200
-    ev.record(e0, stream)
-    for q_ in copies:
-        q_.gemv(cy, cx)
-    ev.record(e1, stream)
-    tg.synchronize()
-    c1_cold_us = ev.elapsed_ms(e0, e1) * 1e3 / n_copies
-    for q_ in copies:
-        q_.free()
-    del copies
+    c1 = None
+    if not args.headline_only:
+        n_copies = (512 << 20) // (ci * cn) + 1
+        crng = np.random.default_rng(101)
+        Wc = crng.integers(-127, 128, (ci, cn), dtype=np.int8)
+        sc = crng.uniform(0.001, 0.02, cn).astype(np.float32)
+        copies = [tg.QWeight(Wc, sc) for _ in range(n_copies)]
+        cx = tg.DeviceBuffer.from_numpy(crng.standard_normal(ci).astype(np.float32))
+        cy = tg.DeviceBuffer(4 * cn)
+        for q_ in copies[:8]:
+            q_.gemv(cy, cx)
+        tg.synchronize()
+        ev.record(e0, stream)
+        for _ in range(200):
+            copies[0].gemv(cy, cx)
+        ev.record(e1, stream)
+        tg.synchronize()
+        c1_warm_us = ev.elapsed_ms(e0, e1) * 1e3 / 200
+        ev.record(e0, stream)
+        for q_ in copies:
+            q_.gemv(cy, cx)
+        ev.record(e1, stream)
+        tg.synchronize()
+        c1_cold_us = ev.elapsed_ms(e0, e1) * 1e3 / n_copies
+        for q_ in copies:
+            q_.free()
+        del copies
+        c1 = {
+            "entry": "tg_qgemv_dev",
+            "algorithmic_bytes": c1_bytes,
+            "warm_us_per_launch": c1_warm_us,
+            "cold_us_per_launch": c1_cold_us,
+            "cold_GBps": c1_bytes / c1_cold_us / 1e3,
+            "timing": f"HIP events around 200 launches on one matrix (warm) and one launch on each of {n_copies} distinct copies "
+                      f"({n_copies * ci * cn >> 20} MB, cold); 1.3 MB per launch is launch-latency bound on this machine",
+        }
 
     # ---- long-prompt prefill (the matrix-matrix path) on a fresh session ----
     long_prefill = None
@@ -267,7 +279,7 @@ def main():
     # ---- the 270m shape, reported beside the headline: 64-token prompt + 256 greedy steps, and a 16384-token
     # prefill + 256 greedy steps at that context.  Its layer weights (100 MB) fit the 256 MB memory-side cache. ----
     small = None
-    if args.model == "1B" and not args.no_small_model:
+    if args.model == "1B" and not args.headline_only:
         del sess, model
         scfg = tg.named_config("270m")
         simg = tgw.random_weight_image(scfg, args.seed + 1)
@@ -346,15 +358,7 @@ def main():
             "frac": lm_bytes / bare_us / 1e3 / HBM_PEAK_GBS,
             "timing": "HIP events around 50 back-to-back launches of the plain GEMV (no norm prologue, no argmax epilogue)",
         },
-        "gemv_640x2048": {
-            "entry": "tg_qgemv_dev",
-            "algorithmic_bytes": c1_bytes,
-            "warm_us_per_launch": c1_warm_us,
-            "cold_us_per_launch": c1_cold_us,
-            "cold_GBps": c1_bytes / c1_cold_us / 1e3,
-            "timing": f"HIP events around 200 launches on one matrix (warm) and one launch on each of {n_copies} distinct copies "
-                      f"({n_copies * ci * cn >> 20} MB, cold); 1.3 MB per launch is launch-latency bound on this machine",
-        },
+        "gemv_640x2048": c1,
         "decode_step": {
             "gpu_ms_per_step_events": gpu_ms / args.steps,
             "weight_bytes_per_token": step_bytes,
