@@ -219,6 +219,11 @@ struct AttnPlanDev {
 		const int tile = tg_attn_prefill_query_tile(n_tokens, g_n_cu);
 		if (n_tokens == S && tile == tq) return TG_OK;
 		release();
+		const int rc = build_uncached(n_tokens, tile);
+		if (rc != TG_OK) release();  // nothing half-built stays behind as a cache hit
+		return rc;
+	}
+	int build_uncached(int n_tokens, int tile) {
 		int nslots = 0;
 		use = tg_attn_prefill_plan(n_tokens, g_n_cu, tile, items, split, nslots);
 		S = n_tokens;
