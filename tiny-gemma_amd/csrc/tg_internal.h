@@ -321,6 +321,30 @@ __device__ __forceinline__ void tg_quant16(const float *v, float mul, tg_i32x4 p
 		pl[2][q] = (int)d2;
 	}
 }
+// v[8] consecutive k of one row -> the 8 bytes of each plane (half of a lane's piece)
+__device__ __forceinline__ void tg_quant8(const float *v, float mul, uint2 pl[3]) {
+	unsigned d[3][2];
+#pragma unroll
+	for (int q = 0; q < 2; q++) {
+		unsigned d0 = 0, d1 = 0, d2 = 0;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int xi = (int)rintf(v[4 * q + i] * mul);
+			const int a0 = (xi << 24) >> 24;
+			const int r1 = (xi - a0) >> 8;
+			const int a1 = (r1 << 24) >> 24;
+			const int a2 = (r1 - a1) >> 8;
+			d0 |= (unsigned)(a0 & 255) << (8 * i);
+			d1 |= (unsigned)(a1 & 255) << (8 * i);
+			d2 |= (unsigned)(a2 & 255) << (8 * i);
+		}
+		d[0][q] = d0;
+		d[1][q] = d1;
+		d[2][q] = d2;
+	}
+#pragma unroll
+	for (int p = 0; p < 3; p++) pl[p] = uint2{d[p][0], d[p][1]};
+}
 // where the 16 bytes of (row m, k0 = multiple of 16) of plane 0 go; planes are 64 pieces apart
 __device__ __forceinline__ tg_i32x4 *tg_plane_dst(int8_t *apack, int m, int k0, int K) {
 	const int kb = k0 >> 5, hb = (k0 >> 4) & 1;

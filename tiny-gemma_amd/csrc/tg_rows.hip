@@ -42,10 +42,11 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 	for (int d = threadIdx.x; d < hidden; d += RNT) x[(size_t)s * hidden + d] = scales[d] * (emb_scale * (float)row[d]);
 }
 
-// One wave per row, the row held in registers (16 consecutive elements per lane and round; ROUNDS = 2 covers rows of
-// up to 2048 elements), wave reductions only: [post-norm + residual (+ residual out)] + pre-norm.  The normalised row
-// goes out as fp32 (out != nullptr) and/or straight as the int8 digit planes + row factors of the MFMA GEMM that
-// consumes it (apack != nullptr): the same bits the stand-alone quantising pre-pass would produce from the fp32 row.
+// One wave per row, the row held in registers (8 consecutive elements per lane and round; ROUNDS = 3 covers the
+// 1152-wide rows with 24 values per lane, which keeps the kernel at four rows per SIMD), wave reductions only:
+// [post-norm + residual (+ residual out)] + pre-norm.  The normalised row goes out as fp32 (out != nullptr) and/or
+// straight as the int8 digit planes + row factors of the MFMA GEMM that consumes it (apack != nullptr): the same bits
+// the stand-alone quantising pre-pass would produce from the fp32 row.
 template <int ROUNDS>
 __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *in2, const float *w_pre,
                                                         const float *w_post, const float *resid, float *resid_out, int S, int dim,
@@ -54,30 +55,30 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 	const int lane = threadIdx.x & 63, s = blockIdx.x * (RNT / 64) + (threadIdx.x >> 6);
 	if (s >= S) return;  // uniform over the wave
 	const float eps = 1e-06f;
-	const int npieces = dim >> 4;
+	const int npieces = dim >> 3;
 	bool act[ROUNDS];
 	size_t off[ROUNDS];  // element offset of this lane's piece inside a row (clamped to piece 0 when the lane idles)
-	f32x4 v[ROUNDS][4], rs[ROUNDS][4], wpo[ROUNDS][4], wpr[ROUNDS][4];
+	f32x4 v[ROUNDS][2], rs[ROUNDS][2], wpo[ROUNDS][2], wpr[ROUNDS][2];
 	// every load of the row is requested before the first use
 #pragma unroll
 	for (int r = 0; r < ROUNDS; r++) {
 		const int piece = lane + 64 * r;
 		act[r] = piece < npieces;
-		off[r] = act[r] ? (size_t)piece * 16 : 0;
+		off[r] = act[r] ? (size_t)piece * 8 : 0;
 #pragma unroll
-		for (int q = 0; q < 4; q++) v[r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)s * dim + off[r] + 4 * q);
+		for (int q = 0; q < 2; q++) v[r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)s * dim + off[r] + 4 * q);
 	}
 	if (in2 != nullptr) {  // the row arrives as two addends (a product computed in two halves of K)
 #pragma unroll
 		for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-			for (int q = 0; q < 4; q++) v[r][q] += *reinterpret_cast<const f32x4 *>(in2 + (size_t)s * dim + off[r] + 4 * q);
+			for (int q = 0; q < 2; q++) v[r][q] += *reinterpret_cast<const f32x4 *>(in2 + (size_t)s * dim + off[r] + 4 * q);
 	}
 	if (resid != nullptr) {
 #pragma unroll
 		for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-			for (int q = 0; q < 4; q++) {
+			for (int q = 0; q < 2; q++) {
 				rs[r][q] = *reinterpret_cast<const f32x4 *>(resid + (size_t)s * dim + off[r] + 4 * q);
 				wpo[r][q] = *reinterpret_cast<const f32x4 *>(w_post + off[r] + 4 * q);
 			}
@@ -86,13 +87,13 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 #pragma unroll
 		for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-			for (int q = 0; q < 4; q++) wpr[r][q] = *reinterpret_cast<const f32x4 *>(w_pre + off[r] + 4 * q);
+			for (int q = 0; q < 2; q++) wpr[r][q] = *reinterpret_cast<const f32x4 *>(w_pre + off[r] + 4 * q);
 	}
 	float ss = 0.0f;
 #pragma unroll
 	for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-		for (int q = 0; q < 4; q++) {
+		for (int q = 0; q < 2; q++) {
 			if (!act[r]) v[r][q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
 			for (int e = 0; e < 4; e++) ss = fmaf(v[r][q][e], v[r][q][e], ss);
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 #pragma unroll
 		for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-			for (int q = 0; q < 4; q++) {
+			for (int q = 0; q < 2; q++) {
 				f32x4 t;
 #pragma unroll
 				for (int e = 0; e < 4; e++) {
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 #pragma unroll
 	for (int r = 0; r < ROUNDS; r++)
 #pragma unroll
-		for (int q = 0; q < 4; q++) {
+		for (int q = 0; q < 2; q++) {
 			f32x4 y;
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
@@ -143,16 +144,18 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 #pragma unroll
 	for (int r = 0; r < ROUNDS; r++) {
 		if (!act[r]) continue;
-		float y[16];
+		float y[8];
 #pragma unroll
-		for (int q = 0; q < 4; q++)
+		for (int q = 0; q < 2; q++)
 #pragma unroll
 			for (int e = 0; e < 4; e++) y[4 * q + e] = v[r][q][e];
-		tg_i32x4 pl[3];
-		tg_quant16(y, mul, pl);
-		tg_i32x4 *dst = tg_plane_dst(apack, s, (int)off[r], dim);
+		uint2 pl[3];
+		tg_quant8(y, mul, pl);
+		// two neighbouring lanes share a 16-byte piece of every plane
+		const int k0 = (int)off[r];
+		uint2 *dst = reinterpret_cast<uint2 *>(tg_plane_dst(apack, s, k0 & ~15, dim)) + ((k0 >> 3) & 1);
 #pragma unroll
-		for (int p = 0; p < 3; p++) dst[p * 64] = pl[p];
+		for (int p = 0; p < 3; p++) dst[p * 128] = pl[p];  // planes are 64 pieces of 16 bytes apart
 	}
 }
 
@@ -256,12 +259,12 @@ void tg_launch_norm_rows(float *out, const float *in, const float *in2, const fl
                          float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(S);
 	const dim3 grid((unsigned)((S + RNT / 64 - 1) / (RNT / 64))), block(RNT);
-	// dim is a legal row dimension: a multiple of 16, at most 2048 where a norm is applied (hidden sizes 640 and 1152)
+	// dim is a legal row dimension: a multiple of 16, at most 1536 where a norm is applied (hidden sizes 640 and 1152)
 	if (dim <= 1024)
-		hipLaunchKernelGGL(norm_rows_kernel<1>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
+		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
 		                   Mpad);
 	else
-		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
+		hipLaunchKernelGGL(norm_rows_kernel<3>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
 		                   Mpad);
 }
 
