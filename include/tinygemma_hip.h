@@ -114,6 +114,9 @@ int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin,
 int tg_session_reset(tg_session *s); /* empty KV caches, position 0 */
 void tg_session_destroy(tg_session *s);
 int tg_session_position(const tg_session *s);
+/* tg_forward_prefill keeps its scratch (the reference's PrefillState, decode.hpp:281-351: a few hundred MB for a
+ * 4096-token prompt) in the session for the next prefill; this frees it.  Decode needs none of it. */
+int tg_session_release_workspace(tg_session *s);
 
 /* gemma::forward_prefill (transformer.hpp:49) + ops::argmax_logits (ops.hpp:744).
  * logits (host, [n_vocab]) and argmax may each be NULL.  Needs an empty session. */

@@ -323,4 +323,9 @@ def test_half_k_grid_copies_equal_the_plain_grid(tg, oracle, weight_images, tabl
         tg.check(tg.lib().tg_set_gemm_split(1))
     (tok_a, lg_a), (tok_b, lg_b) = out
     assert tok_a == tok_b and normrel(lg_a, lg_b) < 2e-5
+    # the prefill scratch can be dropped; decode goes on without it and the next prefill allocates it again
+    sess.release_workspace()
+    nxt, _ = sess.decode(tok_b)
+    sess.reset()
+    assert sess.prefill(prompt)[0] == tok_b and sess.decode(tok_b)[0] == nxt
     assert not np.array_equal(lg_a, lg_b)   # the two paths really differ (the split was taken)

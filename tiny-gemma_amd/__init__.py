@@ -88,6 +88,7 @@ def lib():
     L.tg_session_create.argtypes = [C.c_void_p, c_f32p, c_f32p, c_f32p, c_f32p, c_f32p, C.c_float, C.c_float, C.c_int,
                                     C.POINTER(C.c_void_p)]
     L.tg_session_reset.argtypes = [C.c_void_p]
+    L.tg_session_release_workspace.argtypes = [C.c_void_p]
     L.tg_session_destroy.argtypes = [C.c_void_p]
     L.tg_session_position.argtypes = [C.c_void_p]
     L.tg_forward_prefill.argtypes = [C.c_void_p, c_i32p, C.c_int, c_f32p, c_i32p]
@@ -264,6 +265,9 @@ class Session:
         if gelu_table is not None:
             gsize = gelu_table.size
         check(lib().tg_session_create(model.h, _f(rc), _f(rs), _f(lc), _f(ls), _f(gelu_table), gmin, gmax, gsize, C.byref(self.h)))
+
+    def release_workspace(self):
+        check(lib().tg_session_release_workspace(self.h))
 
     def reset(self):
         check(lib().tg_session_reset(self.h))

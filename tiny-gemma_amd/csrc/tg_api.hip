@@ -1122,6 +1122,18 @@ int tg_set_gemm_split(int enable) {
 	return TG_OK;
 }
 
+int tg_session_release_workspace(tg_session *s) {
+	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	TG_HIP(hipStreamSynchronize(g_stream));
+	if (s->pf_ws) (void)hipFree(s->pf_ws);
+	s->pf_ws = nullptr;
+	s->pf_ws_bytes = 0;
+	s->taps = nullptr;  // prefill taps live in the workspace
+	s->tap_rows = 0;
+	s->pf_plan.release();
+	return TG_OK;
+}
+
 int tg_set_taps(int enable) {
 	g_keep_taps = enable != 0;
 	return TG_OK;
