@@ -1,10 +1,12 @@
 // Test harness: plain-C entry points around tiny-gemma_amd/host/tokenizer.hpp so that the Python tests can
-// drive it next to the reference's tokenizer (oracle/ref_wrap.cpp: ref_tok_*), same signatures.
+// drive it next to the reference's tokenizer (oracle/ref_wrap.cpp: ref_tok_*), same signatures; and around the
+// prompt builder of the pass key run (tiny-gemma_amd/host/passkey.hpp).
 #include <algorithm>
 #include <cstring>
 #include <string>
 #include <vector>
 
+#include "../../tiny-gemma_amd/host/passkey.hpp"
 #include "../../tiny-gemma_amd/host/tokenizer.hpp"
 
 using tinygemma::sentencepiece::Tokenizer;
@@ -48,5 +50,17 @@ int tok_decode(void *tp, const int *ids, int n, char *out, int cap) {
 	}
 }
 int tok_byte_of(void *tp, int token) { return static_cast<Tokenizer *>(tp)->byte_of(token); }
+
+int passkey_prompt(int n_garbage, int n_garbage_prefix, int key, char *out, int cap) {
+	const std::string p = tinygemma::passkey::build_prompt(n_garbage, n_garbage_prefix, key);
+	std::memcpy(out, p.data(), std::min((size_t)cap, p.size()));
+	return (int)p.size();
+}
+void passkey_draw(unsigned seed, int n_garbage, int *n_garbage_prefix, int *key) {
+	std::mt19937 gen(seed);
+	auto d = tinygemma::passkey::draw(n_garbage, gen);
+	*n_garbage_prefix = d.first;
+	*key = d.second;
+}
 
 }  // extern "C"

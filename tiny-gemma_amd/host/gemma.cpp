@@ -12,59 +12,11 @@
 // Build: g++ -std=c++20 -O2 gemma.cpp -o gemma -L.. -ltinygemma_hip -Wl,-rpath,'$ORIGIN/..'
 
 #include <cstdio>
-#include <functional>
 #include <iostream>
-#include <map>
 #include <string>
 
+#include "options.hpp"
 #include "tinygemma.hpp"
-
-namespace {
-
-struct Options {
-	std::map<std::string, std::pair<std::function<void(const std::string &)>, std::string>> opts;
-	void add(const std::string &name, std::string &dst, const std::string &help) {
-		opts[name] = {[&dst](const std::string &v) { dst = v; }, help};
-	}
-	void add(const std::string &name, int &dst, const std::string &help) {
-		opts[name] = {[&dst](const std::string &v) {
-			              try {
-				              dst = std::stoi(v);
-			              } catch (...) {
-				              throw std::invalid_argument("expected integer for " + v);
-			              }
-		              },
-		              help};
-	}
-	void add(const std::string &name, float &dst, const std::string &help) {
-		opts[name] = {[&dst](const std::string &v) {
-			              try {
-				              dst = std::stof(v);
-			              } catch (...) {
-				              throw std::invalid_argument("expected float for " + v);
-			              }
-		              },
-		              help};
-	}
-	int usage(const char *prog, const std::string &msg) const {
-		std::cerr << "Error: " << msg << "\n\nCLI Application for Gemma 3 text generation.\nUsage: " << prog << " [options]\n\nOptions:\n";
-		for (const auto &[name, o] : opts) std::cerr << "  --" << name << "\t" << o.second << '\n';
-		return 1;
-	}
-	int parse(int argc, char **argv) const {
-		for (int i = 1; i < argc; ++i) {
-			const std::string arg = argv[i];
-			if (arg.rfind("--", 0) != 0) return usage(argv[0], "unexpected token: " + arg);
-			auto it = opts.find(arg.substr(2));
-			if (it == opts.end()) return usage(argv[0], "unknown option: " + arg);
-			if (i + 1 == argc) return usage(argv[0], "missing value for " + arg);
-			it->second.first(argv[++i]);
-		}
-		return 0;
-	}
-};
-
-}  // namespace
 
 int main(int argc, char **argv) {
 	using namespace tinygemma;
@@ -76,7 +28,7 @@ int main(int argc, char **argv) {
 	int chat_format = 0;
 	int terminate_on_eos = 0;
 
-	Options app;
+	Options app("CLI Application for Gemma 3 text generation.");
 	app.add("weights_path", weights_path, "File path for model weights.");
 	app.add("model_size", model_size, "Model size to load.");
 	app.add("prompt", prompt, "The prompt.");
