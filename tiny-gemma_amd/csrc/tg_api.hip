@@ -455,6 +455,8 @@ int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 			if (g_rowscale) (void)hipFree(g_rowscale);
 			g_apack = nullptr;
 			g_rowscale = nullptr;
+			g_apack_bytes = 0;  // a failed allocation below must not leave the old sizes standing for the freed buffers
+			g_rowscale_n = 0;
 			TG_HIP(hipMalloc((void **)&g_apack, need));
 			TG_HIP(hipMalloc((void **)&g_rowscale, need_rs * sizeof(float)));
 			g_apack_bytes = need;
@@ -845,9 +847,7 @@ int tg_session_reset(tg_session *s) {
 	TG_HIP(hipMemset(s->xr, 0, sizeof(float) * (size_t)(2 * c.n_layers + 1) * c.hidden_size));
 	TG_HIP(hipDeviceSynchronize());
 	s->pos = s->bp_local = s->bp_global = s->steps = 0;
-	if (s->taps) {
-		s->taps = nullptr;
-	}
+	s->taps = nullptr;
 	s->tap_rows = 0;
 	return TG_OK;
 }
@@ -1207,11 +1207,6 @@ int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out) {
 // ---------------------------------------------------------------------------------------------
 // forward_prefill
 // ---------------------------------------------------------------------------------------------
-}  // extern "C"
-
-
-extern "C" {
-
 int tg_attention_prefill(float *o, const float *q, const float *k, const float *v, int S, int is_sw, int sw_context) {
 	if (int rc = ensure_init()) return rc;
 	if (!o || !q || !k || !v || S < 1 || sw_context < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
@@ -1258,15 +1253,6 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	const int L = c.n_layers, h = c.hidden_size, f = c.intermediate_size, hd = c.head_dim;
 	const int qo = c.n_head * hd, nq = qo + 2 * hd;
 	const size_t S = (size_t)n;
-	auto cleanup = [&]() {};  // the workspace belongs to the session
-#define TG_TRY(expr)                                                                             \
-	do {                                                                                         \
-		hipError_t e_ = (expr);                                                                  \
-		if (e_ != hipSuccess) {                                                                  \
-			cleanup();                                                                           \
-			return tg_fail(TG_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));       \
-		}                                                                                        \
-	} while (0)
 	// PrefillState (decode.hpp:281-351): carved out of one arena the session keeps (hipMalloc/hipFree of a few hundred
 	// MB per call cost milliseconds), 256-byte aligned pieces
 	const bool keep_taps = g_keep_taps && n <= PREFILL_TAP_MAX_ROWS;
@@ -1287,7 +1273,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		if (s->pf_ws) (void)hipFree(s->pf_ws);
 		s->pf_ws = nullptr;
 		s->pf_ws_bytes = 0;
-		TG_TRY(hipMalloc(&s->pf_ws, need));
+		TG_HIP(hipMalloc(&s->pf_ws, need));
 		s->pf_ws_bytes = need;
 	}
 	uint8_t *ws = (uint8_t *)s->pf_ws;
@@ -1304,9 +1290,9 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		if (!keep_taps) return hipSuccess;
 		return hipMemcpyAsync(s->taps + (size_t)b * S * h, x, sizeof(float) * S * h, hipMemcpyDeviceToDevice, g_stream);
 	};
-	TG_TRY(hipMemcpyAsync(d_ids, ids, sizeof(int) * S, hipMemcpyHostToDevice, g_stream));
+	TG_HIP(hipMemcpyAsync(d_ids, ids, sizeof(int) * S, hipMemcpyHostToDevice, g_stream));
 	tg_launch_embed_rows(x, d_ids, n, m->wte, m->wte_scales, h, c.n_vocab, g_stream);
-	TG_TRY(tap(0));
+	TG_HIP(tap(0));
 	// xn = rmsnorm(x, attn_pre of layer 0)
 	// With the int8 MFMA GEMM the norm writes the GEMM's digit planes itself and the fp32 row is not stored.
 	const bool pk = g_gemm_mfma;
@@ -1331,7 +1317,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0, nullptr, o_h2);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
 		tg_launch_norm_rows(pk ? nullptr : xn, t, o_h2, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
-		TG_TRY(tap(2 * l + 1));
+		TG_HIP(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
 		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, 0, amax);
 		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g, nullptr, d_h2);
@@ -1341,7 +1327,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		const bool last = l + 1 == L;
 		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, d_h2, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
 		                    g_stream);
-		TG_TRY(tap(2 * l + 2));
+		TG_HIP(tap(2 * l + 2));
 	}
 	// LM head on the last position only (modules.hpp:232-240): xn already holds rmsnorm(x, RMSw)
 	{
@@ -1353,20 +1339,19 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		tg_launch_gemv(g, TG_ROLE_LMHEAD_PLAIN, g_stream);
 		tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 0, g_stream);
 	}
-	TG_TRY(hipGetLastError());
+	TG_HIP(hipGetLastError());
 	// KVCache::update_prefill's counters (decode.hpp:99-104)
 	s->pos = n;
 	s->bp_local = (n >= c.n_pos_local) ? c.n_pos_local : n;
 	s->bp_global = (n >= c.n_pos) ? c.n_pos : n;
 	s->steps = 1;
 	int ctr[3] = {s->pos, s->bp_local, s->bp_global};
-	TG_TRY(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
-	if (logits) TG_TRY(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)c.n_vocab, hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
+	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)c.n_vocab, hipMemcpyDeviceToHost, g_stream));
 	int32_t tok = -1;
-	TG_TRY(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
-	TG_TRY(hipStreamSynchronize(g_stream));
+	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
 	if (argmax) *argmax = tok;
-#undef TG_TRY
 	return TG_OK;
 }
 
