@@ -157,6 +157,9 @@ int tg_set_gemm_mode(int mfma);
 /* prefill, int8 matrix path: 1 (default) = the output and down projections run as two half-K copies of their grid
  * when that fills the last round of workgroups better (the following norm adds the halves); 0 = never */
 int tg_set_gemm_split(int enable);
+/* prefill, int8 matrix path: 1 (default) = one resident workgroup per compute unit walks its share of the output
+ * tiles, the operand prefetch running on from one tile into the next; 0 = one workgroup per tile.  Same results. */
+int tg_set_gemm_resident(int enable);
 /* prefill attention: 1 (default) = bf16 matrix cores on three bf16 planes of every fp32 operand (six cross terms per
  * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), workgroups of 32 query positions
  * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;

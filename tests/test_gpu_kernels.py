@@ -155,8 +155,9 @@ def _digit_plane_closed_form(A, W, s):
     a1 = ((r1 + 128) & 255) - 128
     a2 = (r1 - a1) >> 8
     assert np.abs(a2).max() <= 127 and np.array_equal(65536 * a2 + 256 * a1 + a0, xi)
-    Wi = W.astype(np.int64)
-    s0, s1, s2 = (a @ Wi for a in (a0, a1, a2))
+    # |sum| <= 127 * 128 * K < 2^31: float64 products and sums of these integers are exact (and go through BLAS)
+    Wf = W.astype(np.float64)
+    s0, s1, s2 = ((a.astype(np.float64) @ Wf).astype(np.int64) for a in (a0, a1, a2))
     f32 = lambda z: z.astype(np.float32)
     inner = f32(f32(s1).astype(np.float64) * 256.0 + f32(s0).astype(np.float64))   # one rounding: fused multiply-add
     v = f32(f32(s2).astype(np.float64) * 65536.0 + inner.astype(np.float64))
@@ -174,6 +175,29 @@ def test_qgemm_mfma_equals_digit_plane_closed_form(tg, shape):
     Cm = np.empty((m, n), np.float32)
     tg.launch_qgemm(Cm, A, W, s, m, i, n)
     assert np.array_equal(Cm, _digit_plane_closed_form(A, W, s))
+
+
+@pytest.mark.parametrize("shape", [(2048, 1152, 6912, 21), (1920, 1152, 6912, 22), (2300, 1024, 6912, 23), (6200, 640, 2048, 24)])
+def test_qgemm_resident_workgroups_equal_one_per_tile_and_the_closed_form(tg, shape):
+    """From three output tiles per compute unit on, one resident workgroup per unit walks the tiles with the operand
+    prefetch running across tile boundaries.  Same bits as one workgroup per tile and as the closed form.  The
+    shapes cover the item walk's cases: 18 stages of K (tile boundaries alternate between the middle and the end of
+    a group of four stages) and 16; row blocks a multiple of 8 (split by XCD), 49 (XCD mapping on the flat list), and
+    tile counts that are no multiple of 8 (no XCD mapping); a last row block that is partly padding."""
+    m, i, n, seed = shape
+    A, W, s = gi.gemm_inputs(m, i, n, seed)
+    A[1] *= np.float32(1e-4)
+    out = []
+    try:
+        for resident in (1, 0):
+            tg.check(tg.lib().tg_set_gemm_resident(resident))
+            Cm = np.full((m, n), np.nan, np.float32)
+            tg.launch_qgemm(Cm, A, W, s, m, i, n)
+            out.append(Cm)
+    finally:
+        tg.check(tg.lib().tg_set_gemm_resident(1))
+    assert np.array_equal(out[0], out[1])
+    assert np.array_equal(out[0], _digit_plane_closed_form(A, W, s))
 
 
 def test_device_resident_gemv_matches_host_entry(tg, oracle):

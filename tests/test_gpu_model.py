@@ -303,6 +303,27 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
     assert e.value.code == -1
 
 
+def test_resident_gemm_workgroups_change_no_bit_of_a_long_prefill(tg, oracle):
+    """3000 tokens through two layers of the 270m shape: the up|gate product has 24 x 32 output tiles, three per
+    compute unit, and runs on resident workgroups (fused gelu(gate) * up epilogue inside the tile walk).  Same
+    arithmetic as one workgroup per tile: the logits must not differ in a single bit."""
+    cfg = tg.named_config("270m", 2)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 22))
+    sess = model.session(gsize=1024)
+    prompt = gi.prompt_ids(34, 3000)
+    out = []
+    try:
+        for resident in (1, 0):
+            tg.check(tg.lib().tg_set_gemm_resident(resident))
+            sess.reset()
+            out.append(sess.prefill(prompt))
+    finally:
+        tg.check(tg.lib().tg_set_gemm_resident(1))
+    (tok_a, lg_a), (tok_b, lg_b) = out
+    assert tok_a == tok_b and np.array_equal(lg_a, lg_b)
+
+
 def test_half_k_grid_copies_equal_the_plain_grid(tg, oracle, weight_images, tables):
     """Prefill with the output/down projections computed as two half-K copies added by the following norm
     (taken when the plain grid fills its last round badly: here 1000 rows x 5 column tiles) against the

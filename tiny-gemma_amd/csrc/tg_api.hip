@@ -330,6 +330,7 @@ int tg_init(int device) {
 	snprintf(g_devname, sizeof(g_devname), "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
 	g_n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	TG_HIP(hipStreamCreate(&g_stream));
+	if (g_gemm_resident_wgs > 0) g_gemm_resident_wgs = g_n_cu;
 	g_device = device;
 	g_inited = true;
 	return TG_OK;
@@ -1131,6 +1132,11 @@ int tg_session_release_workspace(tg_session *s) {
 	s->taps = nullptr;  // prefill taps live in the workspace
 	s->tap_rows = 0;
 	s->pf_plan.release();
+	return TG_OK;
+}
+
+int tg_set_gemm_resident(int enable) {
+	g_gemm_resident_wgs = enable ? g_n_cu : 0;
 	return TG_OK;
 }
 

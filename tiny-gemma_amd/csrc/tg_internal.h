@@ -204,6 +204,8 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
                          float *C_half2, hipStream_t s);
+// workgroups of the resident form of the MFMA GEMM (one per compute unit; set at init), 0: one workgroup per tile
+extern int g_gemm_resident_wgs;
 bool tg_gemm_mfma_wants_split(int M, int K, int ntiles, int n_cu);
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
