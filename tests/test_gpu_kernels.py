@@ -279,7 +279,20 @@ def test_attention_prefill_split_key_ranges(tg, oracle, attn_mode, S):
     assert normrel(o[:, rows, :], _dense_rows(q, k, v, rows, False, 512)) < 2e-6
     if S <= 2000:
         assert normrel(o, oracle.attention_prefill(q, k, v, False, 512)) < 2e-6
-    # the same tokens through a local layer: 513-key window, never split
+    # the same tokens through a local layer: 513-key window
     ol = tg.attention_prefill(q, k, v, True, 512)
     assert normrel(ol[:, rows, :], _dense_rows(q, k, v, rows, True, 512)) < 2e-6
     assert np.array_equal(ol[:, :513, :], o[:, :513, :]) or normrel(ol[:, :513, :], o[:, :513, :]) < 2e-6
+
+
+@pytest.mark.parametrize("S,ctx", [(33, 512), (178, 512), (300, 15), (300, 47), (513, 512), (514, 512), (1000, 100), (1000, 512)])
+def test_attention_prefill_short_prompts_cut_into_key_chunks(tg, attn_mode, S, ctx):
+    """Prompts with fewer query tiles than compute units: causal and local layers are both cut into chunks of key
+    tiles (down to one tile) and merged.  With a window of 15 or 47 keys a chunk starts before the window of the
+    tile's later queries: a chunk without a single valid key for some query must come out as weight 0."""
+    q, k, v = gi.attn_prefill_inputs(S, 900 + S + ctx)
+    rows = np.arange(S)
+    for is_sw in (False, True):
+        o = tg.attention_prefill(q, k, v, is_sw, ctx)
+        assert np.isfinite(o).all()
+        assert normrel(o, _dense_rows(q, k, v, rows, is_sw, ctx)) < 2e-6

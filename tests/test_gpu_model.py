@@ -303,6 +303,28 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
     assert e.value.code == -1
 
 
+def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
+    """A 100-token prompt: the down projection (K = 2048) runs in four parts of K over workgroups and the output
+    projection (K = 1024) in two, the following norm adds the partial results.  Against the same prefill with the
+    products unsplit: same id, logits equal to fp32 rounding of the extra additions, and really a different path."""
+    cfg = tg.named_config("270m", 2)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 23))
+    sess = model.session(gsize=1024)
+    prompt = gi.prompt_ids(35, 100)
+    out = []
+    try:
+        for split in (1, 0):
+            tg.check(tg.lib().tg_set_gemm_split(split))
+            sess.reset()
+            out.append(sess.prefill(prompt))
+    finally:
+        tg.check(tg.lib().tg_set_gemm_split(1))
+    (tok_a, lg_a), (tok_b, lg_b) = out
+    assert tok_a == tok_b and normrel(lg_a, lg_b) < 2e-5
+    assert not np.array_equal(lg_a, lg_b)
+
+
 def test_resident_gemm_workgroups_change_no_bit_of_a_long_prefill(tg, oracle):
     """3000 tokens through two layers of the 270m shape: the up|gate product has 24 x 32 output tiles, three per
     compute unit, and runs on resident workgroups (fused gelu(gate) * up epilogue inside the tile walk).  Same

@@ -35,7 +35,7 @@ int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
 int g_n_cu = 256;
-bool g_gemm_split = true;       // prefill: products with a badly filled last round of workgroups run as two half-K copies
+bool g_gemm_split = true;       // prefill: products that would leave most compute units idle run in 2 or 4 parts of K
 int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 
@@ -149,15 +149,15 @@ TgGemv gemv_base(const PackedMat &p) {
 //   prepacked : the producer of A already wrote the digit planes and row factors
 //   amax_in   : partial row maxima of A left by its producer ([amax_parts][rows]; saves the pass over A that finds them)
 //   amax_out  : GEGLU only: where this product leaves the partial row maxima of C, one part per column tile
-//   C_half2   : MFMA path, STORE only, and only where tg_gemm_mfma_wants_split says so: the product runs as two half-K
-//               copies, the second half's partial result goes here and the consumer adds the two
+//   kparts    : MFMA path, STORE only, and only what tg_gemm_mfma_k_parts says: the product runs in 2 or 4 parts of K,
+//               part p's partial result goes to C + p * part_stride and the consumer adds them
 void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
                  int lut_size, int8_t *apack, float *rowscale, bool prepacked = false, const float *amax_in = nullptr,
-                 int amax_parts = 0, float *amax_out = nullptr, float *C_half2 = nullptr) {
+                 int amax_parts = 0, float *amax_out = nullptr, int kparts = 1, size_t part_stride = 0) {
 	if (g_gemm_mfma) {
 		if (!prepacked) tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, amax_in, amax_parts, g_stream);
-		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, amax_out, C_half2,
-		                    g_stream);
+		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, amax_out, kparts,
+		                    part_stride, g_stream);
 	} else {
 		(void)lda;  // the exact kernel reads dense rows (lda == K at every call site)
 		tg_launch_gemm(C, A, p.W, p.scales, m, p.K, p.ntiles, p.C, epi, lut, gmin, geps, lut_size, g_stream);
@@ -208,26 +208,28 @@ struct tg_model {
 };
 
 namespace {
-// Device copy of the balanced work list of causal prefill layers of S tokens, with its scratch.
+// Device copy of the balanced work list of the causal (window < 0) or the local prefill layers of S tokens, with
+// its scratch.
 struct AttnPlanDev {
 	TgAttnPrefillPlan p;
 	bool use = false;
-	int S = -1, tq = 0;  // token count and query tile size the lists were built for
+	int S = -1, tq = 0, window = -1;  // what the lists were built for
 	void *bufs[4] = {nullptr, nullptr, nullptr, nullptr};
 	std::vector<int4> items, split;  // host copies stay alive until the uploads have completed
-	int build(int n_tokens) {
+	int build(int n_tokens, int win) {
 		const int tile = tg_attn_prefill_query_tile(n_tokens, g_n_cu);
-		if (n_tokens == S && tile == tq) return TG_OK;
+		if (n_tokens == S && tile == tq && win == window) return TG_OK;
 		release();
-		const int rc = build_uncached(n_tokens, tile);
+		const int rc = build_uncached(n_tokens, tile, win);
 		if (rc != TG_OK) release();  // nothing half-built stays behind as a cache hit
 		return rc;
 	}
-	int build_uncached(int n_tokens, int tile) {
+	int build_uncached(int n_tokens, int tile, int win) {
 		int nslots = 0;
-		use = tg_attn_prefill_plan(n_tokens, g_n_cu, tile, items, split, nslots);
+		use = tg_attn_prefill_plan(n_tokens, g_n_cu, tile, win, items, split, nslots);
 		S = n_tokens;
 		tq = tile;
+		window = win;
 		if (!use) return TG_OK;
 		TG_HIP(hipMalloc(&bufs[0], items.size() * sizeof(int4)));
 		TG_HIP(hipMalloc(&bufs[1], split.size() * sizeof(int4)));
@@ -252,6 +254,7 @@ struct AttnPlanDev {
 		use = false;
 		S = -1;
 		tq = 0;
+		window = -1;
 	}
 };
 }  // namespace
@@ -287,7 +290,7 @@ struct tg_session {
 	// session is destroyed, and the work lists of the causal layers for the last prompt length
 	void *pf_ws = nullptr;
 	size_t pf_ws_bytes = 0;
-	AttnPlanDev pf_plan;
+	AttnPlanDev pf_plan, pf_plan_local;
 };
 
 namespace {
@@ -759,6 +762,7 @@ void tg_session_destroy(tg_session *s) {
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
 	s->pf_plan.release();
+	s->pf_plan_local.release();
 	for (float *p : s->kc)
 		if (p) (void)hipFree(p);
 	for (float *p : s->vc)
@@ -1132,6 +1136,7 @@ int tg_session_release_workspace(tg_session *s) {
 	s->taps = nullptr;  // prefill taps live in the workspace
 	s->tap_rows = 0;
 	s->pf_plan.release();
+	s->pf_plan_local.release();
 	return TG_OK;
 }
 
@@ -1238,7 +1243,7 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	if (rc == TG_OK) rc = tg_copy_h2d(dq, qr.data(), sizeof(float) * rows * NH * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dk, k, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
-	if (rc == TG_OK && !is_sw) rc = plan.build(S);
+	if (rc == TG_OK) rc = plan.build(S, (is_sw && S > sw_context + 1) ? sw_context : -1);
 	if (rc != TG_OK) return done(rc);
 	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), nullptr, g_n_cu, g_stream);
 	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
@@ -1269,8 +1274,8 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		return off;
 	};
 	const size_t o_ids = carve(sizeof(int) * S), o_x = carve(sizeof(float) * S * h), o_xn = carve(sizeof(float) * S * h),
-	             o_qkv = carve(sizeof(float) * S * nq), o_ao = carve(sizeof(float) * S * qo), o_t = carve(sizeof(float) * S * h),
-	             o_t2 = carve(sizeof(float) * S * h), o_hb = carve(sizeof(float) * S * f),
+	             o_qkv = carve(sizeof(float) * S * nq), o_ao = carve(sizeof(float) * S * qo), o_t = carve(sizeof(float) * 4 * S * h),  // up to 4 partial results
+	             o_hb = carve(sizeof(float) * S * f),
 	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
 	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
 	             o_amax = carve(g_gemm_mfma ? sizeof(float) * (size_t)std::max(2 * f / TG_CT, c.n_head) * tg_gemm_mfma_rows(n) : 0),
@@ -1285,13 +1290,19 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	uint8_t *ws = (uint8_t *)s->pf_ws;
 	int *d_ids = (int *)(ws + o_ids);
 	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
-	      *t = (float *)(ws + o_t), *t2 = (float *)(ws + o_t2), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
+	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
 	int8_t *apack = (int8_t *)(ws + o_apack);
 	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // partial row maxima: max|ao| per (head, row), then max|hb| per (up|gate tile, row)
 	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
 	s->tap_rows = keep_taps ? n : 0;
-	AttnPlanDev &plan = s->pf_plan;
-	if (int rc = plan.build(n)) return rc;
+	// Work lists of the attention launches.  A local layer whose window covers the whole prompt is a causal layer.
+	const bool local_is_causal = n <= c.n_pos_local + 1;
+	if (int rc = s->pf_plan.build(n, -1)) return rc;
+	if (!local_is_causal) {
+		if (int rc = s->pf_plan_local.build(n, c.n_pos_local)) return rc;
+	}
+	const TgAttnPrefillPlan *plan_global = s->pf_plan.get();
+	const TgAttnPrefillPlan *plan_local = local_is_causal ? plan_global : s->pf_plan_local.get();
 	auto tap = [&](int b) -> hipError_t {
 		if (!keep_taps) return hipSuccess;
 		return hipMemcpyAsync(s->taps + (size_t)b * S * h, x, sizeof(float) * S * h, hipMemcpyDeviceToDevice, g_stream);
@@ -1302,12 +1313,14 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	// xn = rmsnorm(x, attn_pre of layer 0)
 	// With the int8 MFMA GEMM the norm writes the GEMM's digit planes itself and the fp32 row is not stored.
 	const bool pk = g_gemm_mfma;
-	tg_launch_norm_rows(pk ? nullptr : xn, x, nullptr, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale,
+	tg_launch_norm_rows(pk ? nullptr : xn, x, 1, 0, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale,
 	                    g_stream);
-	// products whose plain grid would leave most compute units idle in its last round run as two half-K copies; the
-	// norm that consumes them adds the halves
-	float *o_h2 = (pk && g_gemm_split && tg_gemm_mfma_wants_split(n, qo, m->L[0].o.ntiles_g, g_n_cu)) ? t2 : nullptr;
-	float *d_h2 = (pk && g_gemm_split && tg_gemm_mfma_wants_split(n, f, m->L[0].d.ntiles_g, g_n_cu)) ? t2 : nullptr;
+	// products that would otherwise leave most compute units idle (a badly filled last round of workgroups; a short
+	// prompt's long-K products) run in 2 or 4 parts of K with separate partial results; the norm that consumes them adds
+	// the parts
+	const size_t tpart = S * h;
+	const int o_parts = (pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, qo, m->L[0].o.ntiles_g, g_n_cu) : 1;
+	const int d_parts = (pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, f, m->L[0].d.ntiles_g, g_n_cu) : 1;
 	for (int l = 0; l < L; l++) {
 		const LayerDev &Ld = m->L[(size_t)l];
 		const int mp = s->max_pos[(size_t)l];
@@ -1318,20 +1331,21 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
 		                            g_stream);
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, plan.get(), amax, g_n_cu, g_stream);
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp,
+		                       Ld.is_sw ? plan_local : plan_global, amax, g_n_cu, g_stream);
 		// O (modules.hpp:127-128)
-		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0, nullptr, o_h2);
+		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0, nullptr, o_parts, tpart);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
-		tg_launch_norm_rows(pk ? nullptr : xn, t, o_h2, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
+		tg_launch_norm_rows(pk ? nullptr : xn, t, o_parts, tpart, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
 		TG_HIP(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
 		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, 0, amax);
-		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g, nullptr, d_h2);
+		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g, nullptr, d_parts, tpart);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
 		// the last layer's final norm feeds the LM head GEMV, which reads the fp32 row
 		const bool last = l + 1 == L;
-		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, d_h2, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
+		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, d_parts, tpart, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
 		                    g_stream);
 		TG_HIP(tap(2 * l + 2));
 	}

@@ -135,13 +135,16 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 		}
 		tmax = fmaxf(tmax, tg_red_partner<16>(tmax));
 		tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
-		const float m_new = fmaxf(m_run, tmax);  // finite from the first tile on: it holds a valid key of every query
-		const float alpha = expf(m_run - m_new);
+		const float m_new = fmaxf(m_run, tmax);
+		// A chunk of a local layer's work list may start a few keys before a query's window: nothing valid yet, the
+		// running maximum stays -inf and every weight of the tile must come out as 0, not as exp(-inf + inf).
+		const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;
+		const float alpha = expf(m_run - m_ref);
 		float psum = 0.0f;
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
-			s0[i] = expf(s0[i] - m_new);
-			s1[i] = expf(s1[i] - m_new);
+			s0[i] = expf(s0[i] - m_ref);
+			s1[i] = expf(s1[i] - m_ref);
 			psum += s0[i] + s1[i];
 		}
 		psum += tg_red_partner<16>(psum);
@@ -407,13 +410,14 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 		tmax = fmaxf(tmax, tg_red_partner<16>(tmax));
 		tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
 		const float m_new = fmaxf(m_run, tmax);
-		const float alpha = expf(m_run - m_new);
+		const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // no valid key yet (see the fp32 kernel)
+		const float alpha = expf(m_run - m_ref);
 		float psum = 0.0f;
 		float pv[8];  // the lane's 8 key slots: keys 4g + i, then 16 + 4g + i
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
-			pv[i] = expf(s0[i] - m_new);
-			pv[4 + i] = expf(s1[i] - m_new);
+			pv[i] = expf(s0[i] - m_ref);
+			pv[4 + i] = expf(s1[i] - m_ref);
 			psum += pv[i] + pv[4 + i];
 		}
 		psum += tg_red_partner<16>(psum);
@@ -510,34 +514,51 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 
 int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
 
-// Work list of a causal layer of S tokens, for tg_launch_attn_prefill.  Returns false when no query tile needs
-// splitting (then the plain launch is already balanced).  items: one int4 per workgroup, heaviest first;
-// split: one int4 per split query tile; nslots: chunks that go through scratch.
+// Work list of a layer of S tokens, for tg_launch_attn_prefill: causal (window < 0) or local (a query sees the
+// `window` keys before it and itself).  Returns false when no query tile needs splitting (then the plain launch is
+// already balanced).  items: one int4 per workgroup {query tile, first key tile, end key tile, slot or -1},
+// heaviest first; split: one int4 per split query tile; nslots: chunks that go through scratch.
 // 32 query positions per workgroup once that leaves a workgroup for every other compute unit (measured crossover:
 // between 2048 and 4096 tokens on 256 compute units)
 int tg_attn_prefill_query_tile(int S, int n_cu) {
 	return (g_attn_prefill_bf16x3 == 2 || (g_attn_prefill_bf16x3 == 1 && (S + 31) / 32 >= n_cu / 2)) ? 32 : TQ;
 }
 
-bool tg_attn_prefill_plan(int S, int n_cu, int tq, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
+bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
 	const int nq = (S + tq - 1) / tq;
-	auto ntiles_of = [&](int qt) { return (std::min(qt * tq + tq, S) + TK - 1) / TK; };
+	auto first_tile = [&](int qt) { return (window >= 0 && qt * tq > window) ? (qt * tq - window) / TK : 0; };
+	auto end_tile = [&](int qt) { return (std::min(qt * tq + tq, S) + TK - 1) / TK; };
 	long total = 0;
-	for (int qt = 0; qt < nq; qt++) total += ntiles_of(qt);
-	// about 8 items per compute unit, and never chunks below 16 key tiles (512 keys)
-	const int chunk = (int)std::max<long>(16, total / ((long)n_cu * 8));
+	int longest = 1;
+	for (int qt = 0; qt < nq; qt++) {
+		total += end_tile(qt) - first_tile(qt);
+		longest = std::max(longest, end_tile(qt) - first_tile(qt));
+	}
+	// Long prompts (causal): about 8 items per compute unit, and never chunks below 16 key tiles (512 keys).
+	// Prompts with fewer query tiles than compute units: a workgroup's time is its chain of key tiles (one wave per
+	// SIMD, nothing overlaps), so the chains are cut as short as the number of compute units allows: the smallest
+	// chunk that still gives at most one item per unit.  Local layers of long prompts are balanced as they are.
+	int chunk = window < 0 ? (int)std::max<long>(16, total / ((long)n_cu * 8)) : longest;
+	for (int c = 1; c < chunk; c++) {
+		long n = 0;
+		for (int qt = 0; qt < nq; qt++) n += (end_tile(qt) - first_tile(qt) + c - 1) / c;
+		if (n <= n_cu) {
+			chunk = c;
+			break;
+		}
+	}
 	items.clear();
 	split.clear();
 	nslots = 0;
 	for (int qt = 0; qt < nq; qt++) {
-		const int nt = ntiles_of(qt), nc = (nt + chunk - 1) / chunk;
+		const int t0 = first_tile(qt), nt = end_tile(qt) - t0, nc = (nt + chunk - 1) / chunk;
 		if (nc == 1) {
-			items.push_back(int4{qt, 0, nt, -1});
+			items.push_back(int4{qt, t0, t0 + nt, -1});
 			continue;
 		}
 		split.push_back(int4{qt, nslots, nc, 0});
 		for (int ch = 0; ch < nc; ch++) {  // equal chunks
-			const int tb = (int)((long)nt * ch / nc), te = (int)((long)nt * (ch + 1) / nc);
+			const int tb = t0 + (int)((long)nt * ch / nc), te = t0 + (int)((long)nt * (ch + 1) / nc);
 			items.push_back(int4{qt, tb, te, nslots++});
 		}
 	}
@@ -562,19 +583,19 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 		                          (int)BF_LDS_BYTES);
 		lds_set = true;
 	}
-	const bool whole = plan == nullptr || is_sw;
+	const bool whole = plan == nullptr;  // the caller passes the work list that fits the layer kind, or none
 	const int tq = tg_attn_prefill_query_tile(S, n_cu);  // a plan must have been built for this tile size
 	const dim3 grid(whole ? (unsigned)((S + tq - 1) / tq) : (unsigned)plan->nitems);
 	const int4 *items = whole ? nullptr : plan->items;
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
 	if (g_attn_prefill_bf16x3 && tq == 32)
-		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
+		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
 		                   window, items, po, pml, rowmax_part, Mpad);
 	else if (g_attn_prefill_bf16x3)
-		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<1>, grid, dim3(256), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0,
+		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<1>, grid, dim3(256), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
 		                   window, items, po, pml, rowmax_part, Mpad);
 	else
-		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, whole ? is_sw : 0, window, items,
+		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items,
 		                   po, pml, rowmax_part, Mpad);
 	if (whole) return;
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * tq)), dim3(PNT), 0, s, o, S, ldo, plan->split,

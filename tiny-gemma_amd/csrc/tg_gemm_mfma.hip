@@ -45,7 +45,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GNT = 256;     // threads per workgroup: 4 waves, each owns 32 rows x 128 columns
 constexpr int KSTAGE = 64;   // rows of K per LDS stage
-constexpr int TG_GEMM_SKINNY_ROWS = 256;    // at most this many rows and
+constexpr int TG_GEMM_SKINNY_ROWS = 448;    // at most this many rows and
 constexpr int TG_GEMM_SKINNY_BLOCKS = 128;  // fewer workgroups than this in the plain tiling: split K over the waves
 constexpr int LUT_LDS_MAX = 4096;  // GeLU tables up to this many entries are staged in LDS (Bs holds 16 KB)
 
@@ -561,27 +561,35 @@ __global__ __launch_bounds__(GNT) void gemm_i8_resident_kernel(float *C, const i
 }
 
 // ---- few rows (a short prompt): the same product with the reduction split over the four waves ----------------
-// With M <= 256 the kernel above has only a handful of workgroups (two row blocks x 9 column tiles for the down
+// With a few hundred rows (up to 448: measured crossover between 400 and 512) the kernel above has only a handful of
+// workgroups (two row blocks x 9 column tiles for the down
 // projection of the 1B shape) and each walks all of K alone.  Here a workgroup owns 32 rows x 128 columns and its
 // four waves take the K stages round-robin (stage w, w + 4, ...), each with a private register pipeline: no LDS and
 // no barrier in the main loop, weights fetched straight from global memory in operand order (32 lanes x 16 bytes =
 // 512 contiguous bytes per fragment).  The integer partial sums are added through LDS at the end (exact, so the
 // result equals the unsplit one bit for bit) and wave j finishes column block j.
+// gridDim.z > 1 (plain epilogue only): K is also cut into gridDim.z equal parts over workgroups; part z writes its own
+// partial result C + z * part_stride and the consumer adds them (a long K with few rows and few column tiles would
+// otherwise run on a few dozen compute units, each pulling megabytes of weights through its own L1).
 template <bool GEGLU, bool LUTLDS>
 __global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
                                                              const float *scales, int M, int K, int ldc, const float *lut, float gmin,
-                                                             float geps, float ginv, int lut_size, float *rowmax_part, int Mpad) {
+                                                             float geps, float ginv, int lut_size, float *rowmax_part, int Mpad,
+                                                             size_t part_stride) {
 	__shared__ __attribute__((aligned(16))) i32x4 red[4][3][4][64];  // [wave][plane][quarter of the 16 registers][lane]
 	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
 	__shared__ float pmax[2][32];
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hb = lane >> 5;
-	const int tile = blockIdx.x, mtile = blockIdx.y;
-	const int nstage = K / KSTAGE, last = nstage - 1;
+	const int tile = blockIdx.x, mtile = blockIdx.y, z = blockIdx.z;
+	const int nstage = K / KSTAGE / (int)gridDim.z, last = nstage - 1;  // stages of this workgroup's part of K
 	if (GEGLU && LUTLDS) {  // visible after the barriers of the reduction
 		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
 	}
-	const i32x4 *bsrc = reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + hb * TG_CT + c;
-	const i32x4 *asrc = reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane;
+	C += (size_t)z * part_stride;
+	const i32x4 *bsrc =
+	    reinterpret_cast<const i32x4 *>(Wg + (size_t)tile * (size_t)K * TG_CT) + hb * TG_CT + c + (size_t)z * nstage * 4 * TG_CT;
+	const i32x4 *asrc =
+	    reinterpret_cast<const i32x4 *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 64 + lane + (size_t)z * nstage * 6 * 64;
 
 	// ring of three stages: loads go to ordinary vector registers only, and 3 x 56 of them is what fits beside the
 	// addresses (the 192 accumulators live in the accumulation registers)
@@ -724,7 +732,7 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 // rowmax_part (GEGLU only, may be null): [ntiles][tg_gemm_mfma_rows(M)] floats, max|C[m][tile's columns]|
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
-                         float *C_half2, hipStream_t s) {
+                         int kparts, size_t part_stride, hipStream_t s) {
 	const unsigned mblocks = (unsigned)((M + 127) / 128);
 	const int Mpad = (int)tg_gemm_mfma_rows(M);
 	const float *rowinv = rowfac + Mpad;
@@ -735,21 +743,21 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	float *rmp = geglu ? rowmax_part : nullptr;
 	// few rows and few column tiles: split K over the waves instead of leaving most compute units idle
 	if (M <= TG_GEMM_SKINNY_ROWS && (int)mblocks * ntiles < TG_GEMM_SKINNY_BLOCKS) {
-		const dim3 grid((unsigned)ntiles, (unsigned)((M + 31) / 32)), block(GNT);
+		const dim3 grid((unsigned)ntiles, (unsigned)((M + 31) / 32), (unsigned)(geglu ? 1 : kparts)), block(GNT);
 		if (geglu && lutlds)
 			hipLaunchKernelGGL((gemm_i8_skinny_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, Mpad);
+			                   ginv, lut_size, rmp, Mpad, (size_t)0);
 		else if (geglu)
 			hipLaunchKernelGGL((gemm_i8_skinny_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, Mpad);
+			                   ginv, lut_size, rmp, Mpad, (size_t)0);
 		else
 			hipLaunchKernelGGL((gemm_i8_skinny_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
-			                   geps, ginv, lut_size, rmp, Mpad);
+			                   geps, ginv, lut_size, rmp, Mpad, part_stride);
 		return;
 	}
-	// C_half2 != nullptr (STORE only; see tg_gemm_mfma_wants_split): two half-K copies of the grid, the second writes C_half2
-	const int ksplit = (C_half2 != nullptr && !geglu) ? 2 : 1;
-	const size_t csplit = ksplit == 2 ? (size_t)(C_half2 - C) : 0;
+	// kparts == 2 (STORE only; see tg_gemm_mfma_k_parts): two half-K copies of the grid, the second writes C + part_stride
+	const int ksplit = (kparts == 2 && !geglu) ? 2 : 1;
+	const size_t csplit = ksplit == 2 ? part_stride : 0;
 	// Resident workgroups pay off from three tiles per compute unit on (measured per product inside a 4096-token and a
 	// 1000-token prefill: up|gate with 13.5 and 3.4 tiles per unit -5 % and -3 %; Q|K|V, output and down projections
 	// with 1.1 to 2.3 tiles per unit +1 to +3 us each: the start-up of the item walk is not recovered).
@@ -780,14 +788,23 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 		                   lut_size, rmp, Mpad, ksplit, csplit);
 }
 
-// Whether a STORE product of M rows, K deep, ntiles column tiles should run as two half-K copies whose results the
-// consumer adds: when that fills the last round of workgroups noticeably better.  Needs whole pairs of stages per half.
-bool tg_gemm_mfma_wants_split(int M, int K, int ntiles, int n_cu) {
-	if (M <= TG_GEMM_SKINNY_ROWS || (K / KSTAGE) % 4 != 0) return false;
+// In how many parts of K (1, 2 or 4) a STORE product of M rows, K deep, ntiles column tiles should run; the parts
+// write separate partial results which the consumer adds.
+//   * the few-row kernel: as many parts as leave each at least 8 stages (the down projection of a 178-token prompt:
+//     54 workgroups walking 6912 rows of K become 216 walking 1728);
+//   * the tiled kernel: 2 when that fills the last round of workgroups noticeably better (whole pairs of stages per half).
+int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu) {
+	const int nstage = K / KSTAGE;
+	if (M <= TG_GEMM_SKINNY_ROWS && ((M + 127) / 128) * ntiles < TG_GEMM_SKINNY_BLOCKS) {
+		if (nstage % 4 == 0 && nstage / 4 >= 8) return 4;
+		if (nstage % 2 == 0 && nstage / 2 >= 8) return 2;
+		return 1;
+	}
+	if (M <= TG_GEMM_SKINNY_ROWS || nstage % 4 != 0) return 1;
 	const long wgs = (long)((M + 127) / 128) * ntiles;
 	auto eff = [&](long n) { return (double)n / (double)(((n + n_cu - 1) / n_cu) * n_cu); };
 	// measured: worth it only when the last round is nearly empty (288 workgroups on 256 compute units: -2 % prefill time);
 	// at 0.75 or better the second prologue/epilogue and the extra partial result cost more than the idle units
-	return eff(wgs) < 0.6 && eff(2 * wgs) > eff(wgs) + 0.1;
+	return (eff(wgs) < 0.6 && eff(2 * wgs) > eff(wgs) + 0.1) ? 2 : 1;
 }
 

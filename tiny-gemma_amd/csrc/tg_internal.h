@@ -157,12 +157,12 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 // out = rmsnorm(in, w); if resid != null first in = rmsnorm(in, w_post) + resid is formed and stored to resid_out
 // apack/rowfac non-null: the normalised rows are also (out == nullptr: only) written as digit planes + row factors for
 // tg_launch_gemm_mfma (rowfac as tg_launch_quant_pack lays it out for S rows)
-void tg_launch_norm_rows(float *out, const float *in, const float *in2, const float *w_pre, const float *w_post, const float *resid,
+void tg_launch_norm_rows(float *out, const float *in, int nparts, size_t part_stride, const float *w_pre, const float *w_post, const float *resid,
                          float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s);
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
                                  const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
                                  hipStream_t s);
-// Balanced work list of a causal prefill layer (device copies of what tg_attn_prefill_plan returns) + scratch.
+// Balanced work list of a prefill layer (device copies of what tg_attn_prefill_plan returns) + scratch.
 struct TgAttnPrefillPlan {
 	const int4 *items;  // [nitems] {query tile, first key tile, end key tile, slot or -1}
 	const int4 *split;  // [nsplit] {query tile, first slot, chunks}
@@ -171,7 +171,8 @@ struct TgAttnPrefillPlan {
 };
 extern int g_attn_prefill_bf16x3;  // prefill attention: 0 = fp32 matrix path, 1 = split-bf16 matrix path, 2 = the same with 32-query workgroups at any length
 int tg_attn_prefill_query_tile(int S, int n_cu);  // query positions per workgroup of the kernel a launch will take
-bool tg_attn_prefill_plan(int S, int n_cu, int tq, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
+// window < 0: causal layer; else a local layer whose queries see `window` keys before them and themselves
+bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
 size_t tg_attn_prefill_part_floats(int nslots, int tq);
 size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
@@ -203,10 +204,11 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
                           hipStream_t s);
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
-                         float *C_half2, hipStream_t s);
+                         int kparts, size_t part_stride, hipStream_t s);
 // workgroups of the resident form of the MFMA GEMM (one per compute unit; set at init), 0: one workgroup per tile
 extern int g_gemm_resident_wgs;
-bool tg_gemm_mfma_wants_split(int M, int K, int ntiles, int n_cu);
+// parts of K (1, 2, 4) a plain-epilogue product should run in; part p writes C + p * part_stride, the consumer adds them
+int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu);
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global load of the wave (its fence covers all address spaces), which would drain a software pipeline

@@ -47,8 +47,8 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 // [post-norm + residual (+ residual out)] + pre-norm.  The normalised row goes out as fp32 (out != nullptr) and/or
 // straight as the int8 digit planes + row factors of the MFMA GEMM that consumes it (apack != nullptr): the same bits
 // the stand-alone quantising pre-pass would produce from the fp32 row.
-template <int ROUNDS>
-__global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, const float *in2, const float *w_pre,
+template <int ROUNDS, int NPARTS>
+__global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, size_t part_stride, const float *w_pre,
                                                         const float *w_post, const float *resid, float *resid_out, int S, int dim,
                                                         int8_t *apack, float *rowfac, int Mpad) {
 	typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -68,11 +68,21 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 #pragma unroll
 		for (int q = 0; q < 2; q++) v[r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)s * dim + off[r] + 4 * q);
 	}
-	if (in2 != nullptr) {  // the row arrives as two addends (a product computed in two halves of K)
+	if (NPARTS > 1) {  // the row arrives as NPARTS addends (a product computed in parts of K): all fetched, then added in order
+		f32x4 more[NPARTS > 1 ? NPARTS - 1 : 1][ROUNDS][2];
 #pragma unroll
-		for (int r = 0; r < ROUNDS; r++)
+		for (int p = 1; p < NPARTS; p++)
 #pragma unroll
-			for (int q = 0; q < 2; q++) v[r][q] += *reinterpret_cast<const f32x4 *>(in2 + (size_t)s * dim + off[r] + 4 * q);
+			for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+				for (int q = 0; q < 2; q++)
+					more[p - 1][r][q] = *reinterpret_cast<const f32x4 *>(in + (size_t)p * part_stride + (size_t)s * dim + off[r] + 4 * q);
+#pragma unroll
+		for (int p = 1; p < NPARTS; p++)
+#pragma unroll
+			for (int r = 0; r < ROUNDS; r++)
+#pragma unroll
+				for (int q = 0; q < 2; q++) v[r][q] += more[p - 1][r][q];
 	}
 	if (resid != nullptr) {
 #pragma unroll
@@ -255,17 +265,25 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 	hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)S), dim3(RNT), 0, s, x, ids, wte, scales, hidden, vocab, emb_scale);
 }
 
-void tg_launch_norm_rows(float *out, const float *in, const float *in2, const float *w_pre, const float *w_post, const float *resid,
-                         float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
+// in: nparts (1, 2 or 4) addends of every row, part_stride floats apart
+void tg_launch_norm_rows(float *out, const float *in, int nparts, size_t part_stride, const float *w_pre, const float *w_post,
+                         const float *resid, float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(S);
 	const dim3 grid((unsigned)((S + RNT / 64 - 1) / (RNT / 64))), block(RNT);
 	// dim is a legal row dimension: a multiple of 16, at most 1536 where a norm is applied (hidden sizes 640 and 1152)
-	if (dim <= 1024)
-		hipLaunchKernelGGL(norm_rows_kernel<2>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
-		                   Mpad);
-	else
-		hipLaunchKernelGGL(norm_rows_kernel<3>, grid, block, 0, s, out, in, in2, w_pre, w_post, resid, resid_out, S, dim, apack, rowfac,
-		                   Mpad);
+#define TG_NORM_ROWS(R, P)                                                                                                        \
+	hipLaunchKernelGGL((norm_rows_kernel<R, P>), grid, block, 0, s, out, in, part_stride, w_pre, w_post, resid, resid_out, S, dim, apack, \
+	                   rowfac, Mpad)
+	if (dim <= 1024) {
+		if (nparts == 4) TG_NORM_ROWS(2, 4);
+		else if (nparts == 2) TG_NORM_ROWS(2, 2);
+		else TG_NORM_ROWS(2, 1);
+	} else {
+		if (nparts == 4) TG_NORM_ROWS(3, 4);
+		else if (nparts == 2) TG_NORM_ROWS(3, 2);
+		else TG_NORM_ROWS(3, 1);
+	}
+#undef TG_NORM_ROWS
 }
 
 // Wp/scales: GEMV tiling of the matrix (ntiles tiles of Ct columns); C gets ntiles * Ct columns, or half of that for GEGLU
