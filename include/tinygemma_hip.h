@@ -188,6 +188,18 @@ int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches)
  * times on the session's current buffers, back to back, without advancing the session: for timing one
  * kernel in isolation with events on tg_stream().  The kernels are idempotent on their inputs. */
 int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repeat);
+/* Host-side planning of a prefill, for inspection and tests; no counterpart in the reference, no GPU call.
+ * tg_plan_attention_prefill: the work list of one attention layer of n_tokens on n_cu compute units, causal (window < 0)
+ * or local (a query sees `window` keys before it and itself): *query_tile = query positions per workgroup; items =
+ * 4 ints per workgroup {query tile, first key tile, end key tile, scratch slot or -1} (key tiles of 32 keys), heaviest
+ * first, at most max_items of them written; *n_items = their number (0: the layer runs one workgroup per query tile over
+ * its whole key range); *n_split = query tiles whose key range is cut and merged afterwards.
+ * tg_plan_gemm_k_parts: in how many parts of K (1, 2, 4) a projection of m rows, in_dim -> out_dim, runs when the
+ * consumer can add partial results (output and down projection). */
+int tg_plan_attention_prefill(int n_tokens, int n_cu, int window, int *query_tile, int32_t *items, int max_items, int *n_items,
+                              int *n_split);
+int tg_plan_gemm_k_parts(int m, int in_dim, int out_dim, int n_cu);
+
 
 /* Debug taps: the residual stream of the most recent forward after block b
  * (b = 0: embedding; 2l+1: after attention of layer l; 2l+2: after the MLP of layer l).

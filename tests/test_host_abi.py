@@ -76,3 +76,68 @@ def test_missing_library_is_reported(pkg, tmp_path, monkeypatch):
     monkeypatch.setattr(pkg, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(FileNotFoundError):
         pkg.lib()
+
+
+# ---- host-side planning of a prefill (no GPU) ---------------------------------------------------------------------
+
+def attention_plan(lib, S, n_cu, window):
+    cap = 1 << 16
+    items = np.zeros((cap, 4), np.int32)
+    tq, n, nsplit = C.c_int(), C.c_int(), C.c_int()
+    lib.tg_plan_attention_prefill.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int32), C.c_int,
+                                              C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    rc = lib.tg_plan_attention_prefill(S, n_cu, window, C.byref(tq), items.ctypes.data_as(C.POINTER(C.c_int32)), cap, C.byref(n),
+                                       C.byref(nsplit))
+    assert rc == 0 and n.value <= cap
+    return tq.value, items[:n.value].copy(), nsplit.value
+
+
+@pytest.mark.parametrize("S,window", [(1, -1), (33, -1), (178, -1), (178, 512), (300, 15), (300, 47), (513, 512), (514, 512),
+                                      (1000, -1), (1000, 512), (1000, 100), (4096, -1), (4096, 512), (4099, -1), (16384, -1),
+                                      (16384, 512)])
+def test_attention_work_list_covers_every_visible_key_exactly_once(pkg, S, window):
+    """What the list must guarantee whatever its balance: for every query, every key it may see (causal; local: the
+    `window` keys before it and itself) lies in exactly one work item of the query's tile; slots are numbered 0..n-1;
+    items come heaviest first."""
+    n_cu = 256
+    tq, items, nsplit = attention_plan(pkg.lib(), S, n_cu, window)
+    assert tq in (16, 32)
+    nq = (S + tq - 1) // tq
+    if len(items) == 0:
+        # one workgroup per query tile over its whole range: only where that is balanced or cannot be improved
+        assert nq >= n_cu or nq == 1 or (window >= 0 and S > 2048)
+        return
+    per_tile = {}
+    for qt, tb, te, slot in items:
+        assert 0 <= qt < nq and 0 <= tb < te
+        per_tile.setdefault(int(qt), []).append((int(tb), int(te), int(slot)))
+    assert sorted(per_tile) == list(range(nq))
+    slots = sorted(slot for chunks in per_tile.values() for _, _, slot in chunks if slot >= 0)
+    assert slots == list(range(len(slots)))
+    assert sum(1 for chunks in per_tile.values() if len(chunks) > 1) == nsplit
+    lengths = [int(te - tb) for _, tb, te, _ in items]
+    assert lengths == sorted(lengths, reverse=True)
+    for qt, chunks in per_tile.items():
+        chunks.sort()
+        assert all(a[1] == b[0] for a, b in zip(chunks, chunks[1:]))        # contiguous, disjoint
+        assert (len(chunks) == 1) == (chunks[0][2] == -1)                     # whole tiles write the output themselves
+        q_first, q_last = qt * tq, min(qt * tq + tq, S) - 1
+        lo = max(0, q_first - window) if window >= 0 else 0                   # first key any query of the tile sees
+        assert chunks[0][0] * 32 <= lo and chunks[0][0] * 32 + 32 > lo        # starts at the key tile that holds it
+        assert (chunks[-1][1] - 1) * 32 <= q_last < chunks[-1][1] * 32        # ends at the key tile of the last query
+    if nq < n_cu:
+        # fewer query tiles than compute units: chains as short as the number of units allows (one item per unit);
+        # causal layers of long prompts keep their rule instead (about 8 items per unit, chunks of 16 key tiles or more)
+        assert len(items) <= n_cu or max(lengths) == 1 or (window < 0 and max(lengths) <= 16)
+
+
+def test_gemm_k_parts_rule(pkg):
+    f = pkg.lib().tg_plan_gemm_k_parts
+    f.argtypes = [C.c_int] * 4
+    assert f(178, 6912, 1152, 256) == 4      # few rows, 108 stages of K: 4 x 27
+    assert f(178, 1024, 1152, 256) == 2      # 16 stages: 2 x 8
+    assert f(100, 2048, 640, 256) == 4 and f(100, 1024, 640, 256) == 2
+    assert f(4096, 6912, 1152, 256) == 2     # 288 workgroups on 256 units: two half-K copies
+    assert f(4096, 1152, 6912, 256) == 1     # 18 stages do not split into whole pairs per half
+    assert f(8192, 6912, 1152, 256) == 1     # last round filled to 0.75
+    assert f(1000, 6912, 1152, 256) == 2

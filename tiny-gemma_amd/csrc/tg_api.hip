@@ -1110,6 +1110,31 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
 	return enqueue_decode_step(s, nullptr, false, &only);
 }
 
+int tg_plan_attention_prefill(int n_tokens, int n_cu, int window, int *query_tile, int32_t *items, int max_items, int *n_items,
+                              int *n_split) {
+	if (n_tokens < 1 || n_cu < 1 || !query_tile || !n_items || !n_split || (max_items > 0 && !items))
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	const int tq = tg_attn_prefill_query_tile(n_tokens, n_cu);
+	std::vector<int4> it, sp;
+	int nslots = 0;
+	const bool use = tg_attn_prefill_plan(n_tokens, n_cu, tq, window, it, sp, nslots);
+	*query_tile = tq;
+	*n_items = use ? (int)it.size() : 0;
+	*n_split = use ? (int)sp.size() : 0;
+	for (int i = 0; use && i < (int)it.size() && i < max_items; i++) {
+		items[4 * i + 0] = it[(size_t)i].x;
+		items[4 * i + 1] = it[(size_t)i].y;
+		items[4 * i + 2] = it[(size_t)i].z;
+		items[4 * i + 3] = it[(size_t)i].w;
+	}
+	return TG_OK;
+}
+
+int tg_plan_gemm_k_parts(int m, int in_dim, int out_dim, int n_cu) {
+	if (m < 1 || n_cu < 1 || !legal_in(in_dim) || !legal_out(out_dim) || out_dim % TG_CT) return 1;
+	return tg_gemm_mfma_k_parts(m, in_dim, out_dim / TG_CT, n_cu);
+}
+
 int tg_set_attn_merge_chunk(int keys) {
 	if (keys < 32 || keys > 256 || keys % 16) return tg_fail(TG_ERR_BAD_ARG, "keys per workgroup: a multiple of 16 in 32..256");
 	g_attn_merge_chunk = keys;
