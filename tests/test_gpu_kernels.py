@@ -177,13 +177,15 @@ def test_qgemm_mfma_equals_digit_plane_closed_form(tg, shape):
     assert np.array_equal(Cm, _digit_plane_closed_form(A, W, s))
 
 
-@pytest.mark.parametrize("shape", [(2048, 1152, 6912, 21), (1920, 1152, 6912, 22), (2300, 1024, 6912, 23), (6200, 640, 2048, 24)])
+@pytest.mark.parametrize("shape", [(2048, 1152, 6912, 21), (1920, 1152, 6912, 22), (2300, 1024, 6912, 23), (6200, 640, 2048, 24),
+                                   (2048, 256, 6912, 25)])
 def test_qgemm_resident_workgroups_equal_one_per_tile_and_the_closed_form(tg, shape):
     """From three output tiles per compute unit on, one resident workgroup per unit walks the tiles with the operand
     prefetch running across tile boundaries.  Same bits as one workgroup per tile and as the closed form.  The
     shapes cover the item walk's cases: 18 stages of K (tile boundaries alternate between the middle and the end of
     a group of four stages) and 16; row blocks a multiple of 8 (split by XCD), 49 (XCD mapping on the flat list), and
-    tile counts that are no multiple of 8 (no XCD mapping); a last row block that is partly padding."""
+    tile counts that are no multiple of 8 (no XCD mapping); a last row block that is partly padding.  K = 256 has too
+    few stages for the tile walk and must stay on one workgroup per tile whatever the switch says."""
     m, i, n, seed = shape
     A, W, s = gi.gemm_inputs(m, i, n, seed)
     A[1] *= np.float32(1e-4)

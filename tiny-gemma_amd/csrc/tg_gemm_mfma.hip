@@ -761,7 +761,8 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	// Resident workgroups pay off from three tiles per compute unit on (measured per product inside a 4096-token and a
 	// 1000-token prefill: up|gate with 13.5 and 3.4 tiles per unit -5 % and -3 %; Q|K|V, output and down projections
 	// with 1.1 to 2.3 tiles per unit +1 to +3 us each: the start-up of the item walk is not recovered).
-	if (g_gemm_resident_wgs > 0 && ntiles * (int)mblocks * ksplit >= 3 * g_gemm_resident_wgs) {
+	// (The load cursors of the item walk need at least 8 stages of K per item: K = 256 stays on one workgroup per tile.)
+	if (g_gemm_resident_wgs > 0 && ntiles * (int)mblocks * ksplit >= 3 * g_gemm_resident_wgs && K / KSTAGE / ksplit >= 8) {
 		const int mb = (int)mblocks * ksplit, total = ntiles * mb, G = g_gemm_resident_wgs;
 		const int perm = (total % 8 == 0 && G % 8 == 0) ? 1 : 0;  // workgroups go to the 8 XCDs round-robin
 		const dim3 grid((unsigned)G), block(GNT);
