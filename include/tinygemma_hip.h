@@ -154,8 +154,9 @@ int tg_set_taps(int enable);
  * (exact integer accumulation, fp32-rounding-level accuracy),
  * 0 = the reference's exact per-element order on the vector ALUs (bit-exact with gemm::launch_qgemm, slower) */
 int tg_set_gemm_mode(int mfma);
-/* prefill, int8 matrix path: 1 (default) = the output and down projections run as two half-K copies of their grid
- * when that fills the last round of workgroups better (the following norm adds the halves); 0 = never */
+/* prefill, int8 matrix path: 1 (default) = the output and down projections run in 2 or 4 parts of K with separate
+ * partial results where that keeps more compute units busy (a badly filled last round of workgroups at a few thousand
+ * tokens; the long-K products of a short prompt); the following norm adds the parts.  0 = never */
 int tg_set_gemm_split(int enable);
 /* prefill, int8 matrix path: 1 (default) = one resident workgroup per compute unit walks its share of the output
  * tiles, the operand prefetch running on from one tile into the next; 0 = one workgroup per tile.  Same results. */

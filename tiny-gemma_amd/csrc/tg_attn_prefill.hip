@@ -42,7 +42,7 @@ constexpr int LDS_LD = 260;
 constexpr int PNT = 256;
 
 // items == nullptr: workgroup b owns query tile gridDim.x - 1 - b and all its keys.
-// items != nullptr (causal layers only): items[b] = {query tile, first key tile, end key tile, slot}; slot < 0: the
+// items != nullptr (a work list, see tg_attn_prefill_plan): items[b] = {query tile, first key tile, end key tile, slot}; slot < 0: the
 // item is the whole key range of its query tile and writes o; else it writes part_o[slot][16][NH][HD] (un-normalised)
 // and part_ml[slot][16][NH][2] (running maximum, running sum).
 __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
