@@ -214,8 +214,9 @@ struct AttnPlanDev {
 	TgAttnPrefillPlan p;
 	bool use = false;
 	int S = -1, tq = 0, window = -1;  // what the lists were built for
-	void *bufs[4] = {nullptr, nullptr, nullptr, nullptr};
+	void *bufs[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
 	std::vector<int4> items, split;  // host copies stay alive until the uploads have completed
+	std::vector<int2> tiles;
 	int build(int n_tokens, int win) {
 		const int tile = tg_attn_prefill_query_tile(n_tokens, g_n_cu);
 		if (n_tokens == S && tile == tq && win == window) return TG_OK;
@@ -237,8 +238,13 @@ struct AttnPlanDev {
 		TG_HIP(hipMalloc(&bufs[3], tg_attn_prefill_ml_floats(nslots, tile) * sizeof(float)));
 		TG_HIP(hipMemcpyAsync(bufs[0], items.data(), items.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
 		TG_HIP(hipMemcpyAsync(bufs[1], split.data(), split.size() * sizeof(int4), hipMemcpyHostToDevice, g_stream));
+		tiles.assign((size_t)((n_tokens + tile - 1) / tile), int2{-1, 1});
+		for (const int4 &sp : split) tiles[(size_t)sp.x] = int2{sp.y, sp.z};
+		TG_HIP(hipMalloc(&bufs[4], tiles.size() * sizeof(int2)));
+		TG_HIP(hipMemcpyAsync(bufs[4], tiles.data(), tiles.size() * sizeof(int2), hipMemcpyHostToDevice, g_stream));
 		p.items = (const int4 *)bufs[0];
 		p.split = (const int4 *)bufs[1];
+		p.tiles = (const int2 *)bufs[4];
 		p.nitems = (int)items.size();
 		p.nsplit = (int)split.size();
 		p.part_o = (float *)bufs[2];
@@ -1317,7 +1323,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
 	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
 	int8_t *apack = (int8_t *)(ws + o_apack);
-	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // partial row maxima: max|ao| per (head, row), then max|hb| per (up|gate tile, row)
+	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // partial row maxima max|hb| per (up|gate tile, row)
 	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
 	s->tap_rows = keep_taps ? n : 0;
 	// Work lists of the attention launches.  A local layer whose window covers the whole prompt is a causal layer.
@@ -1356,10 +1362,13 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
 		                            g_stream);
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp,
-		                       Ld.is_sw ? plan_local : plan_global, amax, g_n_cu, g_stream);
+		const TgAttnPrefillPlan *lplan = Ld.is_sw ? plan_local : plan_global;
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, nullptr, g_n_cu,
+		                       g_stream, pk);
+		// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
+		if (pk) tg_launch_attn_prefill_finish(ao, n, qo, lplan, g_n_cu, apack, rowscale, g_stream);
 		// O (modules.hpp:127-128)
-		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, amax ? c.n_head : 0, nullptr, o_parts, tpart);
+		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk, nullptr, 0, nullptr, o_parts, tpart);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
 		tg_launch_norm_rows(pk ? nullptr : xn, t, o_parts, tpart, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
 		TG_HIP(tap(2 * l + 1));

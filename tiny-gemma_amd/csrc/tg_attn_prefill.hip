@@ -510,6 +510,70 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 	}
 }
 
+// Attention output -> operand of the output projection in one launch: per row, the chunks of a split query tile are
+// merged (as attn_prefill_merge_kernel does), the row maximum over all four heads gives the power-of-two row factor,
+// and the row is written as digit planes.  Two rows per workgroup, a thread = 8 consecutive dims of a row (two waves
+// per row: heads 0-1 and 2-3).  Rows of whole query tiles are read from o, where their workgroup wrote them.
+__global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o, int S, int ldo, const int2 *tiles, const float *part_o,
+                                                                 const float *part_ml, int tq, int8_t *apack, float *rowfac, int Mpad) {
+	__shared__ float wmax[PNT / 64];
+	const int tid = threadIdx.x, t = tid & 127, half = tid >> 7;
+	const int row = 2 * (int)blockIdx.x + half, qrow = row < S ? row : S - 1;  // the odd last row is computed twice, written once
+	const int head = t >> 5, d0 = 8 * (t & 31);
+	int2 ti = int2{-1, 1};
+	if (tiles != nullptr) ti = tiles[qrow / tq];
+	float v[8];
+	if (ti.x < 0) {
+		const float *src = o + (size_t)qrow * ldo + head * HD + d0;
+		const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + 4);
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			v[e] = a[e];
+			v[4 + e] = b[e];
+		}
+	} else {
+		const int qi = qrow % tq;
+		float M = -INFINITY;
+		for (int ch = 0; ch < ti.y; ch++) M = fmaxf(M, part_ml[(((size_t)(ti.x + ch) * tq + qi) * NH + head) * 2]);
+		float L = 0.0f;
+		f32x4 a = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, b = a;
+		for (int ch = 0; ch < ti.y; ch++) {
+			const size_t r = ((size_t)(ti.x + ch) * tq + qi) * NH + head;
+			const float wgt = expf(part_ml[r * 2] - M);
+			L = fmaf(part_ml[r * 2 + 1], wgt, L);
+			a += *reinterpret_cast<const f32x4 *>(part_o + r * HD + d0) * wgt;
+			b += *reinterpret_cast<const f32x4 *>(part_o + r * HD + d0 + 4) * wgt;
+		}
+		a = a / L;
+		b = b / L;
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			v[e] = a[e];
+			v[4 + e] = b[e];
+		}
+	}
+	float amax = 0.0f;
+#pragma unroll
+	for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+	amax = tg_wave_max(amax);
+	if ((tid & 63) == 0) wmax[tid >> 6] = amax;
+	__syncthreads();
+	amax = fmaxf(wmax[2 * half], wmax[2 * half + 1]);
+	if (row >= S) return;
+	float mul, inv;
+	tg_row_factors(amax, mul, inv);
+	if (t == 0) {
+		rowfac[row] = mul;
+		rowfac[Mpad + row] = inv;
+	}
+	uint2 pl[3];
+	tg_quant8(v, mul, pl);
+	const int k0 = head * HD + d0;
+	uint2 *dst = reinterpret_cast<uint2 *>(tg_plane_dst(apack, row, k0 & ~15, NH * HD)) + ((k0 >> 3) & 1);
+#pragma unroll
+	for (int p = 0; p < 3; p++) dst[p * 128] = pl[p];  // planes are 64 pieces of 16 bytes apart
+}
+
 }  // namespace
 
 int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
@@ -571,7 +635,8 @@ size_t tg_attn_prefill_ml_floats(int nslots, int tq) { return (size_t)nslots * t
 
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s) {
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s,
+                            bool finish_later) {
 	(void)n_head;
 	(void)hd;
 	const int Mpad = (int)tg_gemm_mfma_rows(S);  // rowmax_part (may be null): [4 heads][Mpad], max|o[row][head's columns]|
@@ -597,7 +662,15 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	else
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items,
 		                   po, pml, rowmax_part, Mpad);
-	if (whole) return;
+	if (whole || finish_later) return;
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * tq)), dim3(PNT), 0, s, o, S, ldo, plan->split,
 	                   plan->part_o, plan->part_ml, rowmax_part, Mpad, tq);
+}
+
+void tg_launch_attn_prefill_finish(const float *o, int S, int ldo, const TgAttnPrefillPlan *plan, int n_cu, int8_t *apack, float *rowfac,
+                                   hipStream_t s) {
+	const int tq = tg_attn_prefill_query_tile(S, n_cu);
+	hipLaunchKernelGGL(attn_prefill_finish_kernel, dim3((unsigned)((S + 1) / 2)), dim3(PNT), 0, s, o, S, ldo,
+	                   plan ? plan->tiles : nullptr, plan ? plan->part_o : nullptr, plan ? plan->part_ml : nullptr, tq, apack, rowfac,
+	                   (int)tg_gemm_mfma_rows(S));
 }

@@ -166,6 +166,7 @@ void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float
 struct TgAttnPrefillPlan {
 	const int4 *items;  // [nitems] {query tile, first key tile, end key tile, slot or -1}
 	const int4 *split;  // [nsplit] {query tile, first slot, chunks}
+	const int2 *tiles;  // [query tiles] {first slot, chunks} of a split query tile, {-1, 1} of a whole one
 	int nitems, nsplit;
 	float *part_o, *part_ml;
 };
@@ -176,7 +177,13 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 size_t tg_attn_prefill_part_floats(int nslots, int tq);
 size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s);
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s,
+                            bool finish_later = false);
+// The rows of o (S x 1024, 4 heads x 256) -> digit planes + row factors of the int8 MFMA GEMM, merging the partial
+// results of split query tiles on the way (instead of attn_prefill_merge_kernel + the two quantising launches);
+// tg_launch_attn_prefill must then have been called with finish_later = true
+void tg_launch_attn_prefill_finish(const float *o, int S, int ldo, const TgAttnPrefillPlan *plan, int n_cu, int8_t *apack, float *rowfac,
+                                   hipStream_t s);
 // exact-order GEMM on the GEMV tiling (ntiles tiles of Ct columns): C[m][N] = (A[m][K] . W) * scales; epi GEGLU writes C[m][N/2]
 void tg_launch_gemm(float *C, const float *A, const int8_t *Wp, const float *scales, int m, int K, int ntiles, int Ct, int epi,
                     const float *lut, float gmin, float geps, int lut_size, hipStream_t s);
