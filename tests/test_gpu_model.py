@@ -103,6 +103,20 @@ def test_library_built_tables(tg, oracle, golden, weight_images, tables):
     toks, worst = compare_run(sess, osess, prompt, 4, tol=5e-5, tol_first=3e-6)
 
 
+@pytest.mark.parametrize("n_prompt", [1, 2, 3, 17, 33, 65, 129, 257])
+def test_ragged_prompt_lengths(tg, oracle, weight_images, tables, n_prompt):
+    """Prompt lengths that fill no tile of any kernel: one token, odd counts (the finishing launch of the attention
+    takes two rows per workgroup), one past a 16-query / 32-key / 128-row boundary.  Two layers, near-continuous
+    GeLU table: every tap and the logits against the checker, then two decode steps from the caches it left."""
+    image = weight_images("270m", 2, 31)
+    model = tg.Transformer(tg.named_config("270m", 2))
+    model.read_weights_mem(image)
+    gsize = 1 << 20
+    sess = model.session(rope=tables[0], rope_sw=tables[1], gelu_table=oracle.gelu_table(-4.0, 4.0, gsize))
+    osess = oracle.model(gi.oracle_config("270m", 2), image=image).session(-4.0, 4.0, gsize)
+    compare_run(sess, osess, gi.prompt_ids(40 + n_prompt, n_prompt), 2, tol=5e-5, tol_first=3e-6)
+
+
 def test_prompt_longer_than_window(tg, oracle, golden, weight_images, tables):
     """600-token prompt on a model with 512-slot ring caches: 513-key window in prefill
     (ops.hpp:437-443), ring of 512 in decode, tail of the prompt in slots 0..511 (decode.hpp:84-104)."""
