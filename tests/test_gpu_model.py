@@ -317,6 +317,29 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
     assert e.value.code == -1
 
 
+@pytest.mark.parametrize("n_prompt", [90, 700, 2100])
+def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
+    """The three prefill attention kernels (fp32 matrix path with 16-query workgroups, split-bf16 with 16 and with
+    32) behind the same work lists and the same finishing launch: same id, logits within fp32 rounding of each
+    other.  700 tokens: local layers with their own (windowed) work list; 2100: the 32-query tile by default."""
+    cfg = tg.named_config("270m", 2)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 24))
+    sess = model.session(gsize=1 << 20)
+    prompt = gi.prompt_ids(36, n_prompt)
+    out = {}
+    try:
+        for mode in (1, 0, 2):
+            tg.check(tg.lib().tg_set_attn_prefill_mode(mode))
+            sess.reset()
+            out[mode] = sess.prefill(prompt)
+    finally:
+        tg.check(tg.lib().tg_set_attn_prefill_mode(1))
+    for mode in (0, 2):
+        assert out[mode][0] == out[1][0]
+        assert normrel(out[mode][1], out[1][1]) < 2e-5
+
+
 def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
     """A 100-token prompt: the down projection (K = 2048) runs in four parts of K over workgroups and the output
     projection (K = 1024) in two, the following norm adds the partial results.  Against the same prefill with the
