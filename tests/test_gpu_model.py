@@ -340,6 +340,28 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
         assert normrel(out[mode][1], out[1][1]) < 2e-5
 
 
+def test_one_session_many_prompt_lengths(tg, oracle):
+    """A session keeps its prefill workspace and the attention work lists of the last prompt length; prompts of other
+    lengths in between (shorter: lists rebuilt, workspace reused; longer: both regrown; workspace released) must not
+    change what a length gives: the same bits every time."""
+    cfg = tg.named_config("270m", 2)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 25))
+    sess = model.session(gsize=1024)
+    prompts = {n: gi.prompt_ids(37, n) for n in (700, 90, 2100, 1)}
+    first = {}
+    for step, n in enumerate([700, 90, 2100, 700, 1, 90, 2100, 700]):
+        if step == 5:
+            sess.release_workspace()
+        sess.reset()
+        tok, logits = sess.prefill(prompts[n])
+        nxt, _ = sess.decode(tok)
+        if n in first:
+            assert tok == first[n][0] and nxt == first[n][2] and np.array_equal(logits, first[n][1])
+        else:
+            first[n] = (tok, logits.copy(), nxt)
+
+
 def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
     """A 100-token prompt: the down projection (K = 2048) runs in four parts of K over workgroups and the output
     projection (K = 1024) in two, the following norm adds the partial results.  Against the same prefill with the
