@@ -147,15 +147,15 @@ TgGemv gemv_base(const PackedMat &p) {
 
 // C[m][N] = scales * (A[m][K] . W) through the selected GEMM; apack/rowscale are scratch for the MFMA path.
 //   prepacked : the producer of A already wrote the digit planes and row factors
-//   amax_in   : partial row maxima of A left by its producer ([amax_parts][rows]; saves the pass over A that finds them)
-//   amax_out  : GEGLU only: where this product leaves the partial row maxima of C, one part per column tile
+//   amax_in   : row maxima of A left by its producer (saves the pass over A that finds them)
+//   amax_out  : GEGLU only: [rows], cleared by the caller; this product folds max|C[row][:]| into it
 //   kparts    : MFMA path, STORE only, and only what tg_gemm_mfma_k_parts says: the product runs in 2 or 4 parts of K,
 //               part p's partial result goes to C + p * part_stride and the consumer adds them
 void launch_gemm(float *C, const float *A, int lda, const PackedMat &p, int m, int epi, const float *lut, float gmin, float geps,
                  int lut_size, int8_t *apack, float *rowscale, bool prepacked = false, const float *amax_in = nullptr,
-                 int amax_parts = 0, float *amax_out = nullptr, int kparts = 1, size_t part_stride = 0) {
+                 float *amax_out = nullptr, int kparts = 1, size_t part_stride = 0) {
 	if (g_gemm_mfma) {
-		if (!prepacked) tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, amax_in, amax_parts, g_stream);
+		if (!prepacked) tg_launch_quant_pack(A, lda, m, p.K, apack, rowscale, amax_in, g_stream);
 		tg_launch_gemm_mfma(C, apack, rowscale, p.Wg, p.scales_g, m, p.K, p.ntiles_g, epi, lut, gmin, geps, lut_size, amax_out, kparts,
 		                    part_stride, g_stream);
 	} else {
@@ -1276,7 +1276,7 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = plan.build(S, (is_sw && S > sw_context + 1) ? sw_context : -1);
 	if (rc != TG_OK) return done(rc);
-	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), nullptr, g_n_cu, g_stream);
+	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), g_n_cu, g_stream);
 	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
 	rc = tg_copy_d2h(orow.data(), dout, sizeof(float) * rows * NH * HD);
 	if (rc != TG_OK) return done(rc);
@@ -1309,7 +1309,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	             o_hb = carve(sizeof(float) * S * f),
 	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
 	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
-	             o_amax = carve(g_gemm_mfma ? sizeof(float) * (size_t)std::max(2 * f / TG_CT, c.n_head) * tg_gemm_mfma_rows(n) : 0),
+	             o_amax = carve(g_gemm_mfma ? sizeof(float) * tg_gemm_mfma_rows(n) : 0),
 	             o_taps = carve(keep_taps ? sizeof(float) * (size_t)(2 * L + 1) * S * h : 0);
 	if (need > s->pf_ws_bytes) {
 		if (s->pf_ws) (void)hipFree(s->pf_ws);
@@ -1323,7 +1323,7 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
 	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
 	int8_t *apack = (int8_t *)(ws + o_apack);
-	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // partial row maxima max|hb| per (up|gate tile, row)
+	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // max|hb| per row, folded by the up|gate product
 	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
 	s->tap_rows = keep_taps ? n : 0;
 	// Work lists of the attention launches.  A local layer whose window covers the whole prompt is a causal layer.
@@ -1363,18 +1363,19 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		                            g_stream);
 		// attention (modules.hpp:123): local layers use sw_context = max_pos
 		const TgAttnPrefillPlan *lplan = Ld.is_sw ? plan_local : plan_global;
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, nullptr, g_n_cu,
-		                       g_stream, pk);
+		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, g_n_cu, g_stream,
+		                       pk);
 		// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
 		if (pk) tg_launch_attn_prefill_finish(ao, n, qo, lplan, g_n_cu, apack, rowscale, g_stream);
 		// O (modules.hpp:127-128)
-		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk, nullptr, 0, nullptr, o_parts, tpart);
+		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk, nullptr, nullptr, o_parts, tpart);
 		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
-		tg_launch_norm_rows(pk ? nullptr : xn, t, o_parts, tpart, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream);
+		tg_launch_norm_rows(pk ? nullptr : xn, t, o_parts, tpart, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream,
+		                    amax);  // also clears the row maxima the up|gate product folds into
 		TG_HIP(tap(2 * l + 1));
 		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
-		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, 0, amax);
-		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, Ld.ug.ntiles_g, nullptr, d_parts, tpart);
+		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, amax);
+		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, nullptr, d_parts, tpart);
 		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
 		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
 		// the last layer's final norm feeds the LM head GEMV, which reads the fp32 row

@@ -47,7 +47,7 @@ constexpr int PNT = 256;
 // and part_ml[slot][16][NH][2] (running maximum, running sum).
 __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
                                                                int ldkv, int ldo, int is_sw, int window, const int4 *items,
-                                                               float *part_o, float *part_ml, float *rowmax_part, int Mpad) {
+                                                               float *part_o, float *part_ml) {
 	__shared__ __attribute__((aligned(16))) float Ks[TK][LDS_LD];
 	__shared__ __attribute__((aligned(16))) float Vs[TK][LDS_LD];
 
@@ -195,20 +195,10 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0 + 4 * g + i;
-		float omax = 0.0f;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) {
-				const float val = oacc[dt][i] / lr[i];
-				op[16 * dt] = val;
-				omax = fmaxf(omax, fabsf(val));
-			}
-		}
-		// the output projection quantises these rows next: leave max|row| over this head's columns for it
-		if (rowmax_part != nullptr) {
-			omax = tg_row16_max(omax);
-			if (c == 0 && qo < S) rowmax_part[(size_t)head * Mpad + qo] = omax;
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
 		}
 	}
 }
@@ -276,7 +266,7 @@ constexpr int NT32 = HD / 32;  // k steps of a score product
 template <int QG>
 __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
                                                                  int ldkv, int ldo, int is_sw, int window, const int4 *items,
-                                                                 float *part_o, float *part_ml, float *rowmax_part, int Mpad) {
+                                                                 float *part_o, float *part_ml) {
 	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 	// Kb[plane][t][key][g]: dims 32t + 8g .. + 7 of a key; Vb[plane][g][dim]: the 8 keys of group g at one dim
 	bf16x8(*Kb)[NT32][TK][4] = reinterpret_cast<bf16x8(*)[NT32][TK][4]>(smem);
@@ -465,19 +455,10 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0w + 4 * g + i;
-		float omax = 0.0f;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) {
-				const float val = oacc[dt][i] / lr[i];
-				op[16 * dt] = val;
-				omax = fmaxf(omax, fabsf(val));
-			}
-		}
-		if (rowmax_part != nullptr) {
-			omax = tg_row16_max(omax);
-			if (c == 0 && qo < S) rowmax_part[(size_t)head * Mpad + qo] = omax;
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
 		}
 	}
 }
@@ -486,7 +467,7 @@ constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
-                                                                const float *part_ml, float *rowmax_part, int Mpad, int tq) {
+                                                                const float *part_ml, int tq) {
 	const int4 sp = split[blockIdx.x / tq];
 	const int qi = blockIdx.x % tq, qpos = sp.x * tq + qi;
 	if (qpos >= S) return;
@@ -504,10 +485,6 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 	}
 	const f32x4 res = acc / L;
 	*reinterpret_cast<f32x4 *>(o + (size_t)qpos * ldo + head * HD + 4 * lane) = res;
-	if (rowmax_part != nullptr) {
-		const float omax = tg_wave_max(fmaxf(fmaxf(fabsf(res[0]), fabsf(res[1])), fmaxf(fabsf(res[2]), fabsf(res[3]))));
-		if (lane == 0) rowmax_part[(size_t)head * Mpad + qpos] = omax;
-	}
 }
 
 // Attention output -> operand of the output projection in one launch: per row, the chunks of a split query tile are
@@ -635,11 +612,10 @@ size_t tg_attn_prefill_ml_floats(int nslots, int tq) { return (size_t)nslots * t
 
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s,
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
                             bool finish_later) {
 	(void)n_head;
 	(void)hd;
-	const int Mpad = (int)tg_gemm_mfma_rows(S);  // rowmax_part (may be null): [4 heads][Mpad], max|o[row][head's columns]|
 	static bool lds_set = false;
 	if (g_attn_prefill_bf16x3 && !lds_set) {  // 96 KB of dynamic LDS needs the opt-in
 		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -655,16 +631,16 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
 	if (g_attn_prefill_bf16x3 && tq == 32)
 		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
-		                   window, items, po, pml, rowmax_part, Mpad);
+		                   window, items, po, pml);
 	else if (g_attn_prefill_bf16x3)
 		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<1>, grid, dim3(256), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
-		                   window, items, po, pml, rowmax_part, Mpad);
+		                   window, items, po, pml);
 	else
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items,
-		                   po, pml, rowmax_part, Mpad);
+		                   po, pml);
 	if (whole || finish_later) return;
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * tq)), dim3(PNT), 0, s, o, S, ldo, plan->split,
-	                   plan->part_o, plan->part_ml, rowmax_part, Mpad, tq);
+	                   plan->part_o, plan->part_ml, tq);
 }
 
 void tg_launch_attn_prefill_finish(const float *o, int S, int ldo, const TgAttnPrefillPlan *plan, int n_cu, int8_t *apack, float *rowfac,

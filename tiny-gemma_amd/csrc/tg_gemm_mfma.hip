@@ -78,40 +78,28 @@ __global__ __launch_bounds__(GNT) void row_scale_kernel(const float *A, int lda,
 	}
 }
 
-// The same factors from partial row maxima the producer of A left behind: rowmax_part[p][Mpad] = max|A[m][columns of
-// part p]| (the GeGLU epilogue writes one part per column tile, prefill attention one per head), so A is not read.
-// Workgroup = 32 rows; thread (r, kq) folds the parts p = kq, kq + 8, ...; the 8 partial maxima of a row meet in LDS.
-__global__ __launch_bounds__(GNT) void row_scale_parts_kernel(const float *rowmax_part, int nparts, int M, float *mul, float *inv,
-                                                              int Mpad) {
-	__shared__ float pmax[8][32];
-	const int tid = threadIdx.x, r = tid & 31, kq = tid >> 5, m = blockIdx.x * 32 + r;
-	float a0 = 0.0f, a1 = 0.0f;
-	int p = kq;
-	for (; p + 8 < nparts; p += 16) {
-		a0 = fmaxf(a0, rowmax_part[(size_t)p * Mpad + m]);
-		a1 = fmaxf(a1, rowmax_part[(size_t)(p + 8) * Mpad + m]);
-	}
-	if (p < nparts) a0 = fmaxf(a0, rowmax_part[(size_t)p * Mpad + m]);
-	pmax[kq][r] = fmaxf(a0, a1);
-	__syncthreads();
-	if (kq == 0) {
-		float amax = pmax[0][r];
-#pragma unroll
-		for (int i = 1; i < 8; i++) amax = fmaxf(amax, pmax[i][r]);
-		float s, rcp;
-		tg_row_factors(m < M ? amax : 0.0f, s, rcp);  // rows of the padding were never written
-		mul[m] = s;
-		inv[m] = rcp;
-	}
-}
-
 // A [M][lda] fp32 -> digit planes in A-operand order.  Workgroup = 32 rows x 128 k; thread = one lane's 16
 // bytes of one (k step, half): row r = tid % 32, k = 128 blockIdx.y + 16 (tid / 32) .. + 15.
-__global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda, int M, int K, const float *mul, int8_t *Apack) {
+// FROM_MAX: `mul` holds the rows' maxima instead (left by the producer of A): the factors are formed here, and the
+// workgroups of the first 128 k also store them for the product's epilogue (mul_out, inv_out).
+template <bool FROM_MAX>
+__global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda, int M, int K, const float *mul, int8_t *Apack,
+                                                         float *mul_out, float *inv_out) {
 	const int tid = threadIdx.x, r = tid & 31, kq = tid >> 5;
 	const int mtile = blockIdx.x, m = mtile * 32 + r;
 	const int k0 = blockIdx.y * 128 + 16 * kq;
 	i32x4 pl[3] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+	float factor = 1.0f;
+	if (FROM_MAX) {
+		float rcp;
+		tg_row_factors(m < M ? mul[m] : 0.0f, factor, rcp);  // rows of the padding were never written
+		if (blockIdx.y == 0 && kq == 0) {
+			mul_out[m] = factor;
+			inv_out[m] = rcp;
+		}
+	} else if (m < M) {
+		factor = mul[m];
+	}
 	if (m < M) {
 		const f32x4 *src = reinterpret_cast<const f32x4 *>(A + (size_t)m * lda + k0);
 		float v[16];
@@ -121,7 +109,7 @@ __global__ __launch_bounds__(GNT) void quant_pack_kernel(const float *A, int lda
 #pragma unroll
 			for (int i = 0; i < 4; i++) v[4 * q + i] = a[i];
 		}
-		tg_quant16(v, mul[m], pl);
+		tg_quant16(v, factor, pl);
 	}
 	i32x4 *dst = tg_plane_dst(Apack, m, k0, K);
 #pragma unroll
@@ -299,9 +287,10 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 		}
 	}
 	if (GEGLU && rowmax_part != nullptr) {
-		// the consumer quantises these rows next: leave max|row| over this tile's columns for it
+		// the consumer quantises these rows next: fold max|row| over this tile's columns into the row's maximum
+		// (non-negative floats order like their bit patterns; the caller cleared the array)
 		omax = fmaxf(omax, tg_red_partner<32>(omax));
-		if (hb == 0) rowmax_part[(size_t)tile * Mpad + m] = omax;
+		if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
 	}
 }
 
@@ -510,7 +499,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_resident_kernel(float *C, const i
 		}
 		if (GEGLU && rowmax_part != nullptr) {
 			omax = fmaxf(omax, tg_red_partner<32>(omax));
-			if (hb == 0) rowmax_part[(size_t)tile * Mpad + m] = m < M ? omax : 0.0f;
+			if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
 		}
 		cur = n1;
 		n1 = n2;
@@ -705,7 +694,7 @@ __global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int
 		omax = fmaxf(omax, tg_red_partner<32>(omax));
 		if (w < 2 && hb == 0) pmax[w][c] = omax;
 		__syncthreads();
-		if (w == 0 && hb == 0) rowmax_part[(size_t)tile * Mpad + m] = fmaxf(pmax[0][c], pmax[1][c]);
+		if (w == 0 && hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(fmaxf(pmax[0][c], pmax[1][c])));
 	}
 }
 
@@ -716,20 +705,20 @@ size_t tg_gemm_mfma_apack_bytes(int M, int K) { return (size_t)((M + 127) / 128)
 size_t tg_gemm_mfma_rows(int M) { return (size_t)((M + 127) / 128) * 128; }
 
 // A [M][lda] fp32 -> digit planes + row factors; rowfac holds 2 * tg_gemm_mfma_rows(M) floats (multipliers, then inverses).
-// rowmax_part != nullptr: [nparts][tg_gemm_mfma_rows(M)] partial row maxima left by the producer of A (no pass over A for them).
-void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax_part, int nparts,
-                          hipStream_t s) {
+// rowmax != nullptr: [tg_gemm_mfma_rows(M)] row maxima left by the producer of A (no pass over A for them).
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax, hipStream_t s) {
 	const int Mpad = (int)tg_gemm_mfma_rows(M);
-	if (rowmax_part != nullptr)
-		hipLaunchKernelGGL(row_scale_parts_kernel, dim3((unsigned)(Mpad / 32)), dim3(GNT), 0, s, rowmax_part, nparts, M, rowfac, rowfac + Mpad,
-		                   Mpad);
-	else
-		hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)(Mpad / 4)), dim3(GNT), 0, s, A, lda, M, K, rowfac, rowfac + Mpad, Mpad);
-	hipLaunchKernelGGL(quant_pack_kernel, dim3((unsigned)(Mpad / 32), (unsigned)(K / 128)), dim3(GNT), 0, s, A, lda, M, K, rowfac, apack);
+	const dim3 grid((unsigned)(Mpad / 32), (unsigned)(K / 128));
+	if (rowmax != nullptr) {
+		hipLaunchKernelGGL(quant_pack_kernel<true>, grid, dim3(GNT), 0, s, A, lda, M, K, rowmax, apack, rowfac, rowfac + Mpad);
+		return;
+	}
+	hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)(Mpad / 4)), dim3(GNT), 0, s, A, lda, M, K, rowfac, rowfac + Mpad, Mpad);
+	hipLaunchKernelGGL(quant_pack_kernel<false>, grid, dim3(GNT), 0, s, A, lda, M, K, rowfac, apack, (float *)nullptr, (float *)nullptr);
 }
 
 // ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns;
-// rowmax_part (GEGLU only, may be null): [ntiles][tg_gemm_mfma_rows(M)] floats, max|C[m][tile's columns]|
+// rowmax_part (GEGLU only, may be null): [tg_gemm_mfma_rows(M)] floats cleared by the caller; max|C[m][:]| is folded into it
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
                          int kparts, size_t part_stride, hipStream_t s) {

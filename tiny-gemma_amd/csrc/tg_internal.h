@@ -158,7 +158,8 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 // apack/rowfac non-null: the normalised rows are also (out == nullptr: only) written as digit planes + row factors for
 // tg_launch_gemm_mfma (rowfac as tg_launch_quant_pack lays it out for S rows)
 void tg_launch_norm_rows(float *out, const float *in, int nparts, size_t part_stride, const float *w_pre, const float *w_post, const float *resid,
-                         float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s);
+                         float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s,
+                         float *clear_rows = nullptr);  // clear_rows: S floats set to 0 (row maxima the next product folds into)
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,
                                  const float *sin_t, float *kc, float *vc, int max_pos, int S, int n_head, int hd, int ldq, int ldkv,
                                  hipStream_t s);
@@ -177,7 +178,7 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 size_t tg_attn_prefill_part_floats(int nslots, int tq);
 size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
-                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, float *rowmax_part, int n_cu, hipStream_t s,
+                            int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
                             bool finish_later = false);
 // The rows of o (S x 1024, 4 heads x 256) -> digit planes + row factors of the int8 MFMA GEMM, merging the partial
 // results of split query tiles on the way (instead of attn_prefill_merge_kernel + the two quantising launches);
@@ -207,8 +208,7 @@ void tg_launch_retile_mfma(int8_t *dst, float *dst_scales, const TgColMap &m, in
 // int8 MFMA prefill GEMM (tg_gemm_mfma.hip): A is first quantised per row into three int8 digit planes in operand order
 size_t tg_gemm_mfma_apack_bytes(int M, int K);
 size_t tg_gemm_mfma_rows(int M);  // rowfac scratch holds twice this many floats
-void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax_part, int nparts,
-                          hipStream_t s);
+void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, float *rowfac, const float *rowmax, hipStream_t s);
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
                          int kparts, size_t part_stride, hipStream_t s);

@@ -50,10 +50,11 @@ __global__ __launch_bounds__(RNT) void embed_rows_kernel(float *x, const int *id
 template <int ROUNDS, int NPARTS>
 __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float *in, size_t part_stride, const float *w_pre,
                                                         const float *w_post, const float *resid, float *resid_out, int S, int dim,
-                                                        int8_t *apack, float *rowfac, int Mpad) {
+                                                        int8_t *apack, float *rowfac, int Mpad, float *clear_rows) {
 	typedef float f32x4 __attribute__((ext_vector_type(4)));
 	const int lane = threadIdx.x & 63, s = blockIdx.x * (RNT / 64) + (threadIdx.x >> 6);
 	if (s >= S) return;  // uniform over the wave
+	if (clear_rows != nullptr && lane == 0) clear_rows[s] = 0.0f;
 	const float eps = 1e-06f;
 	const int npieces = dim >> 3;
 	bool act[ROUNDS];
@@ -267,13 +268,14 @@ void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, co
 
 // in: nparts (1, 2 or 4) addends of every row, part_stride floats apart
 void tg_launch_norm_rows(float *out, const float *in, int nparts, size_t part_stride, const float *w_pre, const float *w_post,
-                         const float *resid, float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s) {
+                         const float *resid, float *resid_out, int S, int dim, int8_t *apack, float *rowfac, hipStream_t s,
+                         float *clear_rows) {
 	const int Mpad = (int)tg_gemm_mfma_rows(S);
 	const dim3 grid((unsigned)((S + RNT / 64 - 1) / (RNT / 64))), block(RNT);
 	// dim is a legal row dimension: a multiple of 16, at most 1536 where a norm is applied (hidden sizes 640 and 1152)
 #define TG_NORM_ROWS(R, P)                                                                                                        \
 	hipLaunchKernelGGL((norm_rows_kernel<R, P>), grid, block, 0, s, out, in, part_stride, w_pre, w_post, resid, resid_out, S, dim, apack, \
-	                   rowfac, Mpad)
+	                   rowfac, Mpad, clear_rows)
 	if (dim <= 1024) {
 		if (nparts == 4) TG_NORM_ROWS(2, 4);
 		else if (nparts == 2) TG_NORM_ROWS(2, 2);
