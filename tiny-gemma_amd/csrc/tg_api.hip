@@ -29,7 +29,10 @@ float *g_rowscale = nullptr;
 size_t g_rowscale_n = 0;
 int g_prefetch_plan = 0;        // which launch prefetches which weights (experiment knob)
 int g_prefetch_blocks = 128;   // extra workgroups per launch that prefetch the next launch's weights (0: off; multiple of 8)
-int g_gemv_max_blocks = 1024;  // workgroups per GEMV launch before workgroups start looping over tiles
+// Workgroups per GEMV launch before workgroups start looping over tiles.  2048 = 8 per compute unit, all resident at
+// once: the LM head's 2048 tiles each get their own (47 us per launch streamed from HBM, 50-54 us with 1024 that
+// walk two tiles each).
+int g_gemv_max_blocks = 2048;
 bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GPU-side dispatch, not by host launches)
 int g_device = -1;
 hipStream_t g_stream = nullptr;
