@@ -26,7 +26,6 @@ namespace {
 
 constexpr int NT = 256;     // threads per workgroup (4 waves)
 constexpr int NWAVE = 4;
-constexpr int DEPTH = 8;    // 16-byte weight loads in flight per lane
 constexpr int LUT_LDS = 1024;  // GeLU tables up to this size are staged in LDS (one 16-byte load per lane)
 constexpr uint32_t STEP_BYTES = NT * 16u;  // the workgroup reads 4 KiB of its slab per step
 
@@ -37,6 +36,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // 302 MB LM head, rotating over three copies so that nothing is left in the memory-side cache from the
 // previous launch, the stream runs at 6.4 TB/s with it and 5.6 TB/s without.
 constexpr int TG_W_DEFAULT = 0, TG_W_NT = 2;
+// 16-byte weight loads in flight per lane.  The per-layer projections run their loop 1 to 9 times and are
+// bound by latency, not by loads in flight: measured on whole decode steps, 2 is 4 % faster than 8 (1B shape;
+// 8 % on the 270m shape), 1 and 3 and up are slower.  The LM head streams 36 steps per tile and wants 8.
+constexpr int TG_DEPTH_LAYER = 2, TG_DEPTH_STREAM = 8;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 	return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
@@ -85,7 +88,8 @@ __device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const f32x4 x
 	acc[3] = fmaf(xv.z, b2f(d3, 2), acc[3]); acc[3] = fmaf(xv.w, b2f(d3, 3), acc[3]);
 }
 
-template <int PRO, int EPI, int AUX>
+// DEPTH: 16-byte weight loads in flight per lane
+template <int PRO, int EPI, int AUX, int DEPTH>
 __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
 	__shared__ __attribute__((aligned(16))) float lut_s[(EPI == TG_EPI_GEGLU) ? LUT_LDS : 4];  // GeLU table of the GeGLU epilogue
@@ -112,12 +116,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	// instructions, and pieces past the end of the slab (lanes beyond K in the last step) read as 0.
 	const uint32_t slab = (uint32_t)g.K * (uint32_t)C;
 	__amdgpu_buffer_rsrc_t rw = make_rsrc(g.W + (size_t)tile * slab, slab);
-	const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.x, (PRO == TG_PRO_PLAIN) ? (uint32_t)g.K * 4u : 0u);
+	const uint32_t xbytes = (PRO == TG_PRO_PLAIN) ? (uint32_t)g.K * 4u : 0u;
+	const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.x, xbytes);
 	const uint32_t voff = (uint32_t)tid * 16u, xoff = (uint32_t)kpos * 16u, xstep = (uint32_t)KL * 16u;
 
 	// The first DEPTH steps of the weight stream do not depend on the prologue and are requested before
-	// its arithmetic starts, but BEHIND the prologue's own (small) loads: a wait for a load also waits for
-	// every load issued before it, and the prologue must not wait for 32 KB of weights to see its inputs.
+	// its arithmetic ends, but BEHIND the prologue's own (small) loads: a wait for a load also waits for
+	// every load issued before it, and the prologue must not wait for the weights to see its inputs.
 	i32x4 v[DEPTH];
 	f32x4 xq[DEPTH];
 	// Column scales of a tile (and, for the GeGLU epilogue, the GeLU table) are requested together with its first
@@ -136,12 +141,9 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		if (lut_in_lds) lutv = *reinterpret_cast<const f32x4 *>(g.lut + (4 * tid < g.lut_size ? 4 * tid : 0));
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
-			v[u] = i32x4{0, 0, 0, 0};
 			xq[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-			if (u < nit) {
-				v[u] = ldw<AUX>(rw, voff, (uint32_t)u * STEP_BYTES);
-				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
-			}
+			v[u] = ldw<AUX>(rw, voff, min((uint32_t)u * STEP_BYTES, slab));  // past the end of the slab: reads as 0
+			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, min((uint32_t)u * xstep, xbytes));
 		}
 	};
 	if (PRO == TG_PRO_PLAIN) issue_weights();
@@ -240,10 +242,18 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				r[i] = ok ? rv : 0.0f;
 				wpo[i] = ok ? wv : 0.0f;
 			}
-			issue_weights();
+			// The weight stream of a per-layer projection starts once the prologue's inputs are here (the empty asm
+			// keeps the scheduler from hoisting it): requested together with them it made a decode step 0.7 % slower.
+			// The LM head, which is bound by its stream, requests it at once.
+			constexpr bool late = (AUX == TG_W_DEFAULT);
+			if (!late) issue_weights();
 			float ss = 0.0f;
 #pragma unroll
 			for (int i = 0; i < PER; i++) ss = fmaf(p[i], p[i], ss);
+			if (late) {
+				asm volatile("" : "+v"(ss) : : "memory");
+				issue_weights();
+			}
 			ss = block_sum(ss, sred);
 			const float irms = 1.0f / sqrtf(ss / (float)h + eps);
 #pragma unroll
@@ -283,30 +293,20 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		idx = idx < xlast ? idx : xlast;  // lanes past K: their weights read as 0, any finite x will do
 		return *reinterpret_cast<const f32x4 *>(&xs[idx]);
 	};
-	int st = 0;
-	for (; st + 2 * DEPTH <= nit; st += DEPTH) {
+	// One short loop body, executed nit/DEPTH (rounded up) times: a launch of a per-layer projection runs its code
+	// once, from a cold instruction cache, so the bytes of code on its path cost more than the loads they would
+	// save.  Loads are unconditional: pieces past the end of the slab read as 0 without a memory access (buffer
+	// range check) and add nothing to the sums.
+	for (int st = 0; st < nit; st += DEPTH) {
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
 			fma16(acc, v[u], xval(u, st + u));
-			v[u] = ldw<AUX>(rw, voff, (uint32_t)(st + DEPTH + u) * STEP_BYTES);
-			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)(st + DEPTH + u) * xstep);
+			// the scalar offset never passes the end of the buffer: the range check then sees 0 records left
+			const uint32_t nxt = (uint32_t)(st + DEPTH + u);
+			v[u] = ldw<AUX>(rw, voff, min(nxt * STEP_BYTES, slab));
+			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, min(nxt * xstep, xbytes));
 		}
 	}
-	// drain: fewer than 2*DEPTH steps left (all conditions are uniform)
-#pragma unroll
-	for (int u = 0; u < DEPTH; u++) {
-		if (st + u < nit) {
-			fma16(acc, v[u], xval(u, st + u));
-			if (st + DEPTH + u < nit) {
-				v[u] = ldw<AUX>(rw, voff, (uint32_t)(st + DEPTH + u) * STEP_BYTES);
-				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)(st + DEPTH + u) * xstep);
-			}
-		}
-	}
-	st += DEPTH;
-#pragma unroll
-	for (int u = 0; u < DEPTH; u++)
-		if (st + u < nit) fma16(acc, v[u], xval(u, st + u));
 
 	// the next tile's first loads go out before this tile's reduction and epilogue
 	const int cur = tile;
@@ -318,10 +318,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		rw = make_rsrc(g.W + (size_t)tile * slab, slab);
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
-			if (u < nit) {
-				v[u] = ldw<AUX>(rw, voff, (uint32_t)u * STEP_BYTES);
-				if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, (uint32_t)u * xstep);
-			}
+			v[u] = ldw<AUX>(rw, voff, min((uint32_t)u * STEP_BYTES, slab));
+			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, min((uint32_t)u * xstep, xbytes));
 		}
 	}
 
@@ -416,20 +414,20 @@ __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *
 	}
 	return g;
 }
-#define TG_GEMV_KERNEL(NAME, PRO, EPI, AUX)                                                                                   \
+#define TG_GEMV_KERNEL(NAME, PRO, EPI, AUX, DEPTH)                                                                                   \
 	__global__ __launch_bounds__(NT) void NAME(const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, \
 	                                           int hidden, int K, const TgGemv g) {                                            \
-		gemv_body<PRO, EPI, AUX>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));                                               \
+		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));                                               \
 	}
-TG_GEMV_KERNEL(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE, TG_W_DEFAULT)        // layer 0: embedding + pre-norm + Q|K|V
-TG_GEMV_KERNEL(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE, TG_W_DEFAULT)            // post-norm + residual + pre-norm + Q|K|V
-TG_GEMV_KERNEL(tg_gemv_oproj, TG_PRO_ATTN_MERGE, TG_EPI_STORE, TG_W_DEFAULT)       // attention merge + output projection
-TG_GEMV_KERNEL(tg_gemv_upgate_geglu, TG_PRO_RESNORM, TG_EPI_GEGLU, TG_W_DEFAULT)   // post-norm + residual + pre-norm + up|gate + gelu*up
-TG_GEMV_KERNEL(tg_gemv_down, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT)             // down projection
-TG_GEMV_KERNEL(tg_gemv_lmhead_argmax, TG_PRO_RESNORM, TG_EPI_LOGITS, TG_W_NT) // last post-norm + final norm + LM head + argmax stage 1
-TG_GEMV_KERNEL(tg_gemv_lmhead_plain, TG_PRO_PLAIN, TG_EPI_LOGITS, TG_W_NT)    // LM head on an already normalised vector (prefill)
-TG_GEMV_KERNEL(tg_gemv_plain, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT)            // stand-alone y = s * (x . W)
-TG_GEMV_KERNEL(tg_gemv_plain_stream, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_NT)          // the same for a matrix too large to stay cached
+TG_GEMV_KERNEL(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)        // layer 0: embedding + pre-norm + Q|K|V
+TG_GEMV_KERNEL(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)            // post-norm + residual + pre-norm + Q|K|V
+TG_GEMV_KERNEL(tg_gemv_oproj, TG_PRO_ATTN_MERGE, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)       // attention merge + output projection
+TG_GEMV_KERNEL(tg_gemv_upgate_geglu, TG_PRO_RESNORM, TG_EPI_GEGLU, TG_W_DEFAULT, TG_DEPTH_LAYER)   // post-norm + residual + pre-norm + up|gate + gelu*up
+TG_GEMV_KERNEL(tg_gemv_down, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)             // down projection
+TG_GEMV_KERNEL(tg_gemv_lmhead_argmax, TG_PRO_RESNORM, TG_EPI_LOGITS, TG_W_NT, TG_DEPTH_STREAM) // last post-norm + final norm + LM head + argmax stage 1
+TG_GEMV_KERNEL(tg_gemv_lmhead_plain, TG_PRO_PLAIN, TG_EPI_LOGITS, TG_W_NT, TG_DEPTH_STREAM)    // LM head on an already normalised vector (prefill)
+TG_GEMV_KERNEL(tg_gemv_plain, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)            // stand-alone y = s * (x . W)
+TG_GEMV_KERNEL(tg_gemv_plain_stream, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_NT, TG_DEPTH_STREAM)          // the same for a matrix too large to stay cached
 
 // Second stage of the greedy argmax, and the per-token bookkeeping: the winning id becomes the
 // next step's input token, is appended to the id log, and KVCache::update_single's counters
