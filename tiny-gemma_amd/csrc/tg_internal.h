@@ -39,9 +39,9 @@
 // is mostly idle.  A launch can therefore carry extra workgroups whose only job is to touch the
 // weights of the NEXT launch, pulling them out of HBM into the memory-side cache and the L2 while
 // the current launch works through its own latency chain.  A hint only: results do not depend on it.
-// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2); prefetch workgroup G touches
-// the slabs of the consumer tiles t with t % 8 == G % 8, the tiles the consumer's workgroups on the
-// same XCD will read.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2); a prefetch workgroup on XCD x touches
+// the slabs of the consumer tiles t with t % 8 == x, the tiles the consumer's workgroups on the same XCD will
+// read.  That matters: the same loads dealt to the XCDs without regard to the consumer gain nothing (measured).
 struct TgPrefetch {
 	const int8_t *ptr;   // first tile slab of the matrix to prefetch (null: nothing)
 	uint32_t slab;       // bytes per tile slab
@@ -53,26 +53,28 @@ __device__ __forceinline__ void tg_prefetch_block(const TgPrefetch &p, int first
 	if (p.ptr == nullptr) return;
 	const int pb = (int)blockIdx.x - first_extra_block;
 	const int x = (int)(blockIdx.x & 7u), q = pb >> 3, Q = p.nblocks >> 3;
-	// this workgroup's tiles are t = x + 8 q + 8 Q j; their 128-byte lines are walked as one flat index so that
-	// narrow slabs (a few KB) still keep all 256 lanes busy; one dword per line brings the line in
-	const int first = x + 8 * q, stride = 8 * Q;
-	if (first >= p.ntiles) return;
-	const int mytiles = (p.ntiles - first + stride - 1) / stride;
-	const uint32_t lps = p.slab >> 7, total = (uint32_t)mytiles * lps;
-	for (uint32_t i0 = threadIdx.x; i0 < total; i0 += 4u * 256u) {
+	// The workgroups on XCD x share that XCD's tiles t = x, x + 8, ...: the 128-byte lines of those slabs are walked
+	// as one flat index, cut into equal shares (a launch waits for its slowest workgroup).  One dword per line
+	// brings the line in.
+	if (x >= p.ntiles) return;
+	const uint32_t nx = (uint32_t)(p.ntiles - x + 7) >> 3;
+	const uint32_t lps = p.slab >> 7, total = nx * lps;
+	const uint32_t per = (total + (uint32_t)Q - 1) / (uint32_t)Q;
+	const uint32_t lo = (uint32_t)q * per, hi = lo + per < total ? lo + per : total;
+	for (uint32_t i0 = lo + threadIdx.x; i0 < hi; i0 += 4u * 256u) {
 		int sink = 0;
 #pragma unroll
 		for (uint32_t k = 0; k < 4; k++) {  // four loads in flight per lane: unconditional (clamped), consumed together
 			uint32_t i = i0 + k * 256u;
-			i = i < total ? i : i0;
+			i = i < hi ? i : i0;
 			const uint32_t j = i / lps, line = i - j * lps;
-			sink += *(const int *)(p.ptr + (size_t)(first + (int)j * stride) * p.slab + (size_t)line * 128u);
+			sink += *(const int *)(p.ptr + (size_t)(x + 8 * (int)j) * p.slab + (size_t)line * 128u);
 		}
 		asm volatile("" ::"v"(sink));  // the values are not needed, the loads are
 	}
 }
 
-// Two jobs: the first pf.nblocks extra workgroups serve pf, the following pf2.nblocks serve pf2.
+// Extra workgroups of a launch: the first p1.nblocks of them prefetch p1, the rest p2.
 __device__ __forceinline__ void tg_prefetch_dispatch(const TgPrefetch &p1, const TgPrefetch &p2, int first_extra_block) {
 	if ((int)blockIdx.x < first_extra_block + p1.nblocks) tg_prefetch_block(p1, first_extra_block);
 	else tg_prefetch_block(p2, first_extra_block + p1.nblocks);
