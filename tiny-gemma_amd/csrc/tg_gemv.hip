@@ -36,10 +36,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // 302 MB LM head, rotating over three copies so that nothing is left in the memory-side cache from the
 // previous launch, the stream runs at 6.4 TB/s with it and 5.6 TB/s without.
 constexpr int TG_W_DEFAULT = 0, TG_W_NT = 2;
-// 16-byte weight loads in flight per lane.  The per-layer projections run their loop 1 to 9 times and are
-// bound by latency, not by loads in flight: measured on whole decode steps, 2 is 4 % faster than 8 (1B shape;
-// 8 % on the 270m shape), 1 and 3 and up are slower.  The LM head streams 36 steps per tile and wants 8.
-constexpr int TG_DEPTH_LAYER = 2, TG_DEPTH_STREAM = 8;
+// 16-byte weight loads in flight per lane of the LM head, which streams 36 steps per tile.  The per-layer
+// projections cover 1 to 9 steps and are bound by latency, not by loads in flight: measured on whole decode steps, a
+// fixed 2 is 4 % faster than a fixed 8 (1B shape; 8 % on the 270m shape); tg_gemv_depth picks theirs per shape.
+constexpr int TG_DEPTH_STREAM = 8;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 	return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
@@ -414,20 +414,27 @@ __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *
 	}
 	return g;
 }
-#define TG_GEMV_KERNEL(NAME, PRO, EPI, AUX, DEPTH)                                                                                   \
-	__global__ __launch_bounds__(NT) void NAME(const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, \
-	                                           int hidden, int K, const TgGemv g) {                                            \
-		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));                                               \
+// The per-layer roles are templates over DEPTH (the launcher picks it from the number of steps); the LM head has
+// one depth.
+#define TG_GEMV_ARGS const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, int hidden, int K, const TgGemv g
+#define TG_GEMV_KERNEL_T(NAME, PRO, EPI, AUX)                                                         \
+	template <int DEPTH>                                                                              \
+	__global__ __launch_bounds__(NT) void NAME(TG_GEMV_ARGS) {                                        \
+		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));         \
 	}
-TG_GEMV_KERNEL(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)        // layer 0: embedding + pre-norm + Q|K|V
-TG_GEMV_KERNEL(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)            // post-norm + residual + pre-norm + Q|K|V
-TG_GEMV_KERNEL(tg_gemv_oproj, TG_PRO_ATTN_MERGE, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)       // attention merge + output projection
-TG_GEMV_KERNEL(tg_gemv_upgate_geglu, TG_PRO_RESNORM, TG_EPI_GEGLU, TG_W_DEFAULT, TG_DEPTH_LAYER)   // post-norm + residual + pre-norm + up|gate + gelu*up
-TG_GEMV_KERNEL(tg_gemv_down, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)             // down projection
+#define TG_GEMV_KERNEL(NAME, PRO, EPI, AUX, DEPTH)                                                    \
+	__global__ __launch_bounds__(NT) void NAME(TG_GEMV_ARGS) {                                        \
+		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));         \
+	}
+TG_GEMV_KERNEL_T(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE, TG_W_DEFAULT)        // layer 0: embedding + pre-norm + Q|K|V
+TG_GEMV_KERNEL_T(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE, TG_W_DEFAULT)            // post-norm + residual + pre-norm + Q|K|V
+TG_GEMV_KERNEL_T(tg_gemv_oproj, TG_PRO_ATTN_MERGE, TG_EPI_STORE, TG_W_DEFAULT)       // attention merge + output projection
+TG_GEMV_KERNEL_T(tg_gemv_upgate_geglu, TG_PRO_RESNORM, TG_EPI_GEGLU, TG_W_DEFAULT)   // post-norm + residual + pre-norm + up|gate + gelu*up
+TG_GEMV_KERNEL_T(tg_gemv_down, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT)             // down projection
+TG_GEMV_KERNEL_T(tg_gemv_plain, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT)            // stand-alone y = s * (x . W)
 TG_GEMV_KERNEL(tg_gemv_lmhead_argmax, TG_PRO_RESNORM, TG_EPI_LOGITS, TG_W_NT, TG_DEPTH_STREAM) // last post-norm + final norm + LM head + argmax stage 1
 TG_GEMV_KERNEL(tg_gemv_lmhead_plain, TG_PRO_PLAIN, TG_EPI_LOGITS, TG_W_NT, TG_DEPTH_STREAM)    // LM head on an already normalised vector (prefill)
-TG_GEMV_KERNEL(tg_gemv_plain, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_DEFAULT, TG_DEPTH_LAYER)            // stand-alone y = s * (x . W)
-TG_GEMV_KERNEL(tg_gemv_plain_stream, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_NT, TG_DEPTH_STREAM)          // the same for a matrix too large to stay cached
+TG_GEMV_KERNEL(tg_gemv_plain_stream, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_NT, TG_DEPTH_STREAM)     // stand-alone, for a matrix too large to stay cached
 
 // Second stage of the greedy argmax, and the per-token bookkeeping: the winning id becomes the
 // next step's input token, is appended to the id log, and KVCache::update_single's counters
@@ -483,6 +490,25 @@ __global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, con
 
 }  // namespace
 
+// Loads in flight per lane for a launch whose loop covers `nit` steps of 4 KiB per workgroup.  A round of the loop
+// costs a memory round trip plus DEPTH steps of arithmetic (the surplus steps of the last round multiply zeros).
+// Measured on whole decode steps: 1 or 2 steps want 2, 7 steps 4 (2 and 8 are 1.2 % and 1.4 % of a step slower),
+// 9 steps 3; the rule below (a round trip worth 5.5 steps of arithmetic, depth at most 4) reproduces that.  Columns
+// of more than 32 steps are a stream and get 8.
+int tg_gemv_depth(int K, int C) {
+	const int kl = NT / (C >> 2), nit = ((K >> 2) + kl - 1) / kl;
+	if (nit <= 2) return 2;
+	if (nit > 32) return 8;
+	int best = 2;
+	float best_cost = 1e30f;
+	for (int d : {2, 3, 4}) {
+		const int rounds = (nit + d - 1) / d;
+		const float cost = (float)rounds * (5.5f + (float)d);
+		if (cost < best_cost) { best_cost = cost; best = d; }
+	}
+	return best;
+}
+
 void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
 	// more than max_blocks tiles: workgroups loop over tiles, so the prologue is paid once per workgroup
 	TgGemv g = g_in;
@@ -495,20 +521,29 @@ void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
 	if (role == TG_ROLE_OPROJ) { a0 = g.part_acc; a1 = g.part_ml; a2 = a3 = nullptr; }
 	if (role == TG_ROLE_QKV_EMBED) { a0 = g.wte; a1 = g.wte_scales; a2 = g.tok; a3 = g.w_pre; }
 #define TG_LAUNCH(KERNEL) hipLaunchKernelGGL(KERNEL, grid, block, 0, s, a0, a1, a2, a3, g.W, g.hidden, g.K, g)
+#define TG_LAUNCH_D(KERNEL)                          \
+	switch (depth) {                                 \
+		case 2: TG_LAUNCH(KERNEL<2>); break;         \
+		case 3: TG_LAUNCH(KERNEL<3>); break;         \
+		case 4: TG_LAUNCH(KERNEL<4>); break;         \
+		default: TG_LAUNCH(KERNEL<8>); break;        \
+	}
+	const int depth = tg_gemv_depth(g.K, g.C);
 	switch (role) {
-		case TG_ROLE_QKV_EMBED: TG_LAUNCH(tg_gemv_qkv_embed); break;
-		case TG_ROLE_QKV: TG_LAUNCH(tg_gemv_qkv); break;
-		case TG_ROLE_OPROJ: TG_LAUNCH(tg_gemv_oproj); break;
-		case TG_ROLE_UPGATE: TG_LAUNCH(tg_gemv_upgate_geglu); break;
-		case TG_ROLE_DOWN: TG_LAUNCH(tg_gemv_down); break;
+		case TG_ROLE_QKV_EMBED: TG_LAUNCH_D(tg_gemv_qkv_embed); break;
+		case TG_ROLE_QKV: TG_LAUNCH_D(tg_gemv_qkv); break;
+		case TG_ROLE_OPROJ: TG_LAUNCH_D(tg_gemv_oproj); break;
+		case TG_ROLE_UPGATE: TG_LAUNCH_D(tg_gemv_upgate_geglu); break;
+		case TG_ROLE_DOWN: TG_LAUNCH_D(tg_gemv_down); break;
 		case TG_ROLE_LMHEAD: TG_LAUNCH(tg_gemv_lmhead_argmax); break;
 		case TG_ROLE_LMHEAD_PLAIN: TG_LAUNCH(tg_gemv_lmhead_plain); break;
 		default:
 			// a matrix of a quarter of the 256 MB memory-side cache or more is streamed as read-once data
 			if ((size_t)g.K * g.C * g.ntiles >= ((size_t)64 << 20)) TG_LAUNCH(tg_gemv_plain_stream);
-			else TG_LAUNCH(tg_gemv_plain);
+			else TG_LAUNCH_D(tg_gemv_plain);
 			break;
 	}
+#undef TG_LAUNCH_D
 #undef TG_LAUNCH
 }
 
