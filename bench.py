@@ -34,7 +34,7 @@ import __graft_entry__ as ge  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one tg_gemv_lmhead_argmax launch from two `rocprofv3 --pmc` runs (FETCH_SIZE x 1.9999 +
 # WRITE_SIZE x 1.0000, both in KiB, scaled on a 256 MiB copy kernel): profiles/decode_1B_hbm_traffic.md
-LMHEAD_TRAFFIC_BYTES = {"1B": 304_494_496}
+LMHEAD_TRAFFIC_BYTES = {"1B": 304_494_817}
 
 MODELS = {
     # name: (prompt tokens, decode bytes of weights+scales per token, LM-head GEMV algorithmic bytes)
