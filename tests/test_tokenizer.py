@@ -104,6 +104,15 @@ def test_encode_and_decode_equal_the_fixture(tokfile, tgold, chat):
         assert ids.tolist() == [2, 105, 2364, 107, 106, 107, 105, 4368, 107]
 
 
+def test_ids_outside_the_vocabulary_decode_to_nothing(tokfile):
+    """The greedy pick of a row of NaN logits is -1 (ops.hpp:749-757); the reference would index its vocabulary
+    with it (tokenizer.hpp:203-218).  Here such ids have no piece and no byte."""
+    t = Tok(tokfile, 2, 1, gi.TOKENIZER_VOCAB, 0)
+    for tok in (-1, -2**31, gi.TOKENIZER_VOCAB, gi.TOKENIZER_VOCAB + 7, 2**31 - 1):
+        assert t.decode_piece(tok, 5) == b"" and t.byte_of(tok) == -1
+    assert t.decode(np.array([-1, 500, gi.TOKENIZER_VOCAB], np.int32)) == t.decode(np.array([500], np.int32))
+
+
 @pytest.mark.parametrize("prev", [1, 5])
 def test_every_piece_decodes_like_the_fixture(tokfile, tgold, prev):
     t = Tok(tokfile, 2, 1, gi.TOKENIZER_VOCAB, 0)

@@ -154,7 +154,12 @@ class Tokenizer {
 		return tokens;
 	}
 
+	// An id outside [0, vocab_size) has no piece (the reference indexes its vocabulary unchecked, tokenizer.hpp:203-218;
+	// such an id can reach a caller: the argmax of a row of NaN logits is -1, ops.hpp:749-757): it decodes to nothing.
+	bool has_piece(int token) const { return token >= 0 && (size_t)token < vocab.size(); }
+
 	std::string decode(int token, int prev_token) const {
+		if (!has_piece(token)) return std::string();
 		std::string piece = vocab[(size_t)token];
 		if (prev_token == 1 && !piece.empty() && piece[0] == ' ') piece = piece.substr(1);
 		if (byte_piece_value(piece) >= 0) throw std::invalid_argument("stoi");  // as the reference does, see the header comment
@@ -163,6 +168,7 @@ class Tokenizer {
 
 	// The byte a piece of the form <0xHH> stands for, -1 for any other token (no counterpart in the reference).
 	int byte_of(int token) const {
+		if (!has_piece(token)) return -1;
 		const int v = byte_piece_value(vocab[(size_t)token]);
 		return v < 256 ? v : -1;
 	}
