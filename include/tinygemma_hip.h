@@ -7,8 +7,13 @@
  * The reference reports the same conditions by `assert` abort or std::runtime_error; the C++
  * mirror in tiny-gemma_amd/host/ turns the codes back into those exceptions.
  *
- * One caller thread, one HIP stream (tg_stream()), the library owns all device memory of models
- * and sessions.  Citations are file:line in the reference checkout.
+ * Threading contract (the reference is single-threaded with no globals, transformer.hpp:167-258): the library is
+ * NOT thread safe.  One caller thread at a time for the whole library: the stream, the tuning knobs (tg_set_*)
+ * and the scratch of the stand-alone GEMM entry points are process-wide and unsynchronised; only the error
+ * message of tg_last_error() is per thread.  One HIP stream (tg_stream()); the library owns all device memory
+ * of models and sessions.  A model outlives its sessions: tg_model_load_weights* returns TG_ERR_STATE while a
+ * session of the model exists, and after tg_model_destroy every call on a surviving session returns
+ * TG_ERR_STATE (no kernel is launched on freed weights).  Citations are file:line in the reference checkout.
  */
 #ifndef TINYGEMMA_HIP_H
 #define TINYGEMMA_HIP_H
@@ -145,10 +150,13 @@ int tg_decode_enqueue_sampled(tg_session *s, int n_steps, float minp, float temp
  * randf[n_decode + 1] (first entry: the token after the prompt) is only read when minp < 1. */
 int tg_generate(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, float minp, float temp, const float *randf,
                 int32_t *out_ids, double *s_prefill, double *s_decode);
-/* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches */
+/* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches.
+ * Refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
+ * replayed graphs ended the process.  Captured graphs are dropped whenever a tuning knob changes. */
 int tg_set_graphs(int enable);
-/* Debug taps of tg_forward_prefill (a copy of the residual stream after every block, for prompts of up to 1024
- * tokens, read back with tg_session_tap): off by default, they cost one device copy per block. */
+/* Debug taps of tg_forward_prefill (a copy of the residual stream after every block: every row of prompts of up
+ * to 1024 tokens, the last row of longer ones; read back with tg_session_tap): off by default, they cost one
+ * device copy per block. */
 int tg_set_taps(int enable);
 /* prefill GEMM: 1 (default) = int8 matrix cores on three int8 digit planes of the row-scaled activations
  * (exact integer accumulation, fp32-rounding-level accuracy),
@@ -202,9 +210,30 @@ int tg_plan_attention_prefill(int n_tokens, int n_cu, int window, int *query_til
 int tg_plan_gemm_k_parts(int m, int in_dim, int out_dim, int n_cu);
 
 
+/* ---- block level: one modules::attention / mlp / lm_head call at a time (parity checks) ---------------------
+ * The reference's unit tests drive these blocks one by one (tests/csrc/test_bench_modules.cpp:13-512) and hold
+ * them to a norm-relative 1e-3.  Host pointers; x is the residual stream [rows][hidden], replaced by the block's
+ * output (post-norm + residual included).  rows > 1 runs the kernels of tg_forward_prefill, rows == 1 the kernels
+ * of a decode step.  The layer's weights are those of the session's model.  The position counter of a session is
+ * shared by all layers, so a session driven through these entry points should be reset before a forward.
+ * They invalidate the prefill taps.
+ *
+ * modules::attention (modules.hpp:89-169).  rows > 1: needs an empty session; afterwards the layer's cache and the
+ * session's counters are those after a prefill of `rows` tokens.  rows == 1: attends to the layer's cache at the
+ * session's position and advances the counters like KVCache::update_single (decode.hpp:49-70). */
+int tg_block_attention(tg_session *s, int layer, float *x, int rows);
+/* modules::mlp (modules.hpp:171-220) */
+int tg_block_mlp(tg_session *s, int layer, float *x, int rows);
+/* modules::lm_head (modules.hpp:222-247): final norm + LM head on the last row; logits (host) [n_vocab] */
+int tg_block_lm_head(tg_session *s, const float *x, int rows, float *logits);
+/* KVCache::update_prefill (decode.hpp:72-105) on one layer of an empty session: keys/values (host) [rows][head_dim];
+ * a local layer keeps the last n_pos_local rows in slots 0..; counters as after a prefill of `rows` tokens */
+int tg_session_kv_prefill(tg_session *s, int layer, const float *keys, const float *values, int rows);
+
 /* Debug taps: the residual stream of the most recent forward after block b
  * (b = 0: embedding; 2l+1: after attention of layer l; 2l+2: after the MLP of layer l).
- * After a prefill `rows` = prompt length, after a decode 1. out is [rows][hidden]. */
+ * After a prefill `rows` = prompt length (1 for a prompt of more than 1024 tokens: only the last row is kept),
+ * after a decode 1. out is [rows][hidden]. */
 int tg_session_tap(tg_session *s, int b, float *out, int rows);
 /* layer's KV cache as the reference holds it (decode.hpp:14-24): keys/values [max_pos][head_dim] */
 int tg_session_kv(tg_session *s, int layer, float *keys, float *values, int *position_ptr, int *buffer_ptr, int *max_pos);

@@ -339,6 +339,10 @@ class Ref:
         L.ref_prefill.argtypes = [C.c_void_p, c_i32p, C.c_int, c_f32p, c_i32p, c_f32p]
         L.ref_decode.argtypes = [C.c_void_p, C.c_int, c_f32p, c_i32p, c_f32p]
         L.ref_kv_read.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
+        L.ref_block_attention.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
+        L.ref_block_mlp.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
+        L.ref_block_lm_head.argtypes = [C.c_void_p, c_f32p, C.c_int, c_f32p]
+        L.ref_kv_prefill.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, C.c_int]
         L.ref_tok_create.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int]
         L.ref_tok_create.restype = C.c_void_p
         L.ref_tok_destroy.argtypes = [C.c_void_p]
@@ -454,6 +458,28 @@ class _RefSession(_Session):
 
     def _decode(self, tok, logits, arg, tp):
         return self.L.ref_decode(self.h, tok, _f(logits), C.byref(arg), _f(tp))
+
+    # ---- one block at a time (modules::attention / mlp / lm_head) ----
+    def block_attention(self, layer, x):
+        x = np.array(x, np.float32, copy=True, order="C").reshape(-1, self.cfg.hidden)
+        run_big_stack(self.L.ref_block_attention, self.h, layer, _f(x), x.shape[0])
+        return x
+
+    def block_mlp(self, layer, x):
+        x = np.array(x, np.float32, copy=True, order="C").reshape(-1, self.cfg.hidden)
+        run_big_stack(self.L.ref_block_mlp, self.h, layer, _f(x), x.shape[0])
+        return x
+
+    def block_lm_head(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cfg.hidden)
+        logits = np.empty(self.cfg.vocab, np.float32)
+        self.L.ref_block_lm_head(self.h, _f(x), x.shape[0], _f(logits))
+        return logits
+
+    def kv_prefill(self, layer, keys, values):
+        keys = np.ascontiguousarray(keys, np.float32)
+        values = np.ascontiguousarray(values, np.float32)
+        self.L.ref_kv_prefill(self.h, layer, _f(keys), _f(values), keys.shape[0])
 
     def kv(self, layer):
         mp, pp, bp = C.c_int32(), C.c_int32(), C.c_int32()

@@ -315,6 +315,66 @@ int ref_kv_read(void *sp, int layer, float *keys, float *values, int *position_p
 	return 0;
 }
 
+// ---- one block at a time, the way the reference's own unit tests drive them (tests/csrc/test_bench_modules.cpp) ----
+// modules::attention (modules.hpp:89-169) of layer `layer` on the residual stream x [rows][hidden], in place.
+// rows > 1: prefill branch (fills the layer's cache from position 0); rows == 1: decode branch at the cache's position.
+int ref_block_attention(void *sp, int layer, float *x, int rows) {
+	RefSession *s = static_cast<RefSession *>(sp);
+	gemma::Transformer *t = &s->m->t;
+	const int hidden = t->cfg.hidden_size;
+	tensor::activation act(1, rows, hidden);
+	std::memcpy(act.data.get(), x, sizeof(float) * rows * hidden);
+	decode::RoPE *r = t->layers[layer].attn.is_sw ? &s->rope_sw : &s->rope;
+	if (rows > 1) {
+		decode::PrefillState pf(1, rows, &(t->cfg));
+		modules::attention(&act, &(t->layers)[layer].attn, &s->d, &(s->d.kvcache[layer]), &pf, r);
+	} else {
+		modules::attention(&act, &(t->layers)[layer].attn, &s->d, &(s->d.kvcache[layer]), nullptr, r);
+	}
+	std::memcpy(x, act.data.get(), sizeof(float) * rows * hidden);
+	return 0;
+}
+
+// modules::mlp (modules.hpp:171-220) of layer `layer` on x [rows][hidden], in place
+int ref_block_mlp(void *sp, int layer, float *x, int rows) {
+	RefSession *s = static_cast<RefSession *>(sp);
+	gemma::Transformer *t = &s->m->t;
+	const int hidden = t->cfg.hidden_size;
+	tensor::activation act(1, rows, hidden);
+	std::memcpy(act.data.get(), x, sizeof(float) * rows * hidden);
+	if (rows > 1) {
+		decode::PrefillState pf(1, rows, &(t->cfg));
+		modules::mlp(&act, &(t->layers)[layer].mlp, &s->d, &pf, &s->table);
+	} else {
+		modules::mlp(&act, &(t->layers)[layer].mlp, &s->d, nullptr, &s->table);
+	}
+	std::memcpy(x, act.data.get(), sizeof(float) * rows * hidden);
+	return 0;
+}
+
+// modules::lm_head (modules.hpp:222-247) on x [rows][hidden]: logits [n_vocab] of the last row
+int ref_block_lm_head(void *sp, const float *x, int rows, float *logits) {
+	RefSession *s = static_cast<RefSession *>(sp);
+	gemma::Transformer *t = &s->m->t;
+	const int hidden = t->cfg.hidden_size;
+	tensor::activation act(1, rows, hidden);
+	std::memcpy(act.data.get(), x, sizeof(float) * rows * hidden);
+	modules::lm_head(&s->o, &act, &(t->lm_head), &(t->RMSw));
+	std::memcpy(logits, s->o.data.get(), sizeof(float) * t->cfg.n_vocab);
+	return 0;
+}
+
+// KVCache::update_prefill (decode.hpp:72-105) on one layer's empty cache: keys/values [rows][head_dim]
+int ref_kv_prefill(void *sp, int layer, const float *keys, const float *values, int rows) {
+	RefSession *s = static_cast<RefSession *>(sp);
+	const int hd = s->m->t.cfg.head_dim;
+	tensor::activation k(1, 1, rows, hd), v(1, 1, rows, hd);
+	std::memcpy(k.data.get(), keys, sizeof(float) * rows * hd);
+	std::memcpy(v.data.get(), values, sizeof(float) * rows * hd);
+	s->d.kvcache[layer].update_prefill(&k, &v);
+	return 0;
+}
+
 // ---- sentencepiece::Tokenizer (tokenizer.hpp:14-239) ----
 void *ref_tok_create(const char *path, int bos_id, int eos_id, int vocab_size, int chat_format) {
 	try {

@@ -52,6 +52,100 @@ MODEL_CASES = {
     "full1B": ("1B", 26, 1, 178, 1024, 2, 1024),          # 178-token prompt + 1024 greedy steps
 }
 
+# The two long benchmark configurations at full size (tests/golden/golden_long.npz):
+# name: (shape, n_layers, seed, prompt tokens, greedy decode steps, GeLU table size)
+LONG_CASES = {
+    "prefill4096_1B": ("1B", 26, 1, 4096, 0, 1024),       # one forward over 4096 random tokens (weights of full1B)
+    "long16k_270m": ("270m", 18, 5, 16384, 256, 1024),    # 16384-token prefill + 256 greedy steps (weights of full270m)
+}
+LONG_DECODE_LOGIT_STEPS = (0, 1, 128, 255)   # decode steps whose logits head is kept
+
+
+def long_kv_rows(n_prompt):
+    """Cache slots of a long prompt kept in the fixture (those below the layer's valid count are used)."""
+    return np.unique(np.array([0, 1, 255, 511, 512, 1000, n_prompt // 2, n_prompt - 2, n_prompt - 1]))
+
+# Block level (tests/golden/golden_blocks.npz): one modules::attention / mlp / lm_head call on a caller-supplied
+# residual stream, on the shape lists of the reference's own unit tests (tests/scripts/unittests/run_tests.sh:6-32,
+# all global attention on the 270m shape) plus what those never run: local layers (513-key window, ring cache) and
+# the 1B shape.  Weights: the seeded generator's one-layer model; its layer 0 is global with window pattern 1 and
+# local with the usual pattern 6.
+# model name: (shape, weight seed, window pattern)
+BLOCK_MODELS = {"270m_global": ("270m", 61, 1), "270m_local": ("270m", 61, 6), "1B_global": ("1B", 62, 1), "1B_local": ("1B", 62, 6)}
+# case name: (model, kind, rows of the residual stream, keys already cached (attention decode), GeLU table size, seed)
+BLOCK_CASES = {}
+for _S in (1024, 281, 593, 480, 217, 57):
+    BLOCK_CASES[f"attn_prefill_{_S}"] = ("270m_global", "attn", _S, 0, 1024, 700 + _S)
+for _S in (281, 593, 480, 217, 57):
+    BLOCK_CASES[f"mlp_prefill_{_S}"] = ("270m_global", "mlp", _S, 0, 8192, 800 + _S)       # the unit tests' table (8192 entries)
+    BLOCK_CASES[f"mlp_prefill_{_S}_lut1024"] = ("270m_global", "mlp", _S, 0, 1024, 800 + _S)  # the command line's table
+BLOCK_CASES["mlp_decode"] = ("270m_global", "mlp", 1, 0, 8192, 901)
+BLOCK_CASES["mlp_decode_lut1024"] = ("270m_global", "mlp", 1, 0, 1024, 901)
+for _S in (648, 209, 830, 103, 389, 57):
+    BLOCK_CASES[f"attn_decode_{_S}"] = ("270m_global", "attn", 1, _S, 1024, 1000 + _S)
+for _S in (103, 389, 209, 57):
+    BLOCK_CASES[f"lm_head_prefill_{_S}"] = ("270m_global", "lm_head", _S, 0, 1024, 1100 + _S)
+BLOCK_CASES["lm_head_decode"] = ("270m_global", "lm_head", 1, 0, 1024, 1201)
+# not covered by the reference's tests
+BLOCK_CASES["attn_prefill_local_700"] = ("270m_local", "attn", 700, 0, 1024, 1301)       # 513-key window
+BLOCK_CASES["attn_decode_local_ring_700"] = ("270m_local", "attn", 1, 700, 1024, 1302)   # ring holds rows 188..699
+BLOCK_CASES["attn_decode_local_300"] = ("270m_local", "attn", 1, 300, 1024, 1303)
+BLOCK_CASES["attn_decode_global_5000"] = ("270m_global", "attn", 1, 5000, 1024, 1304)    # 32-key workgroups + merge launch
+BLOCK_CASES["attn_prefill_1B_217"] = ("1B_global", "attn", 217, 0, 1024, 1401)
+BLOCK_CASES["attn_prefill_1B_local_600"] = ("1B_local", "attn", 600, 0, 1024, 1402)
+BLOCK_CASES["attn_decode_1B_389"] = ("1B_global", "attn", 1, 389, 1024, 1403)
+BLOCK_CASES["mlp_prefill_1B_217"] = ("1B_global", "mlp", 217, 0, 8192, 1404)
+BLOCK_CASES["mlp_prefill_1B_217_lut1024"] = ("1B_global", "mlp", 217, 0, 1024, 1404)
+BLOCK_CASES["mlp_prefill_1B_700_lut1024"] = ("1B_global", "mlp", 700, 0, 1024, 1407)      # more than 448 rows: the tiled GEMM kernels
+BLOCK_CASES["mlp_decode_1B"] = ("1B_global", "mlp", 1, 0, 8192, 1405)
+BLOCK_CASES["mlp_decode_1B_lut1024"] = ("1B_global", "mlp", 1, 0, 1024, 1405)
+BLOCK_CASES["lm_head_decode_1B"] = ("1B_global", "lm_head", 1, 0, 1024, 1406)
+BLOCK_CASES["lm_head_prefill_1B_57"] = ("1B_global", "lm_head", 57, 0, 1024, 1408)
+
+
+def block_config(model):
+    shape, seed, pattern = BLOCK_MODELS[model]
+    cfg = oracle_config(shape, 1)
+    cfg.pattern = pattern
+    return cfg, seed
+
+
+def block_inputs(name):
+    """(x [rows][hidden] ~ N(0,1) like the reference's unit tests, cached keys, cached values)."""
+    model, kind, rows, cached, gsize, seed = BLOCK_CASES[name]
+    hidden = {"270m": 640, "1B": 1152}[BLOCK_MODELS[model][0]]
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    k = rng.standard_normal((cached, 256)).astype(np.float32) if cached else None
+    v = rng.standard_normal((cached, 256)).astype(np.float32) if cached else None
+    return x, k, v
+
+
+def block_rows(rows):
+    """Rows of a block's output kept in the fixture."""
+    return np.unique(np.concatenate([np.arange(0, rows, 29), np.arange(max(0, rows - 4), rows)]))
+
+
+LOGIT_SAMPLE = np.arange(0, 262144, 61)   # logits of an lm_head block kept in the fixture
+
+# Teacher-forced random-token streams (tests/golden/golden_blocks.npz, "stream/..."): after a short random prompt the
+# reference is fed seeded random ids, so every step sees a fresh context (free-running greedy ids of a random-init
+# model settle into a loop of a few tokens).  name: (shape, n_layers, weight seed, prompt tokens, steps, GeLU table size)
+STREAM_CASES = {
+    "stream270m": ("270m", 18, 5, 8, 320, 1024),
+    "stream1B": ("1B", 26, 1, 8, 320, 1024),
+    # the same streams with a near-continuous GeLU table: what is left is fp32 summation order
+    "stream270m_finelut": ("270m", 18, 5, 8, 320, 1 << 20),
+    "stream1B_finelut": ("1B", 26, 1, 8, 320, 1 << 20),
+}
+STREAM_LOGIT_STEPS = (0, 100, 319)
+
+
+def stream_ids(name):
+    shape, n_layers, seed, n_prompt, steps, gsize = STREAM_CASES[name]
+    rng = np.random.default_rng(5000 + seed)
+    return rng.integers(0, 262144, n_prompt).astype(np.int32), rng.integers(0, 262144, steps).astype(np.int32)
+
 
 def gemv_inputs(i, n, seed):
     rng = np.random.default_rng(seed)

@@ -2,18 +2,23 @@
 checker on the same weights, prompts and tables, and against the compiled reference's recorded
 token ids (tests/golden/golden.npz).
 
-Tolerances.  All arithmetic is fp32 on both sides; summation orders differ.  With a near-continuous
-GeLU table (2^20 entries) the two agree to fp32 rounding end to end (<= 5e-5 norm-relative after
-6 layers).  With the reference CLI's 1024-entry step-function table (csrc/include/ops.hpp:22-52)
-an ULP upstream can move a gate activation to the next table entry, which is worth ~1e-4 of a
-layer's output; the compiled reference and the strict-IEEE checker differ from each other by the
-same mechanism.  Those cases are held to 5e-3 per tap, and greedy token ids must be identical.
+Tolerances.  All arithmetic is fp32 on both sides; summation orders differ.  Every bound is about twice what the
+MI355X run measured (the tests print the measured values).  With a near-continuous GeLU table (2^20 entries) the
+two agree to fp32 rounding end to end: first block 5e-7 .. 1.05e-6 (bound 2.5e-6), every block and the logits
+<= 6e-6 after 6 layers (bound 1.5e-5).  With the reference command line's 1024-entry step-function table
+(csrc/include/ops.hpp:22-52) an ULP upstream can move a gate activation to the next table entry; the compiled
+reference and the strict-IEEE checker differ from each other by the same mechanism (tests/conftest.py, check_picks):
+6 layers 2.8e-3 (bound 5e-3), 18 / 26 layers against the reference's recordings 4.1e-3 / 3.7e-3 (bound 8e-3).
+Greedy picks: the reference's, or its runner-up at a near-tie of the reference.  Observed: 270m shape 64 + 256
+free-running picks identical; 1B shape 178 + 1024 free-running picks identical up to step 771, where the reference's
+top-2 gap is 8.4e-3 and the library takes its runner-up; teacher-forced, that step is the only one of 1025 that differs;
+near-tie seed of the 270m shape: 1 of 257 (gap 3.2e-4).
 """
 import numpy as np
 import pytest
 
 import golden_inputs as gi
-from conftest import normrel
+from conftest import NEAR_TIE, check_picks, normrel
 
 pytestmark = pytest.mark.gpu
 
@@ -38,15 +43,17 @@ def build(tg, oracle, weight_images, tables, name, own_tables=False):
     return model, sess, osess, gi.prompt_ids(seed, n_prompt)
 
 
-def compare_run(sess, osess, prompt, n_decode, tol, tol_first):
+def compare_run(sess, osess, prompt, n_decode, tol, tol_first, what=""):
     tok, logits = sess.prefill(prompt)
     otok, ologits, otaps = osess.prefill(prompt, taps=True)
     taps = sess.taps(rows=prompt.size)
     assert taps.shape[0] == otaps.shape[0] + 1
-    assert normrel(taps[1], otaps[0]) < tol_first      # attention block of layer 0: nothing discontinuous upstream
+    first = normrel(taps[1], otaps[0])
+    assert first < tol_first      # attention block of layer 0: nothing discontinuous upstream
     worst = max(normrel(taps[b + 1], otaps[b]) for b in range(otaps.shape[0]))
     assert worst < tol, worst
-    assert normrel(logits, ologits) < tol
+    worst_logits = normrel(logits, ologits)
+    assert worst_logits < tol
     assert tok == otok
     toks = [tok]
     for _ in range(n_decode):
@@ -54,9 +61,12 @@ def compare_run(sess, osess, prompt, n_decode, tol, tol_first):
         otok, ologits, otp = osess.decode(toks[-1], taps=True)
         dt = sess.taps(rows=1)[:, 0, :]
         worst = max(worst, max(normrel(dt[b + 1], otp[b]) for b in range(otp.shape[0])))
+        worst_logits = max(worst_logits, normrel(logits, ologits))
         assert normrel(logits, ologits) < tol
         assert tok == otok
         toks.append(tok)
+    print(f"{what} {prompt.size} tokens + {n_decode} steps against the CPU checker: first block {first:.2e} (bound {tol_first:.0e}), "
+          f"worst block {worst:.2e}, worst logits {worst_logits:.2e} (bound {tol:.0e})", flush=True)
     assert worst < tol, worst
     return np.array(toks, np.int32), worst
 
@@ -66,7 +76,7 @@ def test_prefill_exact_gemm_mode(tg, oracle, golden, weight_images, tables):
     tg.lib().tg_set_gemm_mode(0)
     try:
         model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut")
-        compare_run(sess, osess, prompt, 2, tol=5e-5, tol_first=3e-6)
+        compare_run(sess, osess, prompt, 2, tol=1.5e-5, tol_first=2.5e-6)
     finally:
         tg.lib().tg_set_gemm_mode(1)
 
@@ -82,7 +92,7 @@ def test_embedding_tap_is_exact(tg, oracle, weight_images, tables):
 
 def test_small_model_fine_table(tg, oracle, golden, weight_images, tables):
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut")
-    toks, worst = compare_run(sess, osess, prompt, 12, tol=5e-5, tol_first=3e-6)
+    toks, worst = compare_run(sess, osess, prompt, 12, tol=1.5e-5, tol_first=2.5e-6, what="small6 (near-continuous table)")
     assert np.array_equal(toks, golden["model/small6_finelut/tokens"])
     # and against the compiled reference's own activations (its rope tables differ in the last bits)
     sess.reset()
@@ -93,14 +103,14 @@ def test_small_model_fine_table(tg, oracle, golden, weight_images, tables):
 
 def test_small_model_cli_table(tg, oracle, golden, weight_images, tables):
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
-    toks, worst = compare_run(sess, osess, prompt, 12, tol=5e-3, tol_first=3e-6)
+    toks, worst = compare_run(sess, osess, prompt, 12, tol=5e-3, tol_first=2.5e-6, what="small6 (1024-entry table)")
     assert np.array_equal(toks, golden["model/small6/tokens"])
 
 
 def test_library_built_tables(tg, oracle, golden, weight_images, tables):
     """NULL tables: the library computes RoPE and GeLU tables itself (decode.hpp:176-201, ops.hpp:29-39)."""
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6_finelut", own_tables=True)
-    toks, worst = compare_run(sess, osess, prompt, 4, tol=5e-5, tol_first=3e-6)
+    toks, worst = compare_run(sess, osess, prompt, 4, tol=1.5e-5, tol_first=2.5e-6)
 
 
 @pytest.mark.parametrize("n_prompt", [1, 2, 3, 17, 33, 65, 129, 257])
@@ -114,7 +124,7 @@ def test_ragged_prompt_lengths(tg, oracle, weight_images, tables, n_prompt):
     gsize = 1 << 20
     sess = model.session(rope=tables[0], rope_sw=tables[1], gelu_table=oracle.gelu_table(-4.0, 4.0, gsize))
     osess = oracle.model(gi.oracle_config("270m", 2), image=image).session(-4.0, 4.0, gsize)
-    compare_run(sess, osess, gi.prompt_ids(40 + n_prompt, n_prompt), 2, tol=5e-5, tol_first=3e-6)
+    compare_run(sess, osess, gi.prompt_ids(40 + n_prompt, n_prompt), 2, tol=1.5e-5, tol_first=2.5e-6)
 
 
 def test_prompt_longer_than_window(tg, oracle, golden, weight_images, tables):
@@ -154,48 +164,42 @@ def test_decode_from_empty_session(tg, oracle, weight_images, tables):
     for _ in range(3):
         t, lg = sess.decode(tok)
         ot, olg, _ = osess.decode(tok)
-        assert t == ot and normrel(lg, olg) < 5e-5
+        assert t == ot and normrel(lg, olg) < 1.5e-5
         tok = t
     assert sess.position == 3
-
-
-NEAR_TIE = 0.02   # top-2 logit gap of the reference below which its runner-up is an acceptable pick (logit spread ~0.5)
 
 
 def greedy_vs_golden(sess, golden, name, prompt, n_decode, strict=True):
     """Free-running greedy ids against the compiled reference's.  strict: identical over the whole horizon.
     Otherwise a divergence may only start at a near-tie of the reference, with the reference's runner-up
-    (after it the two runs legitimately see different contexts)."""
+    (after it the two runs legitimately see different contexts).  Returns the first differing step or -1."""
     toks, s_prefill, s_decode = sess.greedy(prompt, n_decode)
     ref = golden[f"model/{name}/tokens"]
     gaps = golden[f"model/{name}/top2_gaps"]
     mism = np.nonzero(toks != ref)[0]
     if mism.size == 0:
+        print(f"{name}: free-running greedy ids identical to the reference's over {n_decode + 1} picks "
+              f"(its smallest top-2 gap: {float(gaps.min()):.2e})", flush=True)
         return -1
     i = int(mism[0])
-    msg = f"greedy ids diverge from the reference at step {i} (reference top-2 gap there: {gaps[i]:.3e})"
+    msg = f"{name}: free-running greedy ids leave the reference's at step {i} (reference top-2 gap there: {gaps[i]:.3e})"
+    print(msg, flush=True)
     assert not strict, msg
     assert gaps[i] < NEAR_TIE and toks[i] == golden[f"model/{name}/top2_ids"][i][1], msg
     return i
 
 
-def teacher_forced_vs_golden(sess, golden, name, prompt, n_decode, max_mismatches=4):
+def teacher_forced_vs_golden(sess, golden, name, prompt, n_decode, max_mismatches=None):
     """Fed the reference's ids step by step, every pick must be the reference's; at a near-tie of the reference
-    (gap < NEAR_TIE) its runner-up is the only other acceptable answer."""
+    its runner-up is the only other acceptable answer (conftest.check_picks)."""
     ref = golden[f"model/{name}/tokens"]
-    gaps = golden[f"model/{name}/top2_gaps"]
-    pairs = golden[f"model/{name}/top2_ids"]
     tok, _ = sess.prefill(prompt, want_logits=False)
     picks = [tok]
     for i in range(n_decode):
         tok, _ = sess.decode(int(ref[i]), want_logits=False)
         picks.append(tok)
-    picks = np.array(picks, np.int32)
-    mism = np.nonzero(picks != ref)[0]
-    assert mism.size <= max_mismatches, mism
-    for i in mism:
-        assert gaps[i] < NEAR_TIE and picks[i] == pairs[i][1], (i, gaps[i], picks[i], pairs[i])
-    return mism
+    return check_picks(picks, ref, golden[f"model/{name}/top2_gaps"], golden[f"model/{name}/top2_ids"], name + " teacher-forced",
+                       max_mismatches=max_mismatches)
 
 
 def check_weights(golden, weight_images, name):
@@ -212,17 +216,19 @@ def test_full_270m_greedy_ids(tg, oracle, golden, weight_images, tables):
     sess.reset()
     tok, logits = sess.prefill(prompt)
     # 18 layers of the 1024-entry table: the checker itself sits 4e-3 from the compiled reference here
-    assert normrel(logits[:4096], golden["model/full270m/prefill_logits_head"]) < 1e-2
+    rel = normrel(logits[:4096], golden["model/full270m/prefill_logits_head"])
+    print(f"full270m: prefill logits head against the reference's {rel:.2e}", flush=True)
+    assert rel < 8e-3
 
 
 def test_full_270m_near_ties(tg, oracle, golden, weight_images, tables):
     """A seed whose greedy path crosses near-ties of the reference's own logits (top-2 gaps down to
     3e-4 against a logit spread of 0.5).  Teacher-forced with the reference's ids, every step must
-    pick the reference's id, except that at a near-tie (gap < 0.02) the reference's runner-up is the
+    pick the reference's id, except that at a near-tie (gap < conftest.NEAR_TIE) the reference's runner-up is the
     only other acceptable answer."""
     check_weights(golden, weight_images, "full270m_ties")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full270m_ties")
-    teacher_forced_vs_golden(sess, golden, "full270m_ties", prompt, 256)
+    teacher_forced_vs_golden(sess, golden, "full270m_ties", prompt, 256, max_mismatches=3)
 
 
 def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
@@ -235,15 +241,18 @@ def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
     check_weights(golden, weight_images, "full1B")
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "full1B")
     first = greedy_vs_golden(sess, golden, "full1B", prompt, 1024, strict=False)
-    assert first < 0 or first > 256                      # and not early: the first 256 steps hold no gap below 0.01
+    assert first < 0 or first >= 394                     # not early: the reference's smallest top-2 gap before step 394 is 0.105
     sess.reset()
-    teacher_forced_vs_golden(sess, golden, "full1B", prompt, 1024, max_mismatches=6)
+    teacher_forced_vs_golden(sess, golden, "full1B", prompt, 1024, max_mismatches=4)
     # last-position activations of the prefill against the reference's
     sess.reset()
     tok, logits = sess.prefill(prompt)
-    assert normrel(logits[:4096], golden["model/full1B/prefill_logits_head"]) < 2e-2
+    rel = normrel(logits[:4096], golden["model/full1B/prefill_logits_head"])
     last = sess.taps(rows=prompt.size)[1:, -1, :]
-    assert normrel(last, golden["model/full1B/prefill_taps_last"]) < 2e-2
+    want = golden["model/full1B/prefill_taps_last"]
+    per_block = [normrel(last[b], want[b]) for b in range(want.shape[0])]
+    print(f"full1B: prefill logits head against the reference's {rel:.2e}; last-row residuals: worst block {max(per_block):.2e}", flush=True)
+    assert rel < 8e-3 and max(per_block) < 8e-3
 
 
 def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
@@ -284,12 +293,16 @@ def test_long_context_merge_path(tg, oracle, weight_images, tables, n_prompt):
     prompt = gi.prompt_ids(21, n_prompt)
     tok, logits = sess.prefill(prompt)
     otok, ologits, _ = osess.prefill(prompt)
-    assert tok == otok and normrel(logits, ologits) < 5e-5
+    worst = normrel(logits, ologits)
+    assert tok == otok
     for _ in range(3):
         t, lg = sess.decode(tok)
         ot, olg, _ = osess.decode(tok)
-        assert t == ot and normrel(lg, olg) < 5e-5
+        assert t == ot
+        worst = max(worst, normrel(lg, olg))
         tok = t
+    print(f"{n_prompt}-token prompt + 3 steps (merge path): worst logits against the CPU checker {worst:.2e} (bound 1.5e-5)", flush=True)
+    assert worst < 1.5e-5
 
 
 def test_error_paths(tg, oracle, weight_images, tables, tmp_path):

@@ -103,6 +103,10 @@ def lib():
     L.tg_session_read_ids.argtypes = [C.c_void_p, c_i32p, C.c_int, c_i32p]
     L.tg_session_tap.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_session_kv.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
+    L.tg_block_attention.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
+    L.tg_block_mlp.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
+    L.tg_block_lm_head.argtypes = [C.c_void_p, c_f32p, C.c_int, c_f32p]
+    L.tg_session_kv_prefill.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, C.c_int]
     _lib = L
     return L
 
@@ -337,6 +341,31 @@ class Session:
         v = np.empty_like(k)
         check(lib().tg_session_kv(self.h, layer, _f(k), _f(v), None, None, None))
         return k, v, pp.value, bp.value
+
+    # ---- block level (modules::attention / mlp / lm_head one call at a time) ----
+    def block_attention(self, layer, x):
+        """x [rows][hidden] -> the attention block's output (rows > 1: prefill kernels, 1 row: decode kernels)."""
+        x = np.array(x, np.float32, copy=True, order="C").reshape(-1, self.cfg.hidden_size)
+        check(lib().tg_block_attention(self.h, layer, _f(x), x.shape[0]))
+        return x
+
+    def block_mlp(self, layer, x):
+        x = np.array(x, np.float32, copy=True, order="C").reshape(-1, self.cfg.hidden_size)
+        check(lib().tg_block_mlp(self.h, layer, _f(x), x.shape[0]))
+        return x
+
+    def block_lm_head(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cfg.hidden_size)
+        logits = np.empty(self.cfg.n_vocab, np.float32)
+        check(lib().tg_block_lm_head(self.h, _f(x), x.shape[0], _f(logits)))
+        return logits
+
+    def kv_prefill(self, layer, keys, values):
+        """KVCache::update_prefill on one layer of an empty session: keys/values [rows][head_dim]."""
+        keys = np.ascontiguousarray(keys, np.float32)
+        values = np.ascontiguousarray(values, np.float32)
+        assert keys.shape == values.shape and keys.shape[1] == self.cfg.head_dim
+        check(lib().tg_session_kv_prefill(self.h, layer, _f(keys), _f(values), keys.shape[0]))
 
     def free(self):
         if self.h:

@@ -41,6 +41,9 @@ int g_n_cu = 256;
 bool g_gemm_split = true;       // prefill: products that would leave most compute units idle run in 2 or 4 parts of K
 int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
+// Counts changes of the tuning knobs.  A captured decode step bakes the knobs of its capture into its launches
+// (prefetch workgroups, grid limits, attention geometry), so a session drops its captured graphs when this has moved.
+unsigned g_knob_epoch = 0;
 
 bool legal_in(int d) { return d == 640 || d == 2048 || d == 1024 || d == 256 || d == 1152 || d == 6912; }            // static_switch.hpp:7-30
 bool legal_out(int d) { return d == 640 || d == 262144 || d == 2048 || d == 256 || d == 1024 || d == 1152 || d == 6912; }  // :32-58
@@ -203,6 +206,8 @@ struct LayerDev {
 struct tg_model {
 	tg_config cfg;
 	bool loaded = false;
+	int n_sessions = 0;     // live sessions: while there are any, the weights are neither reloaded nor freed under them
+	bool orphaned = false;  // tg_model_destroy was called with live sessions: the last of them deletes the struct
 	int8_t *wte = nullptr;  // [vocab][hidden], reference layout (rows are gathered, never streamed)
 	float *wte_scales = nullptr;
 	float *rmsw = nullptr;
@@ -282,6 +287,10 @@ struct tg_session {
 	float *merged_acc = nullptr, *merged_ml = nullptr;  // long contexts: every TG_ATTN_FOLD partials folded into one
 	float *blk_val = nullptr;
 	int *blk_idx = nullptr;
+	bool counted = false;     // this session is included in m->n_sessions
+	unsigned graph_epoch = 0; // g_knob_epoch the cached graphs were captured under
+	float *zeros = nullptr;   // [hidden] of 0: as the pending block output of a post-norm + residual prologue it adds nothing
+	float *blk_x = nullptr, *blk_y = nullptr;  // [hidden] input / output of the block-level entry points
 	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token
 	int *tok_log = nullptr;
 	int tok_log_cap = 0;
@@ -573,7 +582,11 @@ static void model_free_weights(tg_model *m) {
 
 void tg_model_destroy(tg_model *m) {
 	if (!m) return;
-	model_free_weights(m);
+	model_free_weights(m);  // loaded = false: every entry point of a session that is still alive returns TG_ERR_STATE from now on
+	if (m->n_sessions > 0) {
+		m->orphaned = true;  // the sessions still point here; the last tg_session_destroy deletes the struct
+		return;
+	}
 	delete m;
 }
 
@@ -684,6 +697,8 @@ static int build_from_image(tg_model *m, const uint8_t *d_raw) {
 
 template <typename Fill>
 static int load_weights_impl(tg_model *m, Fill fill) {
+	// a session holds device pointers into the weights (and captured graphs bake them in): no reload under a live session
+	if (m->n_sessions > 0) return tg_fail(TG_ERR_STATE, "the model has live sessions: destroy them before loading weights again");
 	model_free_weights(m);
 	const size_t n = tg_weight_file_bytes(&m->cfg);
 	uint8_t *d_raw = nullptr;
@@ -767,7 +782,7 @@ void tg_session_destroy(tg_session *s) {
 	s->graphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
-	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf};
+	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf, s->zeros, s->blk_x, s->blk_y};
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
 	s->pf_plan.release();
@@ -776,6 +791,11 @@ void tg_session_destroy(tg_session *s) {
 		if (p) (void)hipFree(p);
 	for (float *p : s->vc)
 		if (p) (void)hipFree(p);
+	if (s->counted) {
+		tg_model *m = s->m;
+		m->n_sessions -= 1;
+		if (m->orphaned && m->n_sessions == 0) delete m;
+	}
 	delete s;
 }
 
@@ -842,8 +862,14 @@ int tg_session_create(tg_model *m, const float *rope_cos, const float *rope_sin,
 	TG_ALLOC(s->blk_idx, sizeof(int) * (size_t)m->lm.ntiles);
 	TG_ALLOC(s->ctr, sizeof(int) * 8);
 	TG_ALLOC(s->tok_log, sizeof(int) * (size_t)s->tok_log_cap);
+	TG_ALLOC(s->zeros, sizeof(float) * (size_t)h);
+	TG_ALLOC(s->blk_x, sizeof(float) * (size_t)h);
+	TG_ALLOC(s->blk_y, sizeof(float) * (size_t)h);
 #undef TG_ALLOC
+	if (hipMemset(s->zeros, 0, sizeof(float) * (size_t)h) != hipSuccess) return fail(tg_fail(TG_ERR_HIP, "hipMemset failed"));
 	if ((rc = tg_session_reset(s))) return fail(rc);
+	m->n_sessions += 1;
+	s->counted = true;
 	*out = s;
 	return TG_OK;
 }
@@ -906,7 +932,146 @@ struct StepOnly {
 	int kclass, layer, repeat;
 };
 
+static int session_usable(const tg_session *s) {
+	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	if (!s->m || !s->m->loaded) return tg_fail(TG_ERR_STATE, "the session's model has no weights (destroyed, or a load failed)");
+	return TG_OK;
+}
+
+// ---- the launches of a decode step, one function per kernel (modules.hpp:135-220, 242-246) ----
+// Every projection's launch also does what precedes it in the reference's sequence: the post-norm + residual add of the
+// block before it (`pend` = that block's output, `w_post` its post-norm weights, `x` the residual it is added to; the
+// sum goes to `xr_out`) and its own pre-norm.  A `pend` of zeros adds nothing (its norm is 0), which is how the
+// block-level entry points start a block from a caller's residual stream with the same kernels.
+
+// pre-norm + Q|K|V of layer l (modules.hpp:137-144); embed: the residual is the embedding of the device-side token
+static void launch_qkv(tg_session *s, int l, bool embed, const float *pend, const float *w_post, const float *x, float *xr_out) {
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	const LayerDev &Ld = m->L[(size_t)l];
+	TgGemv g = gemv_base(Ld.qkv);
+	g.hidden = c.hidden_size;
+	g.w_pre = Ld.apre;
+	g.xr_out = xr_out;
+	g.y = s->qkv;
+	g.pf = prefetch_of(Ld.o);
+	if (g_prefetch_plan == 1) g.pf2 = prefetch_of(Ld.ug);
+	if (embed) {
+		g.wte = m->wte;
+		g.wte_scales = m->wte_scales;
+		g.tok = s->ctr + 4;
+		g.vocab = c.n_vocab;
+		g.emb_scale = (float)sqrt((double)c.hidden_size);  // ops.hpp:586
+		tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream);
+	} else {
+		g.pend = pend;
+		g.w_post = w_post;
+		g.x = x;
+		tg_launch_gemv(g, TG_ROLE_QKV, g_stream);
+	}
+}
+
+// Attention launch geometry of layer l at the session's position.
+struct AttnGeom {
+	TgAttnDecode a;
+	bool needs_merge;
+	int nblk;
+};
+static AttnGeom attn_geometry(tg_session *s, int l, bool full_grid) {
+	const tg_config &c = s->m->cfg;
+	const LayerDev &Ld = s->m->L[(size_t)l];
+	AttnGeom ag;
+	TgAttnDecode &a = ag.a;
+	memset(&a, 0, sizeof(a));
+	a.qkv = s->qkv;
+	a.rms_q = Ld.rms_q;
+	a.rms_k = Ld.rms_k;
+	a.cos_t = Ld.is_sw ? s->cos_l : s->cos_g;
+	a.sin_t = Ld.is_sw ? s->sin_l : s->sin_g;
+	a.kc = s->kc[(size_t)l];
+	a.vc = s->vc[(size_t)l];
+	a.max_pos = s->max_pos[(size_t)l];
+	a.pos = s->ctr;
+	a.bp_index = Ld.is_sw ? 1 : 2;
+	// a captured step is replayed at other positions: only then are the counters read from device memory
+	a.host_pos = full_grid ? -1 : s->pos;
+	a.host_bp = full_grid ? -1 : (Ld.is_sw ? s->bp_local : s->bp_global);
+	const int valid = std::min(s->pos + 1, a.max_pos);
+	ag.needs_merge = false;
+	a.chunk = attn_chunk_for(valid, &ag.needs_merge);
+	a.part_acc = s->part_acc;
+	a.part_ml = s->part_ml;
+	a.n_head = c.n_head;
+	a.pf = prefetch_of(g_prefetch_plan == 1 ? Ld.d : Ld.ug);
+	// a captured step is replayed at later positions with the same chunk: launch the largest grid that
+	// chunk can need (workgroups past the valid keys exit at once)
+	ag.nblk = full_grid ? (ag.needs_merge ? std::min(TG_ATTN_MAX_BLOCKS, (a.max_pos + a.chunk - 1) / a.chunk) : TG_ATTN_MERGE_MAX)
+	                    : (valid + a.chunk - 1) / a.chunk;
+	return ag;
+}
+// q/k norm, RoPE, KV write, attention partials (modules.hpp:146-161); the merge launch on long contexts
+static void launch_attn(tg_session *s, const AttnGeom &ag) {
+	tg_launch_attn_decode(ag.a, ag.nblk, g_stream);
+	if (ag.needs_merge) tg_launch_attn_merge(ag.a, ag.nblk, s->merged_acc, s->merged_ml, g_stream);
+}
+// merge of the attention partials + O projection (modules.hpp:161-164)
+static void launch_oproj(tg_session *s, int l, const AttnGeom &ag) {
+	const LayerDev &Ld = s->m->L[(size_t)l];
+	TgGemv g = gemv_base(Ld.o);
+	g.pos = s->ctr;
+	g.host_pos = ag.a.host_pos;
+	g.attn_max_pos = ag.a.max_pos;
+	g.attn_chunk = ag.needs_merge ? TG_ATTN_FOLD * ag.a.chunk : ag.a.chunk;  // folded: one partial per TG_ATTN_FOLD workgroups
+	g.part_acc = ag.needs_merge ? s->merged_acc : s->part_acc;
+	g.part_ml = ag.needs_merge ? s->merged_ml : s->part_ml;
+	g.y = s->o_out;
+	if (g_prefetch_plan == 0) g.pf = prefetch_of(Ld.d);
+	tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream);
+}
+// post-norm + residual of the attention block, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
+static void launch_upgate(tg_session *s, int l, const float *pend, const float *x, float *xr_out) {
+	tg_model *m = s->m;
+	const LayerDev &Ld = m->L[(size_t)l];
+	TgGemv g = gemv_base(Ld.ug);
+	g.hidden = m->cfg.hidden_size;
+	g.pend = pend;
+	g.w_post = Ld.apost;
+	g.x = x;
+	g.xr_out = xr_out;
+	g.w_pre = Ld.mpre;
+	g.y = s->hbuf;
+	g.lut = s->lut;
+	g.gmin = s->gmin;
+	g.geps = s->geps;
+	g.lut_size = s->lut_size;
+	if (l + 1 < m->cfg.n_layers) g.pf = prefetch_of(m->L[(size_t)l + 1].qkv);
+	tg_launch_gemv(g, TG_ROLE_UPGATE, g_stream);
+}
+// down projection (modules.hpp:216-217)
+static void launch_down(tg_session *s, int l) {
+	TgGemv g = gemv_base(s->m->L[(size_t)l].d);
+	g.x = s->hbuf;
+	g.y = s->d_out;
+	tg_launch_gemv(g, TG_ROLE_DOWN, g_stream);
+}
+// last post-norm + residual, final norm, LM head, first stage of the argmax (modules.hpp:242-246, ops.hpp:744)
+static void launch_lmhead(tg_session *s, const float *pend, const float *w_post, const float *x, float *xr_out) {
+	tg_model *m = s->m;
+	TgGemv g = gemv_base(m->lm);
+	g.hidden = m->cfg.hidden_size;
+	g.pend = pend;
+	g.w_post = w_post;
+	g.x = x;
+	g.xr_out = xr_out;
+	g.w_pre = m->rmsw;
+	g.y = s->logits;
+	g.blk_val = s->blk_val;
+	g.blk_idx = s->blk_idx;
+	tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream);
+}
+
 static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid, const StepOnly *only = nullptr) {
+	if (int rc = session_usable(s)) return rc;
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
 	const int L = c.n_layers, h = c.hidden_size;
@@ -922,106 +1087,25 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		TG_HIP(prof->mark(k));                     \
 	}
 	for (int l = 0; l < L; l++) {
-		const LayerDev &Ld = m->L[(size_t)l];
-		// --- pre-norm + Q|K|V (modules.hpp:137-144); folds the previous block's post-norm + residual
-		TgGemv g = gemv_base(Ld.qkv);
-		g.hidden = h;
-		g.w_pre = Ld.apre;
-		g.xr_out = s->xr + (size_t)(2 * l) * h;
-		g.y = s->qkv;
-		g.pf = prefetch_of(Ld.o);
-		if (g_prefetch_plan == 1) g.pf2 = prefetch_of(Ld.ug);
+		float *xr_in = s->xr + (size_t)(2 * l) * h, *xr_mid = s->xr + (size_t)(2 * l + 1) * h;
 		TG_MARK(TG_KC_QKV);
 		if (l == 0) {
-			g.wte = m->wte;
-			g.wte_scales = m->wte_scales;
-			g.tok = s->ctr + 4;
-			g.vocab = c.n_vocab;
-			g.emb_scale = (float)sqrt((double)h);  // ops.hpp:586
-			TG_DO(TG_KC_QKV, l, tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream));
+			TG_DO(TG_KC_QKV, l, launch_qkv(s, l, true, nullptr, nullptr, nullptr, xr_in));
 		} else {
-			g.pend = s->d_out;
-			g.w_post = m->L[(size_t)l - 1].mpost;
-			g.x = s->xr + (size_t)(2 * l - 1) * h;
-			TG_DO(TG_KC_QKV, l, tg_launch_gemv(g, TG_ROLE_QKV, g_stream));
+			TG_DO(TG_KC_QKV, l, launch_qkv(s, l, false, s->d_out, m->L[(size_t)l - 1].mpost, s->xr + (size_t)(2 * l - 1) * h, xr_in));
 		}
-		// --- q/k norm, RoPE, KV write, attention (modules.hpp:146-161)
-		TgAttnDecode a;
-		memset(&a, 0, sizeof(a));
-		a.qkv = s->qkv;
-		a.rms_q = Ld.rms_q;
-		a.rms_k = Ld.rms_k;
-		a.cos_t = Ld.is_sw ? s->cos_l : s->cos_g;
-		a.sin_t = Ld.is_sw ? s->sin_l : s->sin_g;
-		a.kc = s->kc[(size_t)l];
-		a.vc = s->vc[(size_t)l];
-		a.max_pos = s->max_pos[(size_t)l];
-		a.pos = s->ctr;
-		a.bp_index = Ld.is_sw ? 1 : 2;
-		// a captured step is replayed at other positions: only then are the counters read from device memory
-		a.host_pos = full_grid ? -1 : s->pos;
-		a.host_bp = full_grid ? -1 : (Ld.is_sw ? s->bp_local : s->bp_global);
-		const int valid = std::min(s->pos + 1, a.max_pos);
-		bool needs_merge = false;
-		a.chunk = attn_chunk_for(valid, &needs_merge);
-		a.part_acc = s->part_acc;
-		a.part_ml = s->part_ml;
-		a.n_head = c.n_head;
-		a.pf = prefetch_of(g_prefetch_plan == 1 ? Ld.d : Ld.ug);
+		const AttnGeom ag = attn_geometry(s, l, full_grid);
 		TG_MARK(TG_KC_ATTN);
-		// a captured step is replayed at later positions with the same chunk: launch the largest grid that
-		// chunk can need (workgroups past the valid keys exit at once)
-		const int nblk = full_grid ? (needs_merge ? std::min(TG_ATTN_MAX_BLOCKS, (a.max_pos + a.chunk - 1) / a.chunk) : TG_ATTN_MERGE_MAX)
-		                           : (valid + a.chunk - 1) / a.chunk;
-		TG_DO(TG_KC_ATTN, l, tg_launch_attn_decode(a, nblk, g_stream); if (needs_merge) tg_launch_attn_merge(a, nblk, s->merged_acc, s->merged_ml, g_stream));
-		// --- merge of the attention partials + O projection (modules.hpp:161-164)
-		g = gemv_base(Ld.o);
-		g.pos = s->ctr;
-		g.host_pos = a.host_pos;
-		g.attn_max_pos = a.max_pos;
-		g.attn_chunk = needs_merge ? TG_ATTN_FOLD * a.chunk : a.chunk;  // folded: one partial per TG_ATTN_FOLD workgroups
-		g.part_acc = needs_merge ? s->merged_acc : s->part_acc;
-		g.part_ml = needs_merge ? s->merged_ml : s->part_ml;
-		g.y = s->o_out;
-		if (g_prefetch_plan == 0) g.pf = prefetch_of(Ld.d);
+		TG_DO(TG_KC_ATTN, l, launch_attn(s, ag));
 		TG_MARK(TG_KC_OPROJ);
-		TG_DO(TG_KC_OPROJ, l, tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream));
-		// --- post-norm + residual, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
-		g = gemv_base(Ld.ug);
-		g.hidden = h;
-		g.pend = s->o_out;
-		g.w_post = Ld.apost;
-		g.x = s->xr + (size_t)(2 * l) * h;
-		g.xr_out = s->xr + (size_t)(2 * l + 1) * h;
-		g.w_pre = Ld.mpre;
-		g.y = s->hbuf;
-		g.lut = s->lut;
-		g.gmin = s->gmin;
-		g.geps = s->geps;
-		g.lut_size = s->lut_size;
-		if (l + 1 < L) g.pf = prefetch_of(m->L[(size_t)l + 1].qkv);
+		TG_DO(TG_KC_OPROJ, l, launch_oproj(s, l, ag));
 		TG_MARK(TG_KC_UPGATE);
-		TG_DO(TG_KC_UPGATE, l, tg_launch_gemv(g, TG_ROLE_UPGATE, g_stream));
-		// --- down projection (modules.hpp:216-217)
-		g = gemv_base(Ld.d);
-		g.x = s->hbuf;
-		g.y = s->d_out;
+		TG_DO(TG_KC_UPGATE, l, launch_upgate(s, l, s->o_out, xr_in, xr_mid));
 		TG_MARK(TG_KC_DOWN);
-		TG_DO(TG_KC_DOWN, l, tg_launch_gemv(g, TG_ROLE_DOWN, g_stream));
+		TG_DO(TG_KC_DOWN, l, launch_down(s, l));
 	}
-	// --- last post-norm + residual, final norm, LM head, argmax (modules.hpp:242-246, ops.hpp:744)
-	TgGemv g = gemv_base(m->lm);
-	g.hidden = h;
-	g.pend = s->d_out;
-	g.w_post = m->L[(size_t)L - 1].mpost;
-	g.x = s->xr + (size_t)(2 * L - 1) * h;
-	g.xr_out = s->xr + (size_t)(2 * L) * h;
-	g.w_pre = m->rmsw;
-	g.y = s->logits;
-	g.blk_val = s->blk_val;
-	g.blk_idx = s->blk_idx;
 	TG_MARK(TG_KC_LMHEAD);
-	TG_DO(TG_KC_LMHEAD, 0, tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream));
+	TG_DO(TG_KC_LMHEAD, 0, launch_lmhead(s, s->d_out, m->L[(size_t)L - 1].mpost, s->xr + (size_t)(2 * L - 1) * h, s->xr + (size_t)(2 * L) * h));
 	TG_MARK(TG_KC_ARGMAX);
 	if (!only) {
 		if (s->sampling)
@@ -1042,8 +1126,9 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 	return TG_OK;
 }
 
+
 int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax) {
-	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
+	if (int rc = session_usable(s)) return rc;
 	TG_HIP(hipMemcpyAsync(s->ctr + 4, &id, sizeof(int), hipMemcpyHostToDevice, g_stream));
 	if (int rc = enqueue_decode_step(s, nullptr, false)) return rc;
 	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)s->m->cfg.n_vocab, hipMemcpyDeviceToHost, g_stream));
@@ -1066,9 +1151,21 @@ static uint64_t decode_graph_key(const tg_session *s) {
 	return (uint64_t)cl | ((uint64_t)ml << 15) | ((uint64_t)cg << 16) | ((uint64_t)mg << 31);
 }
 
+static void session_drop_graphs(tg_session *s) {
+	for (auto &kv : s->graphs) (void)hipGraphExecDestroy(kv.second);
+	s->graphs.clear();
+}
+
 int tg_decode_enqueue(tg_session *s, int n_steps) {
 	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (int rc = session_usable(s)) return rc;
 	const tg_config &c = s->m->cfg;
+	if (g_use_graphs && s->graph_epoch != g_knob_epoch) {
+		// the graphs captured so far hold the launch parameters of other knob settings
+		TG_HIP(hipStreamSynchronize(g_stream));
+		session_drop_graphs(s);
+		s->graph_epoch = g_knob_epoch;
+	}
 	for (int i = 0; i < n_steps; i++) {
 		if (!g_use_graphs) {
 			if (int rc = enqueue_decode_step(s, nullptr, false)) return rc;
@@ -1113,7 +1210,8 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 }
 
 int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repeat) {
-	if (!s || kernel_class < 0 || kernel_class > TG_KC_LMHEAD || repeat < 1 || layer < 0 || layer >= s->m->cfg.n_layers)
+	if (int rc = session_usable(s)) return rc;
+	if (kernel_class < 0 || kernel_class > TG_KC_LMHEAD || repeat < 1 || layer < 0 || layer >= s->m->cfg.n_layers)
 		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	StepOnly only{kernel_class, kernel_class == TG_KC_LMHEAD ? 0 : layer, repeat};
 	return enqueue_decode_step(s, nullptr, false, &only);
@@ -1147,6 +1245,7 @@ int tg_plan_gemm_k_parts(int m, int in_dim, int out_dim, int n_cu) {
 int tg_set_attn_merge_chunk(int keys) {
 	if (keys < 32 || keys > 256 || keys % 16) return tg_fail(TG_ERR_BAD_ARG, "keys per workgroup: a multiple of 16 in 32..256");
 	g_attn_merge_chunk = keys;
+	g_knob_epoch++;
 	return TG_OK;
 }
 
@@ -1191,21 +1290,36 @@ int tg_set_gemm_mode(int mfma) {
 
 int tg_set_prefetch_plan(int plan) {
 	g_prefetch_plan = plan;
+	g_knob_epoch++;
 	return TG_OK;
 }
 
 int tg_set_prefetch_blocks(int n) {
 	if (n < 0 || (n & 7)) return tg_fail(TG_ERR_BAD_ARG, "prefetch workgroups must be a non-negative multiple of 8");
 	g_prefetch_blocks = n;
+	g_knob_epoch++;
 	return TG_OK;
 }
 
 int tg_set_gemv_max_blocks(int n) {
 	g_gemv_max_blocks = n;
+	g_knob_epoch++;
 	return TG_OK;
 }
 
+// A profiler that traces kernels hooks every launch; replaying captured graphs under rocprofv3 --kernel-trace ended the
+// process on this software stack (ROCm 7.2), so graph replay is refused while a profiler's tool library is loaded.
+static bool profiler_attached() {
+	const char *names[] = {"ROCP_TOOL_LIBRARIES", "ROCPROFILER_LIBRARY_CTOR", "ROCPROF_OUTPUT_PATH"};  // what rocprofv3 exports
+	for (const char *n : names)
+		if (getenv(n) != nullptr) return true;
+	const char *pre = getenv("LD_PRELOAD");
+	return pre != nullptr && strstr(pre, "rocprof") != nullptr;
+}
+
 int tg_set_graphs(int enable) {
+	if (enable && profiler_attached())
+		return tg_fail(TG_ERR_STATE, "graph replay is not available under a profiler (a kernel trace of replayed graphs ended the process); use plain launches");
 	g_use_graphs = enable != 0;
 	return TG_OK;
 }
@@ -1288,19 +1402,31 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	return done(TG_OK);
 }
 
-int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, int32_t *argmax) {
-	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+// ---- forward_prefill in pieces: workspace, the launches of one attention block and of one MLP block ----
+namespace {
+// PrefillState (decode.hpp:281-351): carved out of one arena the session keeps (hipMalloc/hipFree of a few hundred
+// MB per call cost milliseconds), 256-byte aligned pieces, plus the attention work lists of this prompt length.
+struct PrefillCtx {
+	tg_session *s = nullptr;
+	int n = 0;
+	bool pk = false;         // int8 matrix path: producers write digit planes (apack + rowscale) instead of fp32 rows
+	int tap_rows = 0;        // rows of the residual stream kept per block (0: none; n; or 1 = the last row of a long prompt)
+	int *d_ids = nullptr;
+	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr, *amax = nullptr;
+	int8_t *apack = nullptr;
+	const TgAttnPrefillPlan *plan_global = nullptr, *plan_local = nullptr;
+	int o_parts = 1, d_parts = 1;
+	size_t tpart = 0;
+};
+
+int prefill_setup(tg_session *s, int n, PrefillCtx *ctx, bool with_taps) {
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
-	if (n < 1) return tg_fail(TG_ERR_BAD_ARG, "empty prompt");
-	if (s->pos != 0) return tg_fail(TG_ERR_STATE, "prefill needs an empty session (decode.hpp:78-79)");
-	if (n > c.n_pos) return tg_fail(TG_ERR_STATE, "prompt longer than n_pos");
 	const int L = c.n_layers, h = c.hidden_size, f = c.intermediate_size, hd = c.head_dim;
 	const int qo = c.n_head * hd, nq = qo + 2 * hd;
 	const size_t S = (size_t)n;
-	// PrefillState (decode.hpp:281-351): carved out of one arena the session keeps (hipMalloc/hipFree of a few hundred
-	// MB per call cost milliseconds), 256-byte aligned pieces
-	const bool keep_taps = g_keep_taps && n <= PREFILL_TAP_MAX_ROWS;
+	// taps: every row of a short prompt, the last row of a long one
+	const int tap_rows = !(g_keep_taps && with_taps) ? 0 : (n <= PREFILL_TAP_MAX_ROWS ? n : 1);
 	size_t need = 0;
 	auto carve = [&](size_t bytes) {
 		const size_t off = need;
@@ -1313,8 +1439,11 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
 	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
 	             o_amax = carve(g_gemm_mfma ? sizeof(float) * tg_gemm_mfma_rows(n) : 0),
-	             o_taps = carve(keep_taps ? sizeof(float) * (size_t)(2 * L + 1) * S * h : 0);
+	             o_taps = carve(sizeof(float) * (size_t)(2 * L + 1) * (size_t)tap_rows * h);
 	if (need > s->pf_ws_bytes) {
+		TG_HIP(hipStreamSynchronize(g_stream));
+		s->taps = nullptr;  // they live in the workspace
+		s->tap_rows = 0;
 		if (s->pf_ws) (void)hipFree(s->pf_ws);
 		s->pf_ws = nullptr;
 		s->pf_ws_bytes = 0;
@@ -1322,75 +1451,142 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		s->pf_ws_bytes = need;
 	}
 	uint8_t *ws = (uint8_t *)s->pf_ws;
-	int *d_ids = (int *)(ws + o_ids);
-	float *x = (float *)(ws + o_x), *xn = (float *)(ws + o_xn), *qkv = (float *)(ws + o_qkv), *ao = (float *)(ws + o_ao),
-	      *t = (float *)(ws + o_t), *hb = (float *)(ws + o_hb), *rowscale = (float *)(ws + o_rs);
-	int8_t *apack = (int8_t *)(ws + o_apack);
-	float *amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // max|hb| per row, folded by the up|gate product
-	s->taps = keep_taps ? (float *)(ws + o_taps) : nullptr;
-	s->tap_rows = keep_taps ? n : 0;
+	ctx->s = s;
+	ctx->n = n;
+	ctx->pk = g_gemm_mfma != 0;
+	ctx->tap_rows = tap_rows;
+	ctx->d_ids = (int *)(ws + o_ids);
+	ctx->x = (float *)(ws + o_x);
+	ctx->xn = (float *)(ws + o_xn);
+	ctx->qkv = (float *)(ws + o_qkv);
+	ctx->ao = (float *)(ws + o_ao);
+	ctx->t = (float *)(ws + o_t);
+	ctx->hb = (float *)(ws + o_hb);
+	ctx->rowscale = (float *)(ws + o_rs);
+	ctx->apack = (int8_t *)(ws + o_apack);
+	ctx->amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // max|hb| per row, folded by the up|gate product
+	s->taps = tap_rows ? (float *)(ws + o_taps) : nullptr;
+	s->tap_rows = tap_rows;
 	// Work lists of the attention launches.  A local layer whose window covers the whole prompt is a causal layer.
 	const bool local_is_causal = n <= c.n_pos_local + 1;
 	if (int rc = s->pf_plan.build(n, -1)) return rc;
 	if (!local_is_causal) {
 		if (int rc = s->pf_plan_local.build(n, c.n_pos_local)) return rc;
 	}
-	const TgAttnPrefillPlan *plan_global = s->pf_plan.get();
-	const TgAttnPrefillPlan *plan_local = local_is_causal ? plan_global : s->pf_plan_local.get();
-	auto tap = [&](int b) -> hipError_t {
-		if (!keep_taps) return hipSuccess;
-		return hipMemcpyAsync(s->taps + (size_t)b * S * h, x, sizeof(float) * S * h, hipMemcpyDeviceToDevice, g_stream);
-	};
-	TG_HIP(hipMemcpyAsync(d_ids, ids, sizeof(int) * S, hipMemcpyHostToDevice, g_stream));
-	tg_launch_embed_rows(x, d_ids, n, m->wte, m->wte_scales, h, c.n_vocab, g_stream);
-	TG_HIP(tap(0));
-	// xn = rmsnorm(x, attn_pre of layer 0)
-	// With the int8 MFMA GEMM the norm writes the GEMM's digit planes itself and the fp32 row is not stored.
-	const bool pk = g_gemm_mfma;
-	tg_launch_norm_rows(pk ? nullptr : xn, x, 1, 0, m->L[0].apre, nullptr, nullptr, nullptr, n, h, pk ? apack : nullptr, rowscale,
-	                    g_stream);
+	ctx->plan_global = s->pf_plan.get();
+	ctx->plan_local = local_is_causal ? ctx->plan_global : s->pf_plan_local.get();
 	// products that would otherwise leave most compute units idle (a badly filled last round of workgroups; a short
 	// prompt's long-K products) run in 2 or 4 parts of K with separate partial results; the norm that consumes them adds
 	// the parts
-	const size_t tpart = S * h;
-	const int o_parts = (pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, qo, m->L[0].o.ntiles_g, g_n_cu) : 1;
-	const int d_parts = (pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, f, m->L[0].d.ntiles_g, g_n_cu) : 1;
+	ctx->tpart = S * h;
+	ctx->o_parts = (ctx->pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, qo, m->L[0].o.ntiles_g, g_n_cu) : 1;
+	ctx->d_parts = (ctx->pk && g_gemm_split) ? tg_gemm_mfma_k_parts(n, f, m->L[0].d.ntiles_g, g_n_cu) : 1;
+	return TG_OK;
+}
+
+hipError_t prefill_tap(const PrefillCtx &p, int b) {
+	if (!p.tap_rows) return hipSuccess;
+	const size_t h = (size_t)p.s->m->cfg.hidden_size, rows = (size_t)p.tap_rows;
+	return hipMemcpyAsync(p.s->taps + (size_t)b * rows * h, p.x + ((size_t)p.n - rows) * h, sizeof(float) * rows * h, hipMemcpyDeviceToDevice,
+	                      g_stream);
+}
+
+// xn (or its digit planes) = rmsnorm(x, w_pre): the first norm of a forward, or of a block run on its own
+void prefill_first_norm(const PrefillCtx &p, const float *w_pre, bool clear_amax) {
+	const int h = p.s->m->cfg.hidden_size;
+	tg_launch_norm_rows(p.pk ? nullptr : p.xn, p.x, 1, 0, w_pre, nullptr, nullptr, nullptr, p.n, h, p.pk ? p.apack : nullptr, p.rowscale, g_stream,
+	                    clear_amax ? p.amax : nullptr);
+}
+
+// modules::attention, prefill branch (modules.hpp:98-133), from the pre-normalised rows to the output projection's
+// partial results in p.t; the post-norm + residual is the norm launch that follows
+void prefill_attention_launches(const PrefillCtx &p, int l) {
+	tg_session *s = p.s;
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	const int h = c.hidden_size, hd = c.head_dim, qo = c.n_head * hd, nq = qo + 2 * hd, n = p.n;
+	const LayerDev &Ld = m->L[(size_t)l];
+	const int mp = s->max_pos[(size_t)l];
+	// Q|K|V (modules.hpp:106-108)
+	launch_gemm(p.qkv, p.xn, h, Ld.qkv, n, TG_EPI_STORE, nullptr, 0, 0, 0, p.apack, p.rowscale, p.pk);
+	// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
+	tg_launch_qk_norm_rope_rows(p.qkv, p.qkv + qo, p.qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
+	                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq, g_stream);
+	// attention (modules.hpp:123): local layers use sw_context = max_pos
+	const TgAttnPrefillPlan *lplan = Ld.is_sw ? p.plan_local : p.plan_global;
+	tg_launch_attn_prefill(p.ao, p.qkv, p.qkv + qo, p.qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, g_n_cu, g_stream,
+	                       p.pk);
+	// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
+	if (p.pk) tg_launch_attn_prefill_finish(p.ao, n, qo, lplan, g_n_cu, p.apack, p.rowscale, g_stream);
+	// O (modules.hpp:127-128)
+	launch_gemm(p.t, p.ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, p.apack, p.rowscale, p.pk, nullptr, nullptr, p.o_parts, p.tpart);
+}
+
+// modules::mlp, prefill branch (modules.hpp:179-201), from the pre-normalised rows to the down projection's partial
+// results in p.t.  The norm launch before it must have cleared p.amax.
+void prefill_mlp_launches(const PrefillCtx &p, int l) {
+	tg_session *s = p.s;
+	const tg_config &c = s->m->cfg;
+	const LayerDev &Ld = s->m->L[(size_t)l];
+	const int h = c.hidden_size, f = c.intermediate_size, n = p.n;
+	// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
+	launch_gemm(p.hb, p.xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, p.apack, p.rowscale, p.pk, nullptr, p.amax);
+	launch_gemm(p.t, p.hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, p.apack, p.rowscale, false, p.amax, nullptr, p.d_parts, p.tpart);
+}
+
+// x = rmsnorm(t, w_post) + x, then xn (or its digit planes) = rmsnorm(x, next_pre)  (modules.hpp:130-132, 188, 199-201)
+void prefill_block_end(const PrefillCtx &p, int nparts, const float *w_post, const float *next_pre, bool want_fp32, bool clear_amax) {
+	const int h = p.s->m->cfg.hidden_size;
+	const bool planes = p.pk && !want_fp32;
+	tg_launch_norm_rows(planes ? nullptr : p.xn, p.t, nparts, p.tpart, next_pre, w_post, p.x, p.x, p.n, h, planes ? p.apack : nullptr, p.rowscale,
+	                    g_stream, clear_amax ? p.amax : nullptr);
+}
+
+// KVCache::update_prefill's counters (decode.hpp:99-104) after n tokens
+int set_counters_after_prefill(tg_session *s, int n) {
+	const tg_config &c = s->m->cfg;
+	s->pos = n;
+	s->bp_local = (n >= c.n_pos_local) ? c.n_pos_local : n;
+	s->bp_global = (n >= c.n_pos) ? c.n_pos : n;
+	int ctr[3] = {s->pos, s->bp_local, s->bp_global};
+	TG_HIP(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));  // ctr[] is on this function's stack
+	return TG_OK;
+}
+}  // namespace
+
+int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, int32_t *argmax) {
+	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (int rc = session_usable(s)) return rc;
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	if (n < 1) return tg_fail(TG_ERR_BAD_ARG, "empty prompt");
+	if (s->pos != 0) return tg_fail(TG_ERR_STATE, "prefill needs an empty session (decode.hpp:78-79)");
+	if (n > c.n_pos) return tg_fail(TG_ERR_STATE, "prompt longer than n_pos");
+	const int L = c.n_layers, h = c.hidden_size;
+	const size_t S = (size_t)n;
+	PrefillCtx p;
+	if (int rc = prefill_setup(s, n, &p, true)) return rc;
+	TG_HIP(hipMemcpyAsync(p.d_ids, ids, sizeof(int) * S, hipMemcpyHostToDevice, g_stream));
+	tg_launch_embed_rows(p.x, p.d_ids, n, m->wte, m->wte_scales, h, c.n_vocab, g_stream);
+	TG_HIP(prefill_tap(p, 0));
+	// With the int8 MFMA GEMM a norm writes the next GEMM's digit planes itself and the fp32 row is not stored.
+	prefill_first_norm(p, m->L[0].apre, false);
 	for (int l = 0; l < L; l++) {
 		const LayerDev &Ld = m->L[(size_t)l];
-		const int mp = s->max_pos[(size_t)l];
-		// Q|K|V (modules.hpp:106-108)
-		launch_gemm(qkv, xn, h, Ld.qkv, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk);
-		// q/k norm + RoPE from position 0, KV write (modules.hpp:115-121)
-		tg_launch_qk_norm_rope_rows(qkv, qkv + qo, qkv + qo + hd, Ld.rms_q, Ld.rms_k, Ld.is_sw ? s->cos_l : s->cos_g,
-		                            Ld.is_sw ? s->sin_l : s->sin_g, s->kc[(size_t)l], s->vc[(size_t)l], mp, n, c.n_head, hd, nq, nq,
-		                            g_stream);
-		// attention (modules.hpp:123): local layers use sw_context = max_pos
-		const TgAttnPrefillPlan *lplan = Ld.is_sw ? plan_local : plan_global;
-		tg_launch_attn_prefill(ao, qkv, qkv + qo, qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, g_n_cu, g_stream,
-		                       pk);
-		// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
-		if (pk) tg_launch_attn_prefill_finish(ao, n, qo, lplan, g_n_cu, apack, rowscale, g_stream);
-		// O (modules.hpp:127-128)
-		launch_gemm(t, ao, qo, Ld.o, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, pk, nullptr, nullptr, o_parts, tpart);
-		// x = rmsnorm(t, attn_post) + x ; xn = rmsnorm(x, mlp_pre) (modules.hpp:130-132, 188)
-		tg_launch_norm_rows(pk ? nullptr : xn, t, o_parts, tpart, Ld.mpre, Ld.apost, x, x, n, h, pk ? apack : nullptr, rowscale, g_stream,
-		                    amax);  // also clears the row maxima the up|gate product folds into
-		TG_HIP(tap(2 * l + 1));
-		// up|gate + gelu*up (modules.hpp:190-195), down (modules.hpp:196-197)
-		launch_gemm(hb, xn, h, Ld.ug, n, TG_EPI_GEGLU, s->lut, s->gmin, s->geps, s->lut_size, apack, rowscale, pk, nullptr, amax);
-		launch_gemm(t, hb, f, Ld.d, n, TG_EPI_STORE, nullptr, 0, 0, 0, apack, rowscale, false, amax, nullptr, d_parts, tpart);
-		// x = rmsnorm(t, mlp_post) + x ; xn = rmsnorm(x, next pre-norm) (modules.hpp:199-201)
-		const float *next_pre = (l + 1 < L) ? m->L[(size_t)l + 1].apre : m->rmsw;
+		prefill_attention_launches(p, l);
+		prefill_block_end(p, p.o_parts, Ld.apost, Ld.mpre, false, true);  // also clears the row maxima the up|gate product folds into
+		TG_HIP(prefill_tap(p, 2 * l + 1));
+		prefill_mlp_launches(p, l);
 		// the last layer's final norm feeds the LM head GEMV, which reads the fp32 row
 		const bool last = l + 1 == L;
-		tg_launch_norm_rows((pk && !last) ? nullptr : xn, t, d_parts, tpart, next_pre, Ld.mpost, x, x, n, h, (pk && !last) ? apack : nullptr, rowscale,
-		                    g_stream);
-		TG_HIP(tap(2 * l + 2));
+		prefill_block_end(p, p.d_parts, Ld.mpost, last ? m->rmsw : m->L[(size_t)l + 1].apre, last, false);
+		TG_HIP(prefill_tap(p, 2 * l + 2));
 	}
 	// LM head on the last position only (modules.hpp:232-240): xn already holds rmsnorm(x, RMSw)
 	{
 		TgGemv g = gemv_base(m->lm);
-		g.x = xn + (S - 1) * h;
+		g.x = p.xn + (S - 1) * h;
 		g.y = s->logits;
 		g.blk_val = s->blk_val;
 		g.blk_idx = s->blk_idx;
@@ -1398,13 +1594,8 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 		tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 0, g_stream);
 	}
 	TG_HIP(hipGetLastError());
-	// KVCache::update_prefill's counters (decode.hpp:99-104)
-	s->pos = n;
-	s->bp_local = (n >= c.n_pos_local) ? c.n_pos_local : n;
-	s->bp_global = (n >= c.n_pos) ? c.n_pos : n;
 	s->steps = 1;
-	int ctr[3] = {s->pos, s->bp_local, s->bp_global};
-	TG_HIP(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
+	if (int rc = set_counters_after_prefill(s, n)) return rc;
 	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)c.n_vocab, hipMemcpyDeviceToHost, g_stream));
 	int32_t tok = -1;
 	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
@@ -1412,6 +1603,126 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	if (argmax) *argmax = tok;
 	return TG_OK;
 }
+
+// ---------------------------------------------------------------------------------------------
+// block level (parity checks of one modules::attention / mlp / lm_head call at a time)
+// ---------------------------------------------------------------------------------------------
+static int block_args_ok(tg_session *s, int layer, const float *x, int rows) {
+	if (int rc = session_usable(s)) return rc;
+	const tg_config &c = s->m->cfg;
+	if (!x || rows < 1 || layer < 0 || layer >= c.n_layers) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (rows > c.n_pos) return tg_fail(TG_ERR_STATE, "more rows than n_pos");
+	return TG_OK;
+}
+
+int tg_session_kv_prefill(tg_session *s, int layer, const float *keys, const float *values, int rows) {
+	if (int rc = block_args_ok(s, layer, keys, rows)) return rc;
+	if (!values) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (s->pos != 0 && s->pos != rows) return tg_fail(TG_ERR_STATE, "the session's position counter is shared by all layers: reset it, or give every layer the same number of rows");
+	const int hd = s->m->cfg.head_dim, mp = s->max_pos[(size_t)layer];
+	const int start = rows >= mp ? rows - mp : 0;  // decode.hpp:84-86: the tail of a context longer than the cache
+	const size_t bytes = sizeof(float) * (size_t)(rows - start) * hd;
+	TG_HIP(hipMemcpyAsync(s->kc[(size_t)layer], keys + (size_t)start * hd, bytes, hipMemcpyHostToDevice, g_stream));
+	TG_HIP(hipMemcpyAsync(s->vc[(size_t)layer], values + (size_t)start * hd, bytes, hipMemcpyHostToDevice, g_stream));
+	return set_counters_after_prefill(s, rows);
+}
+
+int tg_block_attention(tg_session *s, int layer, float *x, int rows) {
+	if (int rc = block_args_ok(s, layer, x, rows)) return rc;
+	tg_model *m = s->m;
+	const int h = m->cfg.hidden_size;
+	const LayerDev &Ld = m->L[(size_t)layer];
+	if (rows == 1) {
+		// decode branch (modules.hpp:135-169) with the kernels of a decode step; the launch that follows the output
+		// projection in a step (up|gate) forms post-norm + residual, its own product is not used
+		if (s->pos >= m->cfg.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
+		TG_HIP(hipMemcpyAsync(s->blk_x, x, sizeof(float) * (size_t)h, hipMemcpyHostToDevice, g_stream));
+		launch_qkv(s, layer, false, s->zeros, Ld.apost, s->blk_x, nullptr);
+		const AttnGeom ag = attn_geometry(s, layer, false);
+		launch_attn(s, ag);
+		launch_oproj(s, layer, ag);
+		launch_upgate(s, layer, s->o_out, s->blk_x, s->blk_y);
+		TG_HIP(hipGetLastError());
+		TG_HIP(hipMemcpyAsync(x, s->blk_y, sizeof(float) * (size_t)h, hipMemcpyDeviceToHost, g_stream));
+		// KVCache::update_single advanced this layer's counters (decode.hpp:68-69); the session has one set for all layers
+		s->pos += 1;
+		s->bp_local += 1;
+		s->bp_global += 1;
+		int ctr[3] = {s->pos, s->bp_local, s->bp_global};
+		TG_HIP(hipMemcpyAsync(s->ctr, ctr, sizeof(ctr), hipMemcpyHostToDevice, g_stream));
+		TG_HIP(hipStreamSynchronize(g_stream));
+		s->taps = nullptr;
+		s->tap_rows = 0;
+		return TG_OK;
+	}
+	if (s->pos != 0) return tg_fail(TG_ERR_STATE, "prefill needs an empty session (decode.hpp:78-79)");
+	PrefillCtx p;
+	if (int rc = prefill_setup(s, rows, &p, false)) return rc;
+	const size_t bytes = sizeof(float) * (size_t)rows * h;
+	TG_HIP(hipMemcpyAsync(p.x, x, bytes, hipMemcpyHostToDevice, g_stream));
+	prefill_first_norm(p, Ld.apre, false);
+	prefill_attention_launches(p, layer);
+	prefill_block_end(p, p.o_parts, Ld.apost, Ld.mpre, false, false);
+	TG_HIP(hipGetLastError());
+	TG_HIP(hipMemcpyAsync(x, p.x, bytes, hipMemcpyDeviceToHost, g_stream));
+	return set_counters_after_prefill(s, rows);
+}
+
+int tg_block_mlp(tg_session *s, int layer, float *x, int rows) {
+	if (int rc = block_args_ok(s, layer, x, rows)) return rc;
+	tg_model *m = s->m;
+	const int h = m->cfg.hidden_size;
+	const LayerDev &Ld = m->L[(size_t)layer];
+	if (rows == 1) {
+		// decode branch (modules.hpp:203-220): the launch that follows the down projection in a step (the next Q|K|V)
+		// forms post-norm + residual
+		TG_HIP(hipMemcpyAsync(s->blk_x, x, sizeof(float) * (size_t)h, hipMemcpyHostToDevice, g_stream));
+		launch_upgate(s, layer, s->zeros, s->blk_x, nullptr);
+		launch_down(s, layer);
+		launch_qkv(s, layer, false, s->d_out, Ld.mpost, s->blk_x, s->blk_y);
+		TG_HIP(hipGetLastError());
+		TG_HIP(hipMemcpyAsync(x, s->blk_y, sizeof(float) * (size_t)h, hipMemcpyDeviceToHost, g_stream));
+		TG_HIP(hipStreamSynchronize(g_stream));
+		return TG_OK;
+	}
+	PrefillCtx p;
+	if (int rc = prefill_setup(s, rows, &p, false)) return rc;
+	const size_t bytes = sizeof(float) * (size_t)rows * h;
+	TG_HIP(hipMemcpyAsync(p.x, x, bytes, hipMemcpyHostToDevice, g_stream));
+	prefill_first_norm(p, Ld.mpre, true);
+	prefill_mlp_launches(p, layer);
+	prefill_block_end(p, p.d_parts, Ld.mpost, m->rmsw, true, false);
+	TG_HIP(hipGetLastError());
+	TG_HIP(hipMemcpyAsync(x, p.x, bytes, hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+
+int tg_block_lm_head(tg_session *s, const float *x, int rows, float *logits) {
+	if (int rc = block_args_ok(s, 0, x, rows)) return rc;
+	if (!logits) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	tg_model *m = s->m;
+	const int h = m->cfg.hidden_size;
+	// both branches take the last row (modules.hpp:232-246)
+	TG_HIP(hipMemcpyAsync(s->blk_x, x + (size_t)(rows - 1) * h, sizeof(float) * (size_t)h, hipMemcpyHostToDevice, g_stream));
+	if (rows == 1) {
+		launch_lmhead(s, s->zeros, m->rmsw, s->blk_x, nullptr);  // the decode step's kernel: final norm in its prologue
+	} else {
+		// the prefill's sequence: a row norm, then the LM head on the normalised row
+		tg_launch_norm_rows(s->blk_y, s->blk_x, 1, 0, m->rmsw, nullptr, nullptr, nullptr, 1, h, nullptr, nullptr, g_stream);
+		TgGemv g = gemv_base(m->lm);
+		g.x = s->blk_y;
+		g.y = s->logits;
+		g.blk_val = s->blk_val;
+		g.blk_idx = s->blk_idx;
+		tg_launch_gemv(g, TG_ROLE_LMHEAD_PLAIN, g_stream);
+	}
+	TG_HIP(hipGetLastError());
+	TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)m->cfg.n_vocab, hipMemcpyDeviceToHost, g_stream));
+	TG_HIP(hipStreamSynchronize(g_stream));
+	return TG_OK;
+}
+
 
 int tg_generate_greedy(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode, int32_t *out_ids, double *s_prefill,
                        double *s_decode) {
@@ -1537,7 +1848,8 @@ int tg_session_tap(tg_session *s, int b, float *out, int rows) {
 	TG_HIP(hipStreamSynchronize(g_stream));
 	const size_t h = (size_t)c.hidden_size;
 	if (s->taps) {
-		if (rows != s->tap_rows) return tg_fail(TG_ERR_BAD_ARG, "rows must equal the prompt length");
+		if (rows != s->tap_rows)
+			return tg_fail(TG_ERR_BAD_ARG, "rows must equal the prompt length (1 for a prompt of more than 1024 tokens: only its last row is kept)");
 		TG_HIP(hipMemcpy(out, s->taps + (size_t)b * s->tap_rows * h, sizeof(float) * (size_t)rows * h, hipMemcpyDeviceToHost));
 	} else {
 		if (rows != 1) return tg_fail(TG_ERR_BAD_ARG, "decode taps have one row");
