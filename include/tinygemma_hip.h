@@ -97,6 +97,15 @@ int tg_dev_copy(void *dst_dev, const void *src_dev, size_t bytes);
 int tg_qgemv_dev(float *y_dev, const float *x_dev, const tg_qweight *w, int logits_variant);
 /* C_dev[m][outDim] = scales * (A_dev[m][inDim] . W); asynchronous */
 int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m);
+/* No counterpart in the reference.  tg_qgemm_dev for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same bits, but the scratch of
+ * the int8 matrix path (three int8 digit planes of the activations + row factors) is a fixed array inside the
+ * library's device image instead of a buffer grown on demand.  It calls no hipMalloc / hipFree and sets nothing up:
+ * tg_init must have run.  Limit: (m rounded up to a multiple of 128) * inDim <= TG_QGEMM_STATIC_MAX_ELEMS, else
+ * TG_ERR_BAD_ARG.  All calls on a GPU share that one array: calls that overlap would race (the library's single
+ * stream orders them); every GPU the library runs on holds the array (about 6.1 MiB) until the process ends. */
+#define TG_QGEMM_STATIC_MAX_ELEMS (2 * 1024 * 1024)
+int tg_qgemm_dev_static(float *C_dev, const float *A_dev, const tg_qweight *w, int m);
 
 /* ---- model level --------------------------------------------------------------------------- */
 /* gemma::Transformer(Config), transformer.hpp:33 */

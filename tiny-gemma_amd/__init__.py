@@ -103,6 +103,7 @@ def lib():
     L.tg_session_read_ids.argtypes = [C.c_void_p, c_i32p, C.c_int, c_i32p]
     L.tg_session_tap.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_session_kv.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
+    L.tg_qgemm_dev_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_block_attention.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_block_mlp.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_block_lm_head.argtypes = [C.c_void_p, c_f32p, C.c_int, c_f32p]
@@ -209,6 +210,10 @@ class QWeight:
 
     def gemm(self, C_dev, A_dev, m):
         check(lib().tg_qgemm_dev(C_dev.p, A_dev.p, self.h, m))
+
+    def gemm_static(self, C_dev, A_dev, m):
+        """tg_qgemm_dev on the library's fixed scratch: allocates nothing."""
+        check(lib().tg_qgemm_dev_static(C_dev.p, A_dev.p, self.h, m))
 
     def free(self):
         if self.h:

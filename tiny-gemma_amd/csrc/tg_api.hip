@@ -332,6 +332,23 @@ int check_config(const tg_config *c) {
 }
 }  // namespace
 
+// ---- the entry point that allocates nothing --------------------------------------------------------------------
+// Scratch of the int8 matrix GEMM (digit planes of the activations + row factors) for callers that cannot allocate:
+// a fixed array in the library's device image.  Each GPU the library runs on holds it until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; kernels get g_static_scratch.
+#define TG_STATIC_ELEMS ((size_t)TG_QGEMM_STATIC_MAX_ELEMS)
+#define TG_STATIC_PLANE_BYTES (3 * TG_STATIC_ELEMS)
+#define TG_STATIC_ROWS (TG_STATIC_ELEMS / 256)  // the narrowest legal inDim is 256
+static __device__ __align__(256) unsigned char tg_static_scratch[TG_STATIC_PLANE_BYTES + 2 * TG_STATIC_ROWS * sizeof(float)];
+static unsigned char *g_static_scratch = nullptr;  // device address of tg_static_scratch on g_device (set by tg_init)
+
+static int static_scratch_init() {
+	void *p = nullptr;
+	TG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(tg_static_scratch)));
+	g_static_scratch = (unsigned char *)p;
+	return TG_OK;
+}
+
 extern "C" {
 
 // ---------------------------------------------------------------------------------------------
@@ -352,6 +369,7 @@ int tg_init(int device) {
 	g_n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	TG_HIP(hipStreamCreate(&g_stream));
 	if (g_gemm_resident_wgs > 0) g_gemm_resident_wgs = g_n_cu;
+	if (int rc = static_scratch_init()) return rc;
 	g_device = device;
 	g_inited = true;
 	return TG_OK;
@@ -486,6 +504,24 @@ int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 		}
 	}
 	launch_gemm(C_dev, A_dev, w->p.K, w->p, m, TG_EPI_STORE, nullptr, 0, 0, 0, g_apack, g_rowscale);
+	TG_HIP(hipGetLastError());
+	return TG_OK;
+}
+
+// tg_qgemm_dev on the fixed scratch above: no hipMalloc/hipFree, nothing set up on the way.  Calls share the one
+// array (the planes of the previous call are overwritten; nothing in it needs to start at zero), so calls that
+// overlap on one GPU would race: the library's single stream orders them.
+int tg_qgemm_dev_static(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
+	if (!g_inited || !g_static_scratch) return tg_fail(TG_ERR_STATE, "tg_init has not run: this entry point sets nothing up itself");
+	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	if (g_gemm_mfma && !w->p.Wg) return tg_fail(TG_ERR_UNSUPPORTED_SHAPE, "no MFMA tiling was built for this matrix (outDim too large)");
+	const size_t rows = tg_gemm_mfma_rows(m);
+	if (rows * (size_t)w->p.K > TG_STATIC_ELEMS)
+		return tg_fail(TG_ERR_BAD_ARG, "m (rounded up to a multiple of 128) x inDim exceeds TG_QGEMM_STATIC_MAX_ELEMS = " +
+		                                   std::to_string(TG_STATIC_ELEMS) + ": use tg_qgemm_dev");
+	// rows <= TG_STATIC_ELEMS / K <= TG_STATIC_ROWS, so the row factors fit behind the planes
+	launch_gemm(C_dev, A_dev, w->p.K, w->p, m, TG_EPI_STORE, nullptr, 0, 0, 0, (int8_t *)g_static_scratch,
+	            (float *)(g_static_scratch + TG_STATIC_PLANE_BYTES));
 	TG_HIP(hipGetLastError());
 	return TG_OK;
 }
