@@ -7,9 +7,14 @@ reference's README quotes its decode tok/s on (1024-token completions, mean prom
 Weights, KV cache and the prompt are resident in HBM before the timed region; nothing crosses
 PCIe inside it (each step feeds the device-side argmax of the previous one).
 
-Prints one JSON line.  `roofline` is for the dominant kernel of a step, the LM-head GEMV
-(tg_gemv_lmhead_argmax: 1152 x 262144 int8 + scales + x + logits = 304,091,648 algorithmic
-bytes per launch), timed with HIP events on the library's stream during real decode steps.
+Prints one JSON line.  `value` is steps / wall time of the one timed region; `decode_step.blocks` gives the
+same region cut into five blocks by HIP events (median and spread).  `roofline` is for the dominant kernel of a
+step, the LM-head GEMV (tg_gemv_lmhead_argmax: 1152 x 262144 int8 + scales + x + logits = 304,091,648
+algorithmic bytes per launch), timed with HIP events on the library's stream during real decode steps; its
+`traffic` is a constant taken from the committed counter profile named beside it, not measured by this run.
+`extra_rooflines` holds the same kind of statement for the decode attention launch and the prefill GEMM;
+`launch_floor` the cost of a dependent launch and of a device-wide barrier on this machine, and the same decode
+steps replayed from captured graphs.
 Reported beside it: `gemv_lmhead_shape` (the plain GEMV entry point tg_qgemv_dev at the same shape,
 launched back to back in rotation over three copies of the matrix so that none is served from cache), `gemv_640x2048` (the bare matvec of the first benchmark configuration, warm and
 rotating over 512 MB of distinct copies) and `prefill.long_prompt` (a 4096-token prefill of the same
@@ -32,6 +37,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as ge  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0   # dense int8 matrix rate
 # HBM bytes of one tg_gemv_lmhead_argmax launch from two `rocprofv3 --pmc` runs (FETCH_SIZE x 1.9999 +
 # WRITE_SIZE x 1.0000, both in KiB, scaled on a 256 MiB copy kernel): profiles/decode_1B_hbm_traffic.md
 LMHEAD_TRAFFIC_BYTES = {"1B": 304_494_817}
@@ -68,9 +74,50 @@ class HipEvents:
         return float(ms.value)
 
 
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(image_path, cfg_name, prompt, n_decode):
-    """Decode tok/s of the CPU path on one core: prefill the same prompt, then n_decode greedy steps."""
+    """Decode tok/s of the CPU path on one core: prefill the same prompt, then n_decode greedy steps.
+    The thread is pinned to the core it is running on for the duration of the sample."""
     orc = ge.load_oracle()
+    old_affinity, pinned = None, None
+    try:
+        old_affinity = os.sched_getaffinity(0)
+        cpu = None
+        try:
+            with open("/proc/self/stat") as f:
+                cpu = int(f.read().rsplit(")", 1)[1].split()[36])   # field 39: processor last run on
+        except (OSError, ValueError, IndexError):
+            pass
+        if cpu not in old_affinity:
+            cpu = min(old_affinity)
+        os.sched_setaffinity(0, {cpu})
+        pinned = cpu
+    except (AttributeError, OSError):
+        pass
+    try:
+        out = _cpu_baseline_run(orc, image_path, cfg_name, prompt, n_decode)
+    finally:
+        if old_affinity is not None:
+            try:
+                os.sched_setaffinity(0, old_affinity)
+            except OSError:
+                pass
+    out["pinned_to_cpu"] = pinned
+    out["host_cpu_model"] = host_cpu_model()
+    return out
+
+
+def _cpu_baseline_run(orc, image_path, cfg_name, prompt, n_decode):
     cfg = orc.named_config(cfg_name)
     if orc.Ref.available():
         kind, sess_model = "reference", orc.Ref().model(cfg, image_path)
@@ -123,7 +170,9 @@ def main():
     from tiny_gemma_amd import weights as tgw
 
     dev = tg.init(0)
-    tg.lib().tg_set_graphs(1 if args.graphs else 0)
+    if tg.lib().tg_set_graphs(1 if args.graphs else 0) != 0:
+        print("bench.py: " + tg.lib().tg_last_error().decode(), file=sys.stderr)
+        sys.exit(2)
     if args.prefetch_blocks is not None:
         tg.check(tg.lib().tg_set_prefetch_blocks(args.prefetch_blocks))
     if args.prefetch_plan is not None:
@@ -132,7 +181,7 @@ def main():
         tg.lib().tg_set_gemv_max_blocks(args.gemv_max_blocks)
     n_prompt, step_bytes, lm_bytes = MODELS[args.model]
     cfg = tg.named_config(args.model)
-    if n_prompt + args.warmup + args.steps + args.profile_steps + 1 > cfg.n_pos:
+    if n_prompt + args.warmup + args.steps + args.profile_steps + 600 > cfg.n_pos:
         print("bench.py: steps exceed the model's context (n_pos)", file=sys.stderr)
         sys.exit(2)
 
@@ -174,20 +223,27 @@ def main():
     e0, e1 = ev.create(), ev.create()
     sess.decode_enqueue(args.warmup)
     tg.synchronize()
-    # ---- timed region: exactly `steps` decode steps ----
-    ev.record(e0, stream)
+    # ---- timed region: exactly `steps` decode steps, enqueued in five blocks with an event between blocks (an event
+    # record does not wait for anything: the stream runs through) ----
+    n_blocks = 5 if args.steps >= 5 else 1
+    sizes = [args.steps // n_blocks + (1 if b < args.steps % n_blocks else 0) for b in range(n_blocks)]
+    marks = [ev.create() for _ in range(n_blocks + 1)]
     t0 = time.perf_counter()
-    sess.decode_enqueue(args.steps)
-    ev.record(e1, stream)
+    ev.record(marks[0], stream)
+    for b in range(n_blocks):
+        sess.decode_enqueue(sizes[b])
+        ev.record(marks[b + 1], stream)
     tg.synchronize()
     wall = time.perf_counter() - t0
-    gpu_ms = ev.elapsed_ms(e0, e1)
+    gpu_ms = ev.elapsed_ms(marks[0], marks[-1])
+    block_tok_s = sorted(sizes[b] / (1e-3 * ev.elapsed_ms(marks[b], marks[b + 1])) for b in range(n_blocks))
     ids = sess.read_ids(1 + args.warmup + args.steps)
     assert ids.size == 1 + args.warmup + args.steps and ids.min() >= 0
 
     # ---- per-kernel-class event timing over further real decode steps ----
     ms_sum = (C.c_double * 7)()
     launches = (C.c_int * 7)()
+    pos_profile = sess.position   # position of the first profiled step
     tg.check(tg.lib().tg_decode_profile(sess.h, args.profile_steps, ms_sum, launches))
     names = ["qkv", "attention", "oproj", "upgate_geglu", "down", "lmhead_argmax", "argmax_finish"]
     per_kernel_us = {n: 1e3 * ms_sum[i] / max(1, launches[i]) for i, n in enumerate(names)}
@@ -195,7 +251,6 @@ def main():
     achieved = lm_bytes / lm_s / 1e9
     # the same kernel re-launched 50x back to back on the session's buffers (dispatch latency amortised)
     L = tg.lib()
-    L.tg_debug_repeat_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
     tg.check(L.tg_debug_repeat_kernel(sess.h, 5, 0, 5))
     tg.synchronize()
     ev.record(e0, stream)
@@ -269,6 +324,80 @@ def main():
             "timing": f"HIP events around 200 launches on one matrix (warm) and one launch on each of {n_copies} distinct copies "
                       f"({n_copies * ci * cn >> 20} MB, cold); 1.3 MB per launch is launch-latency bound on this machine",
         }
+
+    # ---- the decode attention launch as a roofline statement: K and V rows of the valid keys, 2 KiB per key ----
+    n_local = sum(1 for l in range(cfg.n_layers) if l % cfg.window_pattern != cfg.window_pattern - 1)
+    n_global = cfg.n_layers - n_local
+    keys = [n_local * min(p + 1, cfg.n_pos_local) + n_global * min(p + 1, cfg.n_pos) for p in range(pos_profile, pos_profile + args.profile_steps)]
+    attn_bytes = 2 * 4 * cfg.head_dim * (sum(keys) / len(keys)) / cfg.n_layers
+    attn_us = per_kernel_us["attention"]
+    extra_rooflines = {
+        "attention_decode": {
+            "kernel": "attn_decode_kernel", "bound": "hbm", "unit": "GB/s", "peak": HBM_PEAK_GBS,
+            "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_us": attn_us, "achieved": attn_bytes / attn_us / 1e3,
+            "frac": attn_bytes / attn_us / 1e3 / HBM_PEAK_GBS,
+            "note": f"average over {n_local} local layers (ring of {cfg.n_pos_local} keys) and {n_global} global layers at positions "
+                    f"{pos_profile}..{pos_profile + args.profile_steps - 1}; 2*4*head_dim bytes per valid key; a launch over a few hundred "
+                    "keys is bound by its dependent steps (latency), not by bytes",
+        }
+    }
+
+    # ---- the prefill GEMM as a roofline statement: the up-projection-shaped product of a 4096-token prompt ----
+    if not args.headline_only and args.model == "1B":
+        gm, gk, gn = 4096, cfg.hidden_size, cfg.intermediate_size
+        grng = np.random.default_rng(7)
+        gw = tg.QWeight(grng.integers(-127, 128, (gk, gn), dtype=np.int8), grng.uniform(0.001, 0.02, gn).astype(np.float32))
+        ga = tg.DeviceBuffer.from_numpy(grng.standard_normal((gm, gk)).astype(np.float32))
+        gc = tg.DeviceBuffer(4 * gm * gn)
+        for _ in range(3):
+            gw.gemm(gc, ga, gm)
+        tg.synchronize()
+        ev.record(e0, stream)
+        for _ in range(20):
+            gw.gemm(gc, ga, gm)
+        ev.record(e1, stream)
+        tg.synchronize()
+        g_us = ev.elapsed_ms(e0, e1) * 1e3 / 20
+        g_flops = 2.0 * gm * gk * gn
+        extra_rooflines["prefill_gemm"] = {
+            "kernel": "gemm_i8_resident_kernel (+ row_scale_kernel, quant_pack_kernel)", "bound": "mfma", "unit": "TFLOP/s", "peak": INT8_PEAK_TOPS,
+            "shape": [gm, gk, gn], "algorithmic_flops_per_launch": g_flops, "avg_launch_us": g_us,
+            "achieved": g_flops / g_us / 1e6, "frac": g_flops / g_us / 1e6 / INT8_PEAK_TOPS,
+            "note": "tg_qgemm_dev, 20 back-to-back launches incl. the quantising pre-pass; algorithmic 2*M*K*N flops against the dense int8 "
+                    "rate; the matrix cores execute 3x that (three int8 digit planes of the activations)",
+        }
+        gw.free()
+        del ga, gc
+
+    # ---- what a dependent launch and a device-wide barrier cost here; the same steps replayed from captured graphs ----
+    launch_floor = None
+    if not args.headline_only:
+        us = C.c_double()
+        flag = C.c_int32()
+        launch_floor = {}
+        for wgs in (256, 512):
+            tg.check(L.tg_debug_launch_chain(2000, wgs, C.byref(us)))
+            launch_floor[f"dependent_launch_us_{wgs}wg"] = us.value
+        for wgs in (256, 64):
+            for fenced in (1, 0):
+                tg.check(L.tg_debug_grid_barrier(400, wgs, fenced, 1 << 16, C.byref(us), C.byref(flag)))
+                launch_floor[f"grid_barrier_us_{wgs}wg_{'fences' if fenced else 'atomic_data'}"] = None if flag.value else us.value
+        launch_floor["note"] = ("dependent_launch: 2000 back-to-back launches of a kernel that reads what the previous one wrote; grid_barrier: one "
+                                "resident kernel, per round 64 B published per workgroup + device-wide barrier + 64 B read from a workgroup on "
+                                "another XCD; fences = ordinary stores/loads + device-scope fences, atomic_data = the data moves through "
+                                "device-scope atomic accesses; null = a bounded wait gave up")
+        if not args.graphs and L.tg_set_graphs(1) == 0:
+            rates = {}
+            for mode in (1, 0):
+                L.tg_set_graphs(mode)
+                sess.decode_enqueue(8)
+                tg.synchronize()
+                ev.record(e0, stream)
+                sess.decode_enqueue(256)
+                ev.record(e1, stream)
+                tg.synchronize()
+                rates["graph_replay_tok_s" if mode else "stream_tok_s"] = 256 / (1e-3 * ev.elapsed_ms(e0, e1))
+            launch_floor.update(rates)
 
     # ---- long-prompt prefill (the matrix-matrix path) on a fresh session ----
     long_prefill = None
@@ -352,6 +481,8 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": LMHEAD_TRAFFIC_BYTES.get(args.model),
+            "traffic_source": "constant from profiles/decode_1B_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, scaled on a "
+                              "256 MiB copy kernel); not measured by this run",
             "algorithmic_bytes_per_launch": lm_bytes,
             "avg_launch_us": per_kernel_us["lmhead_argmax"],
             "timing": "HIP events around every launch of the kernel inside real decode steps (includes dispatch latency)",
@@ -372,8 +503,12 @@ def main():
                       "one copy, part of which the 256 MB memory-side cache still holds",
         },
         "gemv_640x2048": c1,
+        "extra_rooflines": extra_rooflines,
+        "launch_floor": launch_floor,
         "decode_step": {
             "gpu_ms_per_step_events": gpu_ms / args.steps,
+            "blocks": {"n": n_blocks, "tok_s_median": block_tok_s[len(block_tok_s) // 2], "tok_s_min": block_tok_s[0],
+                       "tok_s_max": block_tok_s[-1], "timing": "HIP events between the blocks of the timed region"},
             "weight_bytes_per_token": step_bytes,
             "weight_stream_GBps": step_bytes * tok_s / 1e9,
             "frac_of_hbm_roofline": step_bytes * tok_s / 1e9 / HBM_PEAK_GBS,

@@ -206,6 +206,16 @@ int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches)
  * times on the session's current buffers, back to back, without advancing the session: for timing one
  * kernel in isolation with events on tg_stream().  The kernels are idempotent on their inputs. */
 int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repeat);
+/* Timing probes of the machine facts the decode design rests on; no counterpart in the reference.
+ * tg_debug_launch_chain: n_launches dependent launches of a trivial kernel of `workgroups` x 256 threads (each reads what
+ * the previous one wrote) on tg_stream(): *us_per_launch = what one link of such a chain costs.
+ * tg_debug_grid_barrier: one resident kernel of `workgroups` workgroups (at most one per compute unit is meaningful)
+ * that runs `rounds` rounds of: publish 64 bytes, device-wide barrier, read a neighbour's 64 bytes.  fenced = 1:
+ * ordinary stores/loads made visible by device-scope fences; 0: the data itself moves through device-scope atomic
+ * accesses and no cache is written back or invalidated.  Every wait gives up after max_spins polls (*timed_out = 1:
+ * the figure is meaningless), so the kernel always ends. */
+int tg_debug_launch_chain(int n_launches, int workgroups, double *us_per_launch);
+int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins, double *us_per_barrier, int *timed_out);
 /* Host-side planning of a prefill, for inspection and tests; no counterpart in the reference, no GPU call.
  * tg_plan_attention_prefill: the work list of one attention layer of n_tokens on n_cu compute units, causal (window < 0)
  * or local (a query sees `window` keys before it and itself): *query_tile = query positions per workgroup; items =

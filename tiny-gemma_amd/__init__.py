@@ -14,7 +14,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libtinygemma_hip.so")
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip", "tg_repack.hip"]
+SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip", "tg_repack.hip", "tg_probe.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
                # leading scalar kernel arguments are preloaded into SGPRs by the dispatcher (no s_load round trip)
@@ -104,6 +104,10 @@ def lib():
     L.tg_session_tap.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_session_kv.argtypes = [C.c_void_p, C.c_int, c_f32p, c_f32p, c_i32p, c_i32p, c_i32p]
     L.tg_qgemm_dev_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.tg_debug_launch_chain.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+    L.tg_debug_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p]
+    L.tg_decode_profile.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double), c_i32p]
+    L.tg_debug_repeat_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
     L.tg_block_attention.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_block_mlp.argtypes = [C.c_void_p, C.c_int, c_f32p, C.c_int]
     L.tg_block_lm_head.argtypes = [C.c_void_p, c_f32p, C.c_int, c_f32p]

@@ -193,6 +193,8 @@ int tg_fail(int code, const std::string &msg) {
 	return code;
 }
 
+hipStream_t tg_probe_stream() { return g_inited ? g_stream : nullptr; }  // for the timing probes of tg_probe.hip
+
 struct tg_qweight {
 	PackedMat p;
 };
