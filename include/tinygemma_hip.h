@@ -163,6 +163,10 @@ int tg_generate(tg_session *s, const int32_t *prompt, int n_prompt, int n_decode
  * Refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
  * replayed graphs ended the process.  Captured graphs are dropped whenever a tuning knob changes. */
 int tg_set_graphs(int enable);
+/* 1 (default): inside one tg_decode_enqueue call the first launch of a step also finishes the previous step's greedy
+ * pick (second stage of the argmax, token log, counters), which saves one launch per token; 0: every step ends with
+ * its own finishing launch.  Same picks either way. */
+int tg_set_chain_picks(int enable);
 /* Debug taps of tg_forward_prefill (a copy of the residual stream after every block: every row of prompts of up
  * to 1024 tokens, the last row of longer ones; read back with tg_session_tap): off by default, they cost one
  * device copy per block. */

@@ -276,6 +276,33 @@ def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
             assert np.array_equal(a, b)
 
 
+def test_chained_picks_equal_a_finishing_launch_per_step(tg, oracle, weight_images, tables):
+    """Inside one tg_decode_enqueue call the first launch of a step finishes the previous step's greedy pick (second
+    stage of the argmax, token log, counters) instead of a launch of its own.  Same ids, same residual stream, same
+    counters as with a finishing launch per step; batches of 1 (nothing to chain), 2 and many; stepwise calls and
+    sampled steps in between."""
+    model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
+    results = []
+    try:
+        for chain in (0, 1):
+            tg.check(tg.lib().tg_set_chain_picks(chain))
+            sess.reset()
+            tok, _ = sess.prefill(prompt, want_logits=False)
+            for n in (1, 2, 17):
+                sess.decode_enqueue(n)
+            tok, _ = sess.decode(int(sess.read_ids(64)[-1]), want_logits=False)   # a stepwise call between batches
+            sess.decode_enqueue(5)
+            sess.decode_enqueue_sampled(3, 0.05, 1.0, np.array([0.3, 0.6, 0.9], np.float32))
+            sess.decode_enqueue(4)
+            tg.synchronize()
+            results.append((sess.read_ids(64).copy(), sess.taps(rows=1).copy(), sess.position, sess.kv(5)[2:]))
+    finally:
+        tg.check(tg.lib().tg_set_chain_picks(1))
+    (ids_a, taps_a, pos_a, ptr_a), (ids_b, taps_b, pos_b, ptr_b) = results
+    assert ids_a.size == 1 + 1 + 2 + 17 + 1 + 5 + 3 + 4 and np.array_equal(ids_a, ids_b)
+    assert np.array_equal(taps_a, taps_b) and pos_a == pos_b == prompt.size + 33 and ptr_a == ptr_b
+
+
 @pytest.mark.parametrize("n_prompt", [1000, 4100])
 def test_long_context_merge_path(tg, oracle, weight_images, tables, n_prompt):
     """More than 768 keys on a global layer: 32-key workgroups plus the merge launch, which folds groups of 64

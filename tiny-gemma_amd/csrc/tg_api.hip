@@ -40,6 +40,7 @@ char g_devname[256] = "";
 int g_n_cu = 256;
 bool g_gemm_split = true;       // prefill: products that would leave most compute units idle run in 2 or 4 parts of K
 int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
+bool g_chain_picks = true;  // inside a batch of greedy decode steps the next step's first launch finishes the previous pick
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 // Counts changes of the tuning knobs.  A captured decode step bakes the knobs of its capture into its launches
 // (prefetch workgroups, grid limits, attention geometry), so a session drops its captured graphs when this has moved.
@@ -303,6 +304,9 @@ struct tg_session {
 	// min-p sampling (allocated on first use): scratch of the three sampler launches and the caller's uniform draws
 	float *probs = nullptr, *seg = nullptr, *bsum = nullptr, *bmax = nullptr, *randf = nullptr;
 	int randf_cap = 0;
+	// The greedy pick of the last enqueued decode step exists only as the per-workgroup maxima of its LM-head launch:
+	// the first launch of the next step finishes it (and does the per-token bookkeeping), or flush_pick() does.
+	bool pick_pending = false;
 	bool sampling = false;  // decode steps enqueued now draw their token instead of taking the argmax
 	float s_minp = 1.0f, s_temp = 1.0f;
 	int rand_base = 0;      // token-log index of the token that uses randf[0]
@@ -925,6 +929,7 @@ int tg_session_reset(tg_session *s) {
 	TG_HIP(hipMemset(s->xr, 0, sizeof(float) * (size_t)(2 * c.n_layers + 1) * c.hidden_size));
 	TG_HIP(hipDeviceSynchronize());
 	s->pos = s->bp_local = s->bp_global = s->steps = 0;
+	s->pick_pending = false;
 	s->taps = nullptr;
 	s->tap_rows = 0;
 	return TG_OK;
@@ -998,6 +1003,14 @@ static void launch_qkv(tg_session *s, int l, bool embed, const float *pend, cons
 		g.wte = m->wte;
 		g.wte_scales = m->wte_scales;
 		g.tok = s->ctr + 4;
+		if (s->pick_pending) {  // this launch finishes the previous step's greedy pick
+			g.am_val = s->blk_val;
+			g.am_idx = s->blk_idx;
+			g.am_n = m->lm.ntiles;
+			g.am_ctr = s->ctr;
+			g.am_log = s->tok_log;
+			s->pick_pending = false;
+		}
 		g.vocab = c.n_vocab;
 		g.emb_scale = (float)sqrt((double)c.hidden_size);  // ops.hpp:586
 		tg_launch_gemv(g, TG_ROLE_QKV_EMBED, g_stream);
@@ -1108,7 +1121,16 @@ static void launch_lmhead(tg_session *s, const float *pend, const float *w_post,
 	tg_launch_gemv(g, TG_ROLE_LMHEAD, g_stream);
 }
 
-static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid, const StepOnly *only = nullptr) {
+// The finishing launch of a pending greedy pick (see tg_session::pick_pending).
+static void flush_pick(tg_session *s) {
+	if (!s->pick_pending) return;
+	tg_launch_argmax_finish(s->blk_val, s->blk_idx, s->m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
+	s->pick_pending = false;
+}
+
+// One decode step.  chain: the greedy pick may stay pending for the next step's first launch to finish (the caller
+// flushes after its last step); otherwise the step ends with the finishing launch.
+static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid, const StepOnly *only = nullptr, bool chain = false) {
 	if (int rc = session_usable(s)) return rc;
 	tg_model *m = s->m;
 	const tg_config &c = m->cfg;
@@ -1149,6 +1171,8 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		if (s->sampling)
 			tg_launch_minp(s->logits, c.n_vocab, s->s_minp, s->s_temp, s->randf, -1, s->rand_base, s->probs, s->seg, s->bsum, s->bmax,
 			               s->ctr, s->tok_log, 0, nullptr, g_stream);
+		else if (chain && !prof && !full_grid)
+			s->pick_pending = true;
 		else
 			tg_launch_argmax_finish(s->blk_val, s->blk_idx, m->lm.ntiles, s->ctr, s->tok_log, 1, g_stream);
 	}
@@ -1206,7 +1230,10 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 	}
 	for (int i = 0; i < n_steps; i++) {
 		if (!g_use_graphs) {
-			if (int rc = enqueue_decode_step(s, nullptr, false)) return rc;
+			if (int rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks)) {
+				flush_pick(s);
+				return rc;
+			}
 			continue;
 		}
 		// One HIP graph per attention launch geometry; every other launch parameter of a decode step
@@ -1239,6 +1266,8 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 			s->steps += 1;
 		}
 	}
+	flush_pick(s);
+	TG_HIP(hipGetLastError());
 	if (s->taps) {
 		TG_HIP(hipStreamSynchronize(g_stream));
 		s->taps = nullptr;
@@ -1353,6 +1382,11 @@ static bool profiler_attached() {
 		if (getenv(n) != nullptr) return true;
 	const char *pre = getenv("LD_PRELOAD");
 	return pre != nullptr && strstr(pre, "rocprof") != nullptr;
+}
+
+int tg_set_chain_picks(int enable) {
+	g_chain_picks = enable != 0;
+	return TG_OK;
 }
 
 int tg_set_graphs(int enable) {

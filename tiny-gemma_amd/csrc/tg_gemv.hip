@@ -88,6 +88,60 @@ __device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const f32x4 x
 	acc[3] = fmaf(xv.z, b2f(d3, 2), acc[3]); acc[3] = fmaf(xv.w, b2f(d3, 3), acc[3]);
 }
 
+// Second stage of the greedy argmax over n per-workgroup (maximum, index) pairs: every thread of the workgroup gets
+// the winner (ops.hpp:749-757: strict '>' from index 0, so the lowest index wins ties; no comparison is true for a
+// row of NaN and the index stays at the reference's initial -1).  s_bv / s_bi: NWAVE entries of LDS.
+__device__ __forceinline__ int argmax_pairs(const float *blk_val, const int *blk_idx, int n, float *s_bv, int *s_bi) {
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+	float bv = -INFINITY;
+	int bi = 0x7fffffff;
+	// all loads first (clamped indices, no branches), then the comparisons: one memory round trip instead of one per pass
+	for (int i0 = 0; i0 < n; i0 += 8 * NT) {
+		float ovs[8];
+		int ois[8];
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			const int i = i0 + u * NT + tid, ic = i < n ? i : n - 1;
+			ovs[u] = blk_val[ic];
+			ois[u] = blk_idx[ic];
+		}
+#pragma unroll
+		for (int u = 0; u < 8; u++) {
+			const bool in = i0 + u * NT + tid < n;
+			if (in && (ovs[u] > bv || (ovs[u] == bv && ois[u] < bi))) { bv = ovs[u]; bi = ois[u]; }
+		}
+	}
+#define TG_STEP(O)                                                      \
+	{                                                                   \
+		const float ov = tg_red_partner<O>(bv);                         \
+		const int oi = tg_red_partner<O>(bi);                           \
+		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }     \
+	}
+	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
+#undef TG_STEP
+	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
+	__syncthreads();
+	bv = s_bv[0];
+	bi = s_bi[0];
+	for (int i = 1; i < NWAVE; i++)
+		if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
+	return bi == 0x7fffffff ? -1 : bi;
+}
+
+// Per-token bookkeeping once the pick is known: it becomes the next step's input token, is appended to the id log, and
+// KVCache::update_single's counters (decode.hpp:68-69) advance once per token.  One thread.
+__device__ __forceinline__ void record_pick(int tok, int *ctr, int *tok_log, int advance) {
+	ctr[4] = tok;
+	const int st = ctr[3];
+	tok_log[st] = tok;
+	ctr[3] = st + 1;
+	if (advance) {
+		ctr[0] += 1;
+		ctr[1] += 1;
+		ctr[2] += 1;
+	}
+}
+
 // DEPTH: 16-byte weight loads in flight per lane
 template <int PRO, int EPI, int AUX, int DEPTH>
 __device__ __forceinline__ void gemv_body(const TgGemv &g) {
@@ -210,7 +264,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		}
 		if (PRO == TG_PRO_EMBED) {
 			// ops.hpp:537-568: s[d] * (sqrt(hidden) * q)
-			int tok = *g.tok;
+			int tok;
+			if (g.am_val != nullptr) {  // the previous step's pick is finished here, by every workgroup for itself
+				tok = argmax_pairs(g.am_val, g.am_idx, g.am_n, s_bv[0], s_bi[0]);
+				if (blockIdx.x == 0 && tid == 0) record_pick(tok, g.am_ctr, g.am_log, 1);
+			} else {
+				tok = *g.tok;
+			}
 			tok = tok < 0 ? 0 : (tok >= g.vocab ? g.vocab - 1 : tok);
 			const int8_t *row = g.wte + (size_t)tok * h;
 #pragma unroll
@@ -436,56 +496,15 @@ TG_GEMV_KERNEL(tg_gemv_lmhead_argmax, TG_PRO_RESNORM, TG_EPI_LOGITS, TG_W_NT, TG
 TG_GEMV_KERNEL(tg_gemv_lmhead_plain, TG_PRO_PLAIN, TG_EPI_LOGITS, TG_W_NT, TG_DEPTH_STREAM)    // LM head on an already normalised vector (prefill)
 TG_GEMV_KERNEL(tg_gemv_plain_stream, TG_PRO_PLAIN, TG_EPI_STORE, TG_W_NT, TG_DEPTH_STREAM)     // stand-alone, for a matrix too large to stay cached
 
-// Second stage of the greedy argmax, and the per-token bookkeeping: the winning id becomes the
-// next step's input token, is appended to the id log, and KVCache::update_single's counters
-// (decode.hpp:68-69) advance once per token.
+// Second stage of the greedy argmax and the per-token bookkeeping as a launch of their own: after a prefill, at the
+// end of a batch of decode steps, and wherever the next launch is not the first projection of a decode step (which
+// otherwise does both itself).
 __global__ __launch_bounds__(NT) void tg_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log,
                                                        int advance) {
 	__shared__ float s_bv[NWAVE];
 	__shared__ int s_bi[NWAVE];
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-	float bv = -INFINITY;
-	int bi = 0x7fffffff;
-	// all loads first (clamped indices, no branches), then the comparisons: one memory round trip instead of one per pass
-	for (int i0 = 0; i0 < n; i0 += 8 * NT) {
-		float ovs[8];
-		int ois[8];
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			const int i = i0 + u * NT + tid, ic = i < n ? i : n - 1;
-			ovs[u] = blk_val[ic];
-			ois[u] = blk_idx[ic];
-		}
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			const bool in = i0 + u * NT + tid < n;
-			if (in && (ovs[u] > bv || (ovs[u] == bv && ois[u] < bi))) { bv = ovs[u]; bi = ois[u]; }
-		}
-	}
-#define TG_STEP(O)                                                      \
-	{                                                                   \
-		const float ov = tg_red_partner<O>(bv);                         \
-		const int oi = tg_red_partner<O>(bi);                           \
-		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }     \
-	}
-	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
-#undef TG_STEP
-	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
-	__syncthreads();
-	if (tid == 0) {
-		for (int i = 1; i < NWAVE; i++)
-			if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
-		if (bi == 0x7fffffff) bi = -1;  // all NaN: the reference's scan leaves -1 (ops.hpp:750)
-		ctr[4] = bi;
-		const int st = ctr[3];
-		tok_log[st] = bi;
-		ctr[3] = st + 1;
-		if (advance) {
-			ctr[0] += 1;
-			ctr[1] += 1;
-			ctr[2] += 1;
-		}
-	}
+	const int bi = argmax_pairs(blk_val, blk_idx, n, s_bv, s_bi);
+	if (threadIdx.x == 0) record_pick(bi, ctr, tok_log, advance);
 }
 
 }  // namespace

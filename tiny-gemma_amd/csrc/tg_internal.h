@@ -104,6 +104,13 @@ struct TgGemv {
 	const int8_t *wte;     // EMBED: [vocab][hidden] row-major int8 (reference layout)
 	const float *wte_scales;
 	const int *tok;        // EMBED: device token id (clamped to [0, vocab))
+	// EMBED, optional: the previous step's greedy pick is still pending as per-workgroup maxima of its LM-head launch.
+	// Every workgroup then finishes that argmax itself (am_n pairs) instead of reading *tok, and workgroup 0 does the
+	// per-token bookkeeping (token log, counters) that the finishing launch would have done.
+	const float *am_val;
+	const int *am_idx;
+	int am_n;
+	int *am_ctr, *am_log;
 	int vocab;
 	float emb_scale;       // EMBED: float(sqrt(hidden))
 	const int *pos;        // ATTN_MERGE: device counters (pos[0] = position of this token)
