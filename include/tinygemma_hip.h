@@ -185,8 +185,13 @@ int tg_set_gemm_resident(int enable);
 /* prefill attention: 1 (default) = bf16 matrix cores on three bf16 planes of every fp32 operand (six cross terms per
  * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), workgroups of 32 query positions
  * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;
- * 0 = fp32 matrix cores, workgroups of 16 */
+ * 3 = the same with 16 at any length; 0 = fp32 matrix cores, workgroups of 16 */
 int tg_set_attn_prefill_mode(int mode);
+/* prefill attention, bf16 modes: where the bf16 planes of K and V come from.  1 (default) = for prompts of 2048
+ * tokens or more a pre-pass splits the K and V rows of a layer once and stores every 32-key tile as the image of the
+ * attention kernel's LDS arrays, which the attention workgroups copy straight into LDS (shorter prompts: as 0);
+ * 2 = the same at any length; 0 = every workgroup splits the tiles it stages itself.  Same arithmetic, same bits. */
+int tg_set_attn_prefill_planes(int mode);
 /* tuning knob: a GEMV launch uses at most n workgroups, which then loop over column tiles (0: one per tile) */
 int tg_set_gemv_max_blocks(int n);
 /* tuning knob: extra workgroups per decode launch that pull the NEXT launch's weights out of HBM into

@@ -252,13 +252,17 @@ def _dense_rows(q, k, v, rows, is_sw, ctx):
     return out
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["fp32_mfma", "bf16x3", "bf16x3_32q"])
+@pytest.fixture(params=[(0, 1), (1, 1), (2, 1), (3, 2), (2, 2)], ids=["fp32_mfma", "bf16x3", "bf16x3_32q", "bf16x3_16q_planes", "bf16x3_32q_planes"])
 def attn_mode(tg, request):
-    """The fp32 matrix path, the split-bf16 path as launched by default, and the latter with 32-query workgroups
-    forced (what long prompts get)."""
-    tg.check(tg.lib().tg_set_attn_prefill_mode(request.param))
-    yield request.param
+    """The fp32 matrix path, the split-bf16 path as launched by default, the latter with 32-query workgroups forced
+    (what long prompts get), and both workgroup sizes fed from pre-split plane images at any length (what prompts of
+    2048 tokens and more get)."""
+    mode, planes = request.param
+    tg.check(tg.lib().tg_set_attn_prefill_mode(mode))
+    tg.check(tg.lib().tg_set_attn_prefill_planes(planes))
+    yield mode
     tg.check(tg.lib().tg_set_attn_prefill_mode(1))
+    tg.check(tg.lib().tg_set_attn_prefill_planes(1))
 
 
 @pytest.mark.parametrize("name", list(gi.ATTN_PREFILL_CASES))

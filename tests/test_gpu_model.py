@@ -359,9 +359,10 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
 
 @pytest.mark.parametrize("n_prompt", [90, 700, 2100])
 def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
-    """The three prefill attention kernels (fp32 matrix path with 16-query workgroups, split-bf16 with 16 and with
-    32) behind the same work lists and the same finishing launch: same id, logits within fp32 rounding of each
-    other.  700 tokens: local layers with their own (windowed) work list; 2100: the 32-query tile by default."""
+    """The prefill attention kernels (fp32 matrix path with 16-query workgroups, split-bf16 with 16 and with 32, the
+    latter two also fed from pre-split plane images) behind the same work lists and the same finishing launch: same
+    id, logits within fp32 rounding of each other.  700 tokens: local layers with their own (windowed) work list;
+    2100: plane images by default."""
     cfg = tg.named_config("270m", 2)
     model = tg.Transformer(cfg)
     model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 24))
@@ -369,15 +370,19 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
     prompt = gi.prompt_ids(36, n_prompt)
     out = {}
     try:
-        for mode in (1, 0, 2):
+        for mode, planes in ((1, 0), (0, 0), (2, 0), (3, 2), (2, 2)):
             tg.check(tg.lib().tg_set_attn_prefill_mode(mode))
+            tg.check(tg.lib().tg_set_attn_prefill_planes(planes))
             sess.reset()
-            out[mode] = sess.prefill(prompt)
+            out[(mode, planes)] = sess.prefill(prompt)
     finally:
         tg.check(tg.lib().tg_set_attn_prefill_mode(1))
-    for mode in (0, 2):
-        assert out[mode][0] == out[1][0]
-        assert normrel(out[mode][1], out[1][1]) < 2e-5
+        tg.check(tg.lib().tg_set_attn_prefill_planes(1))
+    for key in ((0, 0), (2, 0), (3, 2), (2, 2)):
+        assert out[key][0] == out[(1, 0)][0]
+        assert normrel(out[key][1], out[(1, 0)][1]) < 2e-5
+    # the plane images hold the same bf16 planes the staging code computes: not a bit differs
+    assert np.array_equal(out[(2, 2)][1], out[(2, 0)][1])
 
 
 def test_one_session_many_prompt_lengths(tg, oracle):

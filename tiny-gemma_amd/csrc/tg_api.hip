@@ -1317,8 +1317,14 @@ int tg_set_attn_merge_chunk(int keys) {
 }
 
 int tg_set_attn_prefill_mode(int mode) {
-	if (mode < 0 || mode > 2) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1 or 2");
+	if (mode < 0 || mode > 3) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1, 2 or 3");
 	g_attn_prefill_bf16x3 = mode;
+	return TG_OK;
+}
+
+int tg_set_attn_prefill_planes(int mode) {
+	if (mode < 0 || mode > 2) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1 or 2");
+	g_attn_prefill_planes = mode;
 	return TG_OK;
 }
 
@@ -1447,10 +1453,11 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	for (int hh = 0; hh < NH; hh++)
 		for (size_t t = 0; t < rows; t++) memcpy(&qr[(t * NH + hh) * HD], &q[((size_t)hh * rows + t) * HD], sizeof(float) * HD);
 	float *dq = nullptr, *dk = nullptr, *dv = nullptr, *dout = nullptr;
+	void *dplanes = nullptr;
 	AttnPlanDev plan;
 	auto done = [&](int rc) {
 		(void)hipStreamSynchronize(g_stream);
-		void *ps[] = {dq, dk, dv, dout};
+		void *ps[] = {dq, dk, dv, dout, dplanes};
 		for (void *p : ps)
 			if (p) (void)hipFree(p);
 		plan.release();
@@ -1460,12 +1467,14 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dout, sizeof(float) * rows * NH * HD);
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dk, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dv, sizeof(float) * rows * HD);
+	if (rc == TG_OK) rc = tg_dev_alloc(&dplanes, tg_attn_prefill_planes_bytes(S));
 	if (rc == TG_OK) rc = tg_copy_h2d(dq, qr.data(), sizeof(float) * rows * NH * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dk, k, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = plan.build(S, (is_sw && S > sw_context + 1) ? sw_context : -1);
 	if (rc != TG_OK) return done(rc);
-	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), g_n_cu, g_stream);
+	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), g_n_cu, g_stream, false,
+	                       dplanes);
 	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
 	rc = tg_copy_d2h(orow.data(), dout, sizeof(float) * rows * NH * HD);
 	if (rc != TG_OK) return done(rc);
@@ -1486,6 +1495,7 @@ struct PrefillCtx {
 	int *d_ids = nullptr;
 	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr, *amax = nullptr;
 	int8_t *apack = nullptr;
+	void *planes = nullptr;  // pre-split K/V plane images of the layer being processed (split-bf16 attention)
 	const TgAttnPrefillPlan *plan_global = nullptr, *plan_local = nullptr;
 	int o_parts = 1, d_parts = 1;
 	size_t tpart = 0;
@@ -1511,7 +1521,8 @@ int prefill_setup(tg_session *s, int n, PrefillCtx *ctx, bool with_taps) {
 	             o_apack = carve(g_gemm_mfma ? tg_gemm_mfma_apack_bytes(n, std::max(std::max(f, qo), h)) : 0),
 	             o_rs = carve(g_gemm_mfma ? sizeof(float) * 2 * tg_gemm_mfma_rows(n) : 0),
 	             o_amax = carve(g_gemm_mfma ? sizeof(float) * tg_gemm_mfma_rows(n) : 0),
-	             o_taps = carve(sizeof(float) * (size_t)(2 * L + 1) * (size_t)tap_rows * h);
+	             o_taps = carve(sizeof(float) * (size_t)(2 * L + 1) * (size_t)tap_rows * h),
+	             o_planes = carve(tg_attn_prefill_planes_bytes(n));
 	if (need > s->pf_ws_bytes) {
 		TG_HIP(hipStreamSynchronize(g_stream));
 		s->taps = nullptr;  // they live in the workspace
@@ -1536,6 +1547,7 @@ int prefill_setup(tg_session *s, int n, PrefillCtx *ctx, bool with_taps) {
 	ctx->hb = (float *)(ws + o_hb);
 	ctx->rowscale = (float *)(ws + o_rs);
 	ctx->apack = (int8_t *)(ws + o_apack);
+	ctx->planes = ws + o_planes;
 	ctx->amax = g_gemm_mfma ? (float *)(ws + o_amax) : nullptr;  // max|hb| per row, folded by the up|gate product
 	s->taps = tap_rows ? (float *)(ws + o_taps) : nullptr;
 	s->tap_rows = tap_rows;
@@ -1587,7 +1599,7 @@ void prefill_attention_launches(const PrefillCtx &p, int l) {
 	// attention (modules.hpp:123): local layers use sw_context = max_pos
 	const TgAttnPrefillPlan *lplan = Ld.is_sw ? p.plan_local : p.plan_global;
 	tg_launch_attn_prefill(p.ao, p.qkv, p.qkv + qo, p.qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, g_n_cu, g_stream,
-	                       p.pk);
+	                       p.pk, p.planes);
 	// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
 	if (p.pk) tg_launch_attn_prefill_finish(p.ao, n, qo, lplan, g_n_cu, p.apack, p.rowscale, g_stream);
 	// O (modules.hpp:127-128)

@@ -28,6 +28,7 @@
 #include "tg_internal.h"
 
 #include <algorithm>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -464,6 +465,311 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 }
 constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD);  // 96 KB
 
+// ---- the same kernel fed from pre-split planes by a producer wave ------------------------------------------------
+// In the kernel above every workgroup splits every K/V tile it uses into bf16 planes itself while staging it:
+// measured, that staging (conversions + LDS writes through registers) is a third of a tile's time, and a K/V element
+// is split again by each of the S/16 query tiles that see it.  Here a pre-pass (attn_planes_kernel) splits the K and V
+// rows of a layer once and stores every 32-key tile as the exact image of the LDS arrays Kb and Vb (48 KB each); the
+// attention workgroup then only copies images, with loads that write straight into LDS (no registers, no vector
+// ALU work).  The images are used one per phase in the order K(0), V(0), K(1), V(1), ... (scores of a tile, then its
+// P.V); LDS holds a ring of three of them (144 KB): every wave requests its share of image i + 2 when phase i starts,
+// into the buffer phase i - 1 has just released, so every copy has two phases to arrive.  One workgroup barrier per
+// phase keeps the waves in step.
+constexpr size_t PLANE_IMG = sizeof(bf16x8) * 3 * NT32 * TK * 4;  // bytes of a K image = bytes of a V image (48 KB)
+constexpr size_t PLANE_RING_BYTES = 3 * PLANE_IMG;
+static_assert(PLANE_IMG == sizeof(bf16x8) * 3 * 4 * HD, "K and V images have the same size");
+
+// One workgroup per 32-key tile: planes[tile] = K image, then V image.  Keys past S are written as zeros.
+__global__ __launch_bounds__(PNT) void attn_planes_kernel(unsigned char *planes, const float *k, const float *v, int S, int ldkv) {
+	const int tile = blockIdx.x, tid = threadIdx.x;
+	bf16x8 *Kimg = reinterpret_cast<bf16x8 *>(planes + (size_t)tile * 2 * PLANE_IMG);
+	bf16x8 *Vimg = reinterpret_cast<bf16x8 *>(planes + (size_t)tile * 2 * PLANE_IMG + PLANE_IMG);
+	// K: unit = (t, key, g): dims 32t + 8g .. + 7 of a key -> Kb[plane][t][key][g]
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		const int unit = tid + PNT * u, g = unit & 3, key = (unit >> 2) & 31, t = unit >> 7;
+		const int j = tile * TK + key;
+		float x[8];
+		const float *src = k + (size_t)(j < S ? j : S - 1) * ldkv + 32 * t + 8 * g;
+		const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + 4);
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			x[e] = j < S ? a[e] : 0.0f;
+			x[4 + e] = j < S ? b[e] : 0.0f;
+		}
+		const Planes pl = split8(x);
+		const size_t at = ((size_t)t * TK + key) * 4 + g;
+		Kimg[at] = pl.h;
+		Kimg[(size_t)NT32 * TK * 4 + at] = pl.m;
+		Kimg[(size_t)2 * NT32 * TK * 4 + at] = pl.l;
+	}
+	// V: unit = (g, dim): keys 4g .. 4g+3 and 16+4g .. 16+4g+3 at one dim -> Vb[plane][g][dim]
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		const int unit = tid + PNT * u, d = unit & 255, g = unit >> 8;
+		float x[8];
+#pragma unroll
+		for (int sl = 0; sl < 8; sl++) {
+			const int j = tile * TK + (sl < 4 ? 4 * g + sl : 12 + 4 * g + sl);
+			const float val = v[(size_t)(j < S ? j : S - 1) * ldkv + d];
+			x[sl] = j < S ? val : 0.0f;
+		}
+		const Planes pl = split8(x);
+		const size_t at = (size_t)g * HD + d;
+		Vimg[at] = pl.h;
+		Vimg[(size_t)4 * HD + at] = pl.m;
+		Vimg[(size_t)2 * 4 * HD + at] = pl.l;
+	}
+}
+
+// A wave's share of the copy of one 48 KB image into LDS: loads of 64 lanes x 16 bytes, each landing at
+// (wave-uniform base) + 16 * lane; the NW waves of a workgroup take every NW-th kilobyte.
+template <int NW>
+__device__ __forceinline__ void copy_image_to_lds(const unsigned char *img, unsigned char *lds, int lane, int w) {
+#pragma unroll
+	for (int c = 0; c < (int)(PLANE_IMG / 1024) / NW; c++)
+		__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + (size_t)(c * NW + w) * 1024 + 16 * lane),
+		                                 (__attribute__((address_space(3))) void *)(lds + (c * NW + w) * 1024), 16, 0, 0);
+}
+
+// LDS reads of the matrix operands as the instruction itself.  The compiler cannot tell which LDS bytes a load that
+// writes straight into LDS will touch, so before every LDS read it can see it waits for ALL such loads in flight,
+// which would serialise the copy of a later image with the work on the current one.  These reads it does not see;
+// the wait for them is lds_wait(), which names the registers so that it stays between the reads and their use.
+template <int OFF>
+__device__ __forceinline__ bf16x8 lds_read16(unsigned addr) {
+	bf16x8 r;
+	asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+	return r;
+}
+__device__ __forceinline__ void lds_wait(Planes &a, Planes &b) {
+	asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.h), "+v"(a.m), "+v"(a.l), "+v"(b.h), "+v"(b.m), "+v"(b.l));
+}
+__device__ __forceinline__ void lds_wait(Planes &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.h), "+v"(a.m), "+v"(a.l)); }
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
+	(f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+	static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+// byte offsets inside an image: Kb[plane][t][key][g], Vb[plane][g][dim], 16-byte elements
+constexpr int KOFF_PLANE = NT32 * TK * 4 * 16, KOFF_T = TK * 4 * 16, KOFF_HALF = 16 * 4 * 16;
+constexpr int VOFF_PLANE = 4 * HD * 16, VOFF_DT = 16 * 16;
+template <int T, int HF>
+__device__ __forceinline__ Planes read_k(unsigned kaddr) {
+	Planes f;
+	f.h = lds_read16<T * KOFF_T + HF * KOFF_HALF>(kaddr);
+	f.m = lds_read16<KOFF_PLANE + T * KOFF_T + HF * KOFF_HALF>(kaddr);
+	f.l = lds_read16<2 * KOFF_PLANE + T * KOFF_T + HF * KOFF_HALF>(kaddr);
+	return f;
+}
+template <int DT>
+__device__ __forceinline__ Planes read_v(unsigned vaddr) {
+	Planes f;
+	f.h = lds_read16<DT * VOFF_DT>(vaddr);
+	f.m = lds_read16<VOFF_PLANE + DT * VOFF_DT>(vaddr);
+	f.l = lds_read16<2 * VOFF_PLANE + DT * VOFF_DT>(vaddr);
+	return f;
+}
+
+// Same arguments and outputs as attn_prefill_bf16x3_kernel, except that K and V come as plane images (attn_planes_kernel).
+// Every wave computes (head = wave % 4, query group = wave / 4) and issues its share of the image copies.
+template <int QG>
+__global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o, const float *q, const unsigned char *planes, int S, int ldq,
+                                                                     int ldo, int is_sw, int window, const int4 *items, float *part_o,
+                                                                     float *part_ml) {
+	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // ring of three images
+	constexpr int BQ = 16 * QG, NW = 4 * QG;
+	constexpr int SHARE = (int)(PLANE_IMG / 1024) / NW;  // loads per wave and image: 12 or 6
+	static_assert(SHARE == 12 || SHARE == 6, "the wait counts below are written for these");
+
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, head = w & 3, qh = w >> 2, c = lane & 15, g = lane >> 4;
+	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * BQ, slot = -1;
+	int4 item = int4{0, 0, 0, -1};
+	if (items != nullptr) {
+		item = items[blockIdx.x];
+		q0 = item.x * BQ;
+		slot = item.w;
+	}
+	// whole tiles only: a local layer's range starts at the tile that holds its first key (earlier keys are masked)
+	int kb = (is_sw && q0 > window) ? ((q0 - window) / TK) * TK : 0;
+	int ke = (q0 + BQ < S) ? q0 + BQ : S;  // exclusive
+	if (items != nullptr) {
+		kb = item.y * TK;
+		ke = min(ke, item.z * TK);
+	}
+	const int ntiles = (ke - kb + TK - 1) / TK;
+	// image i (K of tile i / 2 for even i, V for odd i) is the i-th 48 KB piece of the tile sequence; it lives in buffer i % 3
+	const unsigned char *img0 = planes + (size_t)(kb / TK) * 2 * PLANE_IMG;
+	const int nimg = 2 * ntiles;
+
+	const int q0w = q0 + 16 * qh;  // first query of this wave's group
+	const int qpos = q0w + c;
+	const int qrow = qpos < S ? qpos : S - 1;
+	const int klo = is_sw ? qpos - window : 0;
+
+	// Q planes: qp[t] = dims 32t + 8g .. + 7 of query c, scaled by 1/sqrt(hd) (a power of two: commutes with the split)
+	Planes qp[NT32];
+	{
+		const float *qsrc = q + (size_t)qrow * ldq + head * HD + 8 * g;
+#pragma unroll
+		for (int t = 0; t < NT32; t++) {
+			const f32x4 x0 = *reinterpret_cast<const f32x4 *>(qsrc + 32 * t), x1 = *reinterpret_cast<const f32x4 *>(qsrc + 32 * t + 4);
+			float x[8];
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				x[e] = x0[e] * 0.0625f;
+				x[4 + e] = x1[e] * 0.0625f;
+			}
+			qp[t] = split8(x);
+		}
+	}
+	f32x4 oacc[HD / 16];  // oacc[dt][i] = O[query 4 g + i][16 dt + c]
+#pragma unroll
+	for (int dt = 0; dt < HD / 16; dt++) oacc[dt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+	float m_run = -INFINITY, l_run = 0.0f;
+
+	// The Q loads have been consumed above: from here on the only loads this wave has in flight are image copies, in
+	// the order it issues them, so "at most SHARE outstanding" means "all but the youngest image's share have arrived".
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	copy_image_to_lds<NW>(img0, smem, lane, w);
+	copy_image_to_lds<NW>(img0 + PLANE_IMG, smem + PLANE_IMG, lane, w);
+	if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+	else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+	tg_lds_barrier();  // image 0 is complete
+
+	const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+	const unsigned k_lane = (unsigned)((c * 4 + g) * 16), v_lane = (unsigned)((g * HD + c) * 16);
+	int kbuf = 0;  // buffer of image 2 * tile; the V image follows in the next one, and the one after is free
+	for (int tile = 0; tile < ntiles; tile++) {
+		const int vbuf = kbuf == 2 ? 0 : kbuf + 1, fbuf = vbuf == 2 ? 0 : vbuf + 1;
+		const unsigned kaddr = lds0 + (unsigned)kbuf * (unsigned)PLANE_IMG + k_lane;
+		const unsigned vaddr = lds0 + (unsigned)vbuf * (unsigned)PLANE_IMG + v_lane;
+		// a tile that starts behind this group's last query holds none of its keys (the other group still needs it)
+		const bool mine = kb + tile * TK <= q0w + 15;
+
+		// ---- phase 2 * tile: scores.  Image 2 * tile + 2 (the next K) goes into the free buffer meanwhile ----
+		if (2 * tile + 2 < nimg) copy_image_to_lds<NW>(img0 + (size_t)(2 * tile + 2) * PLANE_IMG, smem + fbuf * PLANE_IMG, lane, w);
+		f32x4 s0 = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+		if (mine) {
+			// the two groups of 16 keys; even and odd k steps in separate accumulators; the fragments of step t + 1 are
+			// requested before the matrix instructions of step t
+			f32x4 sa[2][2];
+#pragma unroll
+			for (int hf = 0; hf < 2; hf++) sa[hf][0] = sa[hf][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+			Planes ka = read_k<0, 0>(kaddr), kc = read_k<0, 1>(kaddr);
+			static_for<NT32>([&](auto tc) {
+				constexpr int t = decltype(tc)::value;
+				lds_wait(ka, kc);
+				const Planes a = ka, b = kc;
+				if constexpr (t + 1 < NT32) {
+					ka = read_k<t + 1, 0>(kaddr);
+					kc = read_k<t + 1, 1>(kaddr);
+				}
+				sa[0][t & 1] = mfma6(a, qp[t], sa[0][t & 1]);
+				sa[1][t & 1] = mfma6(b, qp[t], sa[1][t & 1]);
+			});
+			s0 = sa[0][0] + sa[0][1];
+			s1 = sa[1][0] + sa[1][1];
+		}
+		// this wave's share of image 2 * tile + 1 (issued one phase ago) has arrived once at most the share just issued is outstanding
+		if (2 * tile + 2 < nimg) {
+			if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+			else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+		} else {
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		}
+		tg_lds_barrier();  // the K image is released, the V image is complete
+
+		// ---- phase 2 * tile + 1: softmax and P.V.  Image 2 * tile + 3 (the next V) goes into the buffer the K image has left ----
+		if (2 * tile + 3 < nimg) copy_image_to_lds<NW>(img0 + (size_t)(2 * tile + 3) * PLANE_IMG, smem + kbuf * PLANE_IMG, lane, w);
+		if (mine) {
+			Planes va = read_v<0>(vaddr);  // in flight during the softmax
+			const int j0 = kb + tile * TK + 4 * g;
+			float tmax = -INFINITY;
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				const int ja = j0 + i, jb = j0 + 16 + i;
+				if (ja > qpos || ja < klo) s0[i] = -INFINITY;
+				if (jb > qpos || jb < klo) s1[i] = -INFINITY;
+				tmax = fmaxf(tmax, fmaxf(s0[i], s1[i]));
+			}
+			tmax = fmaxf(tmax, tg_red_partner<16>(tmax));
+			tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
+			const float m_new = fmaxf(m_run, tmax);
+			const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // no valid key yet (see the fp32 kernel)
+			const float alpha = expf(m_run - m_ref);
+			float psum = 0.0f;
+			float pv[8];  // the lane's 8 key slots: keys 4g + i, then 16 + 4g + i
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				pv[i] = expf(s0[i] - m_ref);
+				pv[4 + i] = expf(s1[i] - m_ref);
+				psum += pv[i] + pv[4 + i];
+			}
+			psum += tg_red_partner<16>(psum);
+			psum += tg_red_partner<32>(psum);
+			l_run = fmaf(l_run, alpha, psum);
+			m_run = m_new;
+			float ar[4];
+#pragma unroll
+			for (int i = 0; i < 4; i++) ar[i] = __shfl(alpha, 4 * g + i, 64);
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) {
+#pragma unroll
+				for (int i = 0; i < 4; i++) oacc[dt][i] *= ar[i];
+			}
+			// ---- O += P V ----
+			const Planes pp = split8(pv);
+			static_for<HD / 16>([&](auto dc) {
+				constexpr int dt = decltype(dc)::value;
+				lds_wait(va);
+				const Planes vf = va;
+				if constexpr (dt + 1 < HD / 16) va = read_v<dt + 1>(vaddr);
+				oacc[dt] = mfma6(pp, vf, oacc[dt]);
+			});
+		}
+		if (2 * tile + 3 < nimg) {
+			if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+			else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+		} else {
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		}
+		tg_lds_barrier();  // the V image is released, the next K image is complete
+		kbuf = fbuf;
+	}
+
+	if (slot >= 0) {
+		float *po = part_o + (size_t)slot * BQ * NH * HD;
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			float *op = po + ((size_t)(16 * qh + 4 * g + i) * NH + head) * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i];
+		}
+		if (g == 0) {
+			float *pm = part_ml + (((size_t)slot * BQ + 16 * qh + c) * NH + head) * 2;
+			pm[0] = m_run;
+			pm[1] = l_run;
+		}
+		return;
+	}
+	float lr[4];
+#pragma unroll
+	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int qo = q0w + 4 * g + i;
+		if (qo < S) {
+			float *op = o + (size_t)qo * ldo + head * HD + c;
+#pragma unroll
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+		}
+	}
+}
+
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
@@ -553,6 +859,13 @@ __global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o
 
 }  // namespace
 
+// split-bf16 path: K/V split into plane images once per layer and copied straight into LDS (1: for prompts of
+// TG_ATTN_PLANES_MIN_TOKENS tokens or more, where it pays: measured break-even at ~1500 tokens, -8 % prefill time at
+// 2000; 2: always), or every workgroup splits what it stages (0)
+int g_attn_prefill_planes = 1;
+constexpr int TG_ATTN_PLANES_MIN_TOKENS = 2048;
+size_t tg_attn_prefill_planes_bytes(int S) { return (size_t)((S + TK - 1) / TK) * 2 * PLANE_IMG; }
+
 int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
 
 // Work list of a layer of S tokens, for tg_launch_attn_prefill: causal (window < 0) or local (a query sees the
@@ -613,11 +926,15 @@ size_t tg_attn_prefill_ml_floats(int nslots, int tq) { return (size_t)nslots * t
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
                             int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
-                            bool finish_later) {
+                            bool finish_later, void *planes_ws) {
 	(void)n_head;
 	(void)hd;
 	static bool lds_set = false;
 	if (g_attn_prefill_bf16x3 && !lds_set) {  // 96 KB of dynamic LDS needs the opt-in
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
+		                          (int)PLANE_RING_BYTES);
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
+		                          (int)PLANE_RING_BYTES);
 		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
 		                          (int)BF_LDS_BYTES);
 		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -629,7 +946,18 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	const dim3 grid(whole ? (unsigned)((S + tq - 1) / tq) : (unsigned)plan->nitems);
 	const int4 *items = whole ? nullptr : plan->items;
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
-	if (g_attn_prefill_bf16x3 && tq == 32)
+	const bool planes = g_attn_prefill_bf16x3 && planes_ws != nullptr &&
+	                    (g_attn_prefill_planes == 2 || (g_attn_prefill_planes == 1 && S >= TG_ATTN_PLANES_MIN_TOKENS));
+	if (planes) {
+		unsigned char *pw = (unsigned char *)planes_ws;
+		hipLaunchKernelGGL(attn_planes_kernel, dim3((unsigned)((S + TK - 1) / TK)), dim3(PNT), 0, s, pw, k, v, S, ldkv);
+		if (tq == 32)
+			hipLaunchKernelGGL(attn_prefill_planes_kernel<2>, grid, dim3(512), PLANE_RING_BYTES, s, o, q, pw, S, ldq, ldo, is_sw, window, items,
+			                   po, pml);
+		else
+			hipLaunchKernelGGL(attn_prefill_planes_kernel<1>, grid, dim3(256), PLANE_RING_BYTES, s, o, q, pw, S, ldq, ldo, is_sw, window, items,
+			                   po, pml);
+	} else if (g_attn_prefill_bf16x3 && tq == 32)
 		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
 		                   window, items, po, pml);
 	else if (g_attn_prefill_bf16x3)

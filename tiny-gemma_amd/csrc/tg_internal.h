@@ -188,7 +188,11 @@ size_t tg_attn_prefill_part_floats(int nslots, int tq);
 size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
                             int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
-                            bool finish_later = false);
+                            bool finish_later = false, void *planes_ws = nullptr);
+// planes_ws: tg_attn_prefill_planes_bytes(S) bytes of scratch for the pre-split K/V plane images of the split-bf16 path
+// (null: every workgroup splits the tiles it stages itself)
+extern int g_attn_prefill_planes;
+size_t tg_attn_prefill_planes_bytes(int S);
 // The rows of o (S x 1024, 4 heads x 256) -> digit planes + row factors of the int8 MFMA GEMM, merging the partial
 // results of split query tiles on the way (instead of attn_prefill_merge_kernel + the two quantising launches);
 // tg_launch_attn_prefill must then have been called with finish_later = true
