@@ -117,8 +117,15 @@ def test_attention_work_list_covers_every_visible_key_exactly_once(pkg, S, windo
     assert sum(1 for chunks in per_tile.values() if len(chunks) > 1) == nsplit
     lengths = [int(te - tb) for _, tb, te, _ in items]
     assert lengths == sorted(lengths, reverse=True)
+    # every query tile cuts its key range at the same places (multiples of the chunk length from its first key tile),
+    # so that workgroups running side by side walk the same keys
+    full = max(int(te - tb) for qt, tb, te, slot in items if slot >= 0) if nsplit else 0
     for qt, chunks in per_tile.items():
         chunks.sort()
+        if len(chunks) > 1:
+            clen = chunks[0][1] - chunks[0][0]
+            assert all(c[1] - c[0] == clen for c in chunks[:-1]) and clen <= full
+            assert clen // 2 <= chunks[-1][1] - chunks[-1][0] < clen + (clen + 1) // 2
         assert all(a[1] == b[0] for a, b in zip(chunks, chunks[1:]))        # contiguous, disjoint
         assert (len(chunks) == 1) == (chunks[0][2] == -1)                     # whole tiles write the output themselves
         q_first, q_last = qt * tq, min(qt * tq + tq, S) - 1
@@ -127,8 +134,9 @@ def test_attention_work_list_covers_every_visible_key_exactly_once(pkg, S, windo
         assert (chunks[-1][1] - 1) * 32 <= q_last < chunks[-1][1] * 32        # ends at the key tile of the last query
     if nq < n_cu:
         # fewer query tiles than compute units: chains as short as the number of units allows (one item per unit);
-        # causal layers of long prompts keep their rule instead (about 8 items per unit, chunks of 16 key tiles or more)
-        assert len(items) <= n_cu or max(lengths) == 1 or (window < 0 and max(lengths) <= 16)
+        # causal layers of long prompts keep their rule instead (about 8 items per unit, chunks of 16 key tiles or more;
+        # a row's last chunk takes a remainder of less than half a chunk with it)
+        assert len(items) <= n_cu or max(lengths) == 1 or (window < 0 and max(lengths) < 24)
 
 
 def test_gemm_k_parts_rule(pkg):

@@ -42,7 +42,18 @@ constexpr int TK = 32;     // keys per LDS tile
 constexpr int LDS_LD = 260;
 constexpr int PNT = 256;
 
-// items == nullptr: workgroup b owns query tile gridDim.x - 1 - b and all its keys.
+// Query tile of workgroup b of a launch without a work list.  Causal layer: late tiles see the most keys and start
+// first.  Local layer (all tiles cost the same): workgroups go to the 8 XCDs round-robin, and XCD x takes a contiguous
+// run of tiles, so that the workgroups it runs side by side have nearly the same key window and find each other's K/V
+// tiles in its L2.
+__device__ __forceinline__ int plain_query_tile(int is_sw) {
+	const int n = (int)gridDim.x, b = (int)blockIdx.x;
+	if (!is_sw) return n - 1 - b;
+	const int x = b & 7, k = b >> 3, base = n >> 3, rem = n & 7;
+	return x * base + (x < rem ? x : rem) + k;
+}
+
+// items == nullptr: workgroup b owns query tile plain_query_tile() and all its keys.
 // items != nullptr (a work list, see tg_attn_prefill_plan): items[b] = {query tile, first key tile, end key tile, slot}; slot < 0: the
 // item is the whole key range of its query tile and writes o; else it writes part_o[slot][16][NH][HD] (un-normalised)
 // and part_ml[slot][16][NH][2] (running maximum, running sum).
@@ -54,7 +65,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 
 	const int tid = threadIdx.x, lane = tid & 63, head = tid >> 6, c = lane & 15, g = lane >> 4;
 	// late query tiles of a causal layer see the most keys: start them first
-	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TQ, slot = -1;
+	int q0 = plain_query_tile(is_sw) * TQ, slot = -1;
 	int4 item = int4{0, 0, 0, -1};
 	if (items != nullptr) {
 		item = items[blockIdx.x];
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 	constexpr int SU = 4 / QG;    // staging units per thread and operand
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, head = w & 3, qh = w >> 2, c = lane & 15, g = lane >> 4;
-	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * BQ, slot = -1;
+	int q0 = plain_query_tile(is_sw) * BQ, slot = -1;
 	int4 item = int4{0, 0, 0, -1};
 	if (items != nullptr) {
 		item = items[blockIdx.x];
@@ -586,7 +597,7 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 	static_assert(SHARE == 12 || SHARE == 6, "the wait counts below are written for these");
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, head = w & 3, qh = w >> 2, c = lane & 15, g = lane >> 4;
-	int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * BQ, slot = -1;
+	int q0 = plain_query_tile(is_sw) * BQ, slot = -1;
 	int4 item = int4{0, 0, 0, -1};
 	if (items != nullptr) {
 		item = items[blockIdx.x];
@@ -904,20 +915,34 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 	items.clear();
 	split.clear();
 	nslots = 0;
+	// Chunk boundaries are the same for every query tile (multiples of `chunk` key tiles, counted from the query tile's
+	// first key tile for local layers, whose windows all start differently): the workgroups that run next to each
+	// other then walk the same keys at the same time and find each other's K/V tiles in their XCD's L2.  A last chunk
+	// of less than half a chunk is merged into the one before it.
 	for (int qt = 0; qt < nq; qt++) {
-		const int t0 = first_tile(qt), nt = end_tile(qt) - t0, nc = (nt + chunk - 1) / chunk;
+		const int t0 = first_tile(qt), nt = end_tile(qt) - t0;
+		int nc = (nt + chunk - 1) / chunk;
+		if (nc > 1 && nt - (nc - 1) * chunk < (chunk + 1) / 2) nc--;
 		if (nc == 1) {
 			items.push_back(int4{qt, t0, t0 + nt, -1});
 			continue;
 		}
 		split.push_back(int4{qt, nslots, nc, 0});
-		for (int ch = 0; ch < nc; ch++) {  // equal chunks
-			const int tb = t0 + (int)((long)nt * ch / nc), te = t0 + (int)((long)nt * (ch + 1) / nc);
+		for (int ch = 0; ch < nc; ch++) {
+			const int tb = t0 + ch * chunk, te = ch + 1 == nc ? t0 + nt : tb + chunk;
 			items.push_back(int4{qt, tb, te, nslots++});
 		}
 	}
 	if (split.empty()) return false;
-	std::stable_sort(items.begin(), items.end(), [](const int4 &a, const int4 &b) { return a.z - a.y > b.z - b.y; });
+	// Workgroups go to the 8 XCDs round-robin in list order, and each XCD works through its share in order: sorted by
+	// key range first, the 32 workgroups an XCD runs at any time share a key range (causal layers) or neighbouring
+	// windows (local layers).  Longest items first (the full chunks all have one length), then by key range.
+	auto by_keys = [](const int4 &a, const int4 &b) {
+		if (a.z - a.y != b.z - b.y) return a.z - a.y > b.z - b.y;
+		if (a.y != b.y) return a.y < b.y;
+		return a.x < b.x;
+	};
+	std::stable_sort(items.begin(), items.end(), by_keys);
 	return true;
 }
 size_t tg_attn_prefill_part_floats(int nslots, int tq) { return (size_t)nslots * tq * NH * HD; }
