@@ -182,12 +182,18 @@ int tg_set_gemm_split(int enable);
 /* prefill, int8 matrix path: 1 (default) = one resident workgroup per compute unit walks its share of the output
  * tiles, the operand prefetch running on from one tile into the next; 0 = one workgroup per tile.  Same results. */
 int tg_set_gemm_resident(int enable);
-/* prefill attention: 1 (default) = bf16 matrix cores on three bf16 planes of every fp32 operand (six cross terms per
- * product, fp32 accumulation: fp32-level accuracy at 2.7x the fp32 matrix rate), workgroups of 32 query positions
+/* prefill attention: 1 (default) = 16-bit matrix cores on two fp16 or three bf16 planes of every fp32 operand (cross
+ * terms summed in fp32: fp32-level accuracy at several times the fp32 matrix rate), workgroups of 32 query positions
  * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;
  * 3 = the same with 16 at any length; 0 = fp32 matrix cores, workgroups of 16 */
 int tg_set_attn_prefill_mode(int mode);
-/* prefill attention, bf16 modes: where the bf16 planes of K and V come from.  1 (default) = for prompts of 2048
+/* prefill attention, modes 1-3: the operand format of the matrix products.  1 (default) = every fp32 operand as two fp16
+ * planes (x = h + l, 22 significant bits), three products per fp32 product; 0 = three bf16 planes, six products
+ * (24 bits).  The fp16 form runs half the matrix instructions; its operands must lie within +-65504 (q and k are
+ * RMS-normalised, p is a probability, v a projection of a normalised vector): a value outside makes the forward
+ * return TG_ERR_STATE instead of a wrong result, and the bf16 form, which has fp32's range, is the way out. */
+int tg_set_attn_prefill_format(int f16);
+/* prefill attention, modes 1-3: where the planes of K and V come from.  1 (default) = for prompts of 2048
  * tokens or more a pre-pass splits the K and V rows of a layer once and stores every 32-key tile as the image of the
  * attention kernel's LDS arrays, which the attention workgroups copy straight into LDS (shorter prompts: as 0);
  * 2 = the same at any length; 0 = every workgroup splits the tiles it stages itself.  Same arithmetic, same bits. */

@@ -252,17 +252,56 @@ def _dense_rows(q, k, v, rows, is_sw, ctx):
     return out
 
 
-@pytest.fixture(params=[(0, 1), (1, 1), (2, 1), (3, 2), (2, 2)], ids=["fp32_mfma", "bf16x3", "bf16x3_32q", "bf16x3_16q_planes", "bf16x3_32q_planes"])
+ATTN_MODES = {
+    # name: (kernel mode, planes mode, fp16 format)
+    "fp32_mfma": (0, 1, 1),
+    "f16x2": (1, 1, 1),                 # the default: two fp16 planes, 16- or 32-query workgroups by prompt length
+    "f16x2_32q": (2, 1, 1),
+    "f16x2_16q_planes": (3, 2, 1),      # fed from pre-split plane images at any length (what 2048 tokens and more get)
+    "f16x2_32q_planes": (2, 2, 1),
+    "bf16x3": (1, 1, 0),                # three bf16 planes, six products
+    "bf16x3_16q_planes": (3, 2, 0),
+    "bf16x3_32q_planes": (2, 2, 0),
+}
+
+
+@pytest.fixture(params=list(ATTN_MODES.values()), ids=list(ATTN_MODES))
 def attn_mode(tg, request):
-    """The fp32 matrix path, the split-bf16 path as launched by default, the latter with 32-query workgroups forced
-    (what long prompts get), and both workgroup sizes fed from pre-split plane images at any length (what prompts of
-    2048 tokens and more get)."""
-    mode, planes = request.param
-    tg.check(tg.lib().tg_set_attn_prefill_mode(mode))
-    tg.check(tg.lib().tg_set_attn_prefill_planes(planes))
+    """The fp32 matrix path and the split paths: both operand formats, both workgroup sizes, operands staged by the
+    workgroup or copied from pre-split plane images."""
+    mode, planes, f16 = request.param
+    L = tg.lib()
+    tg.check(L.tg_set_attn_prefill_mode(mode))
+    tg.check(L.tg_set_attn_prefill_planes(planes))
+    tg.check(L.tg_set_attn_prefill_format(f16))
     yield mode
-    tg.check(tg.lib().tg_set_attn_prefill_mode(1))
-    tg.check(tg.lib().tg_set_attn_prefill_planes(1))
+    tg.check(L.tg_set_attn_prefill_mode(1))
+    tg.check(L.tg_set_attn_prefill_planes(1))
+    tg.check(L.tg_set_attn_prefill_format(1))
+
+
+def test_attention_prefill_operand_outside_the_fp16_range_is_an_error(tg):
+    """The two-plane fp16 format cannot hold a value beyond +-65504: the call must fail, not return infinities; the
+    three-plane bf16 format takes the same input (fp32's range) and gives the dense float64 result."""
+    S = 70
+    q, k, v = gi.attn_prefill_inputs(S, 77)
+    v[5, 100] = 1.0e5
+    L = tg.lib()
+    try:
+        for planes in (1, 2):
+            tg.check(L.tg_set_attn_prefill_planes(planes))
+            with pytest.raises(tg.TgError) as e:
+                tg.attention_prefill(q, k, v, False, 512)
+            assert e.value.code == -7 and "65504" in str(e.value)
+        tg.check(L.tg_set_attn_prefill_format(0))
+        o = tg.attention_prefill(q, k, v, False, 512)
+        assert normrel(o, _dense_rows(q, k, v, np.arange(S), False, 512)) < 2e-6
+    finally:
+        tg.check(L.tg_set_attn_prefill_planes(1))
+        tg.check(L.tg_set_attn_prefill_format(1))
+    q[0, 3, 7] = np.nan                      # NaN in an operand is reported the same way
+    with pytest.raises(tg.TgError):
+        tg.attention_prefill(q, k, gi.attn_prefill_inputs(S, 77)[2], False, 512)
 
 
 @pytest.mark.parametrize("name", list(gi.ATTN_PREFILL_CASES))

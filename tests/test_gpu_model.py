@@ -359,9 +359,9 @@ def test_error_paths(tg, oracle, weight_images, tables, tmp_path):
 
 @pytest.mark.parametrize("n_prompt", [90, 700, 2100])
 def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
-    """The prefill attention kernels (fp32 matrix path with 16-query workgroups, split-bf16 with 16 and with 32, the
-    latter two also fed from pre-split plane images) behind the same work lists and the same finishing launch: same
-    id, logits within fp32 rounding of each other.  700 tokens: local layers with their own (windowed) work list;
+    """The prefill attention kernels (fp32 matrix path with 16-query workgroups; the split path with 16 and with 32,
+    staged or fed from pre-split plane images, in both operand formats) behind the same work lists and the same
+    finishing launch: same id, logits within fp32 rounding of each other.  700 tokens: local layers with their own (windowed) work list;
     2100: plane images by default."""
     cfg = tg.named_config("270m", 2)
     model = tg.Transformer(cfg)
@@ -369,20 +369,24 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
     sess = model.session(gsize=1 << 20)
     prompt = gi.prompt_ids(36, n_prompt)
     out = {}
+    L = tg.lib()
+    combos = [(1, 0, 1), (0, 0, 1), (2, 0, 1), (3, 2, 1), (2, 2, 1), (1, 0, 0), (2, 2, 0)]   # (kernel mode, planes, fp16 format)
     try:
-        for mode, planes in ((1, 0), (0, 0), (2, 0), (3, 2), (2, 2)):
-            tg.check(tg.lib().tg_set_attn_prefill_mode(mode))
-            tg.check(tg.lib().tg_set_attn_prefill_planes(planes))
+        for mode, planes, f16 in combos:
+            tg.check(L.tg_set_attn_prefill_mode(mode))
+            tg.check(L.tg_set_attn_prefill_planes(planes))
+            tg.check(L.tg_set_attn_prefill_format(f16))
             sess.reset()
-            out[(mode, planes)] = sess.prefill(prompt)
+            out[(mode, planes, f16)] = sess.prefill(prompt)
     finally:
-        tg.check(tg.lib().tg_set_attn_prefill_mode(1))
-        tg.check(tg.lib().tg_set_attn_prefill_planes(1))
-    for key in ((0, 0), (2, 0), (3, 2), (2, 2)):
-        assert out[key][0] == out[(1, 0)][0]
-        assert normrel(out[key][1], out[(1, 0)][1]) < 2e-5
-    # the plane images hold the same bf16 planes the staging code computes: not a bit differs
-    assert np.array_equal(out[(2, 2)][1], out[(2, 0)][1])
+        tg.check(L.tg_set_attn_prefill_mode(1))
+        tg.check(L.tg_set_attn_prefill_planes(1))
+        tg.check(L.tg_set_attn_prefill_format(1))
+    for key in combos[1:]:
+        assert out[key][0] == out[combos[0]][0]
+        assert normrel(out[key][1], out[combos[0]][1]) < 2e-5
+    # the plane images hold the same planes the staging code computes: not a bit differs
+    assert np.array_equal(out[(2, 2, 1)][1], out[(2, 0, 1)][1])
 
 
 def test_one_session_many_prompt_lengths(tg, oracle):
@@ -410,11 +414,13 @@ def test_one_session_many_prompt_lengths(tg, oracle):
 def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
     """A 100-token prompt: the down projection (K = 2048) runs in four parts of K over workgroups and the output
     projection (K = 1024) in two, the following norm adds the partial results.  Against the same prefill with the
-    products unsplit: same id, logits equal to fp32 rounding of the extra additions, and really a different path."""
+    products unsplit: same id, logits equal to fp32 rounding of the extra additions, and really a different path.
+    The GeLU table has 2^20 entries here: with the 1024-entry step table a rounding difference that moves one
+    activation across a bin edge shows as ~2e-4 in the logits, which would say nothing about the split."""
     cfg = tg.named_config("270m", 2)
     model = tg.Transformer(cfg)
     model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 23))
-    sess = model.session(gsize=1024)
+    sess = model.session(gsize=1 << 20)
     prompt = gi.prompt_ids(35, 100)
     out = []
     try:
@@ -425,7 +431,9 @@ def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
     finally:
         tg.check(tg.lib().tg_set_gemm_split(1))
     (tok_a, lg_a), (tok_b, lg_b) = out
-    assert tok_a == tok_b and normrel(lg_a, lg_b) < 2e-5
+    rel = normrel(lg_a, lg_b)
+    print(f"k parts vs unsplit: logits rel {rel:.2e}")
+    assert tok_a == tok_b and rel < 2e-5
     assert not np.array_equal(lg_a, lg_b)
 
 

@@ -181,6 +181,11 @@ TgPrefetch prefetch_of(const PackedMat &p) {
 	return f;
 }
 
+int attn_range_error() {
+	return tg_fail(TG_ERR_STATE, "prefill attention: a q, k or v value is NaN or lies outside the fp16 range (+-65504) of the two-plane operand format; "
+	                             "the result is not valid.  tg_set_attn_prefill_format(0) selects the three-plane bf16 format, which has fp32's range");
+}
+
 int upload_floats(float **dst, const float *src, size_t n) {
 	TG_HIP(hipMalloc((void **)dst, n * sizeof(float)));
 	TG_HIP(hipMemcpy(*dst, src, n * sizeof(float), hipMemcpyHostToDevice));
@@ -294,7 +299,8 @@ struct tg_session {
 	unsigned graph_epoch = 0; // g_knob_epoch the cached graphs were captured under
 	float *zeros = nullptr;   // [hidden] of 0: as the pending block output of a post-norm + residual prologue it adds nothing
 	float *blk_x = nullptr, *blk_y = nullptr;  // [hidden] input / output of the block-level entry points
-	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token
+	int *ctr = nullptr;       // device: [0] position_ptr, [1] buffer_ptr local, [2] buffer_ptr global, [3] step, [4] token,
+	                          // [5] set by the prefill attention when an operand does not fit its fp16 planes
 	int *tok_log = nullptr;
 	int tok_log_cap = 0;
 	int pos = 0, bp_local = 0, bp_global = 0, steps = 0;  // host mirrors
@@ -1322,6 +1328,11 @@ int tg_set_attn_prefill_mode(int mode) {
 	return TG_OK;
 }
 
+int tg_set_attn_prefill_format(int f16) {
+	g_attn_prefill_f16 = f16 != 0;
+	return TG_OK;
+}
+
 int tg_set_attn_prefill_planes(int mode) {
 	if (mode < 0 || mode > 2) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1 or 2");
 	g_attn_prefill_planes = mode;
@@ -1467,16 +1478,21 @@ int tg_attention_prefill(float *o, const float *q, const float *k, const float *
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dout, sizeof(float) * rows * NH * HD);
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dk, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = tg_dev_alloc((void **)&dv, sizeof(float) * rows * HD);
-	if (rc == TG_OK) rc = tg_dev_alloc(&dplanes, tg_attn_prefill_planes_bytes(S));
+	if (rc == TG_OK) rc = tg_dev_alloc(&dplanes, tg_attn_prefill_planes_bytes(S) + 256);  // + the range flag
 	if (rc == TG_OK) rc = tg_copy_h2d(dq, qr.data(), sizeof(float) * rows * NH * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dk, k, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = tg_copy_h2d(dv, v, sizeof(float) * rows * HD);
 	if (rc == TG_OK) rc = plan.build(S, (is_sw && S > sw_context + 1) ? sw_context : -1);
 	if (rc != TG_OK) return done(rc);
+	int *dflag = (int *)((unsigned char *)dplanes + tg_attn_prefill_planes_bytes(S));
+	if (hipMemsetAsync(dflag, 0, sizeof(int), g_stream) != hipSuccess) return done(tg_fail(TG_ERR_HIP, "hipMemsetAsync failed"));
 	tg_launch_attn_prefill(dout, dq, dk, dv, S, NH, HD, NH * HD, HD, NH * HD, is_sw ? 1 : 0, sw_context, plan.get(), g_n_cu, g_stream, false,
-	                       dplanes);
+	                       dplanes, dflag);
 	if (hipGetLastError() != hipSuccess) return done(tg_fail(TG_ERR_HIP, "attention launch failed"));
 	rc = tg_copy_d2h(orow.data(), dout, sizeof(float) * rows * NH * HD);
+	int hflag = 0;
+	if (rc == TG_OK) rc = tg_copy_d2h(&hflag, dflag, sizeof(int));
+	if (rc == TG_OK && hflag) rc = attn_range_error();
 	if (rc != TG_OK) return done(rc);
 	for (int hh = 0; hh < NH; hh++)
 		for (size_t t = 0; t < rows; t++) memcpy(&o[((size_t)hh * rows + t) * HD], &orow[(t * NH + hh) * HD], sizeof(float) * HD);
@@ -1599,7 +1615,7 @@ void prefill_attention_launches(const PrefillCtx &p, int l) {
 	// attention (modules.hpp:123): local layers use sw_context = max_pos
 	const TgAttnPrefillPlan *lplan = Ld.is_sw ? p.plan_local : p.plan_global;
 	tg_launch_attn_prefill(p.ao, p.qkv, p.qkv + qo, p.qkv + qo + hd, n, c.n_head, hd, nq, nq, qo, Ld.is_sw ? 1 : 0, mp, lplan, g_n_cu, g_stream,
-	                       p.pk, p.planes);
+	                       p.pk, p.planes, s->ctr + 5);
 	// with the int8 MFMA GEMM one launch merges split query tiles and writes the output projection's digit planes
 	if (p.pk) tg_launch_attn_prefill_finish(p.ao, n, qo, lplan, g_n_cu, p.apack, p.rowscale, g_stream);
 	// O (modules.hpp:127-128)
@@ -1681,10 +1697,11 @@ int tg_forward_prefill(tg_session *s, const int32_t *ids, int n, float *logits, 
 	s->steps = 1;
 	if (int rc = set_counters_after_prefill(s, n)) return rc;
 	if (logits) TG_HIP(hipMemcpyAsync(logits, s->logits, sizeof(float) * (size_t)c.n_vocab, hipMemcpyDeviceToHost, g_stream));
-	int32_t tok = -1;
-	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
+	int32_t tok_flag[2] = {-1, 0};
+	TG_HIP(hipMemcpyAsync(tok_flag, s->ctr + 4, 2 * sizeof(int), hipMemcpyDeviceToHost, g_stream));
 	TG_HIP(hipStreamSynchronize(g_stream));
-	if (argmax) *argmax = tok;
+	if (argmax) *argmax = tok_flag[0];
+	if (tok_flag[1]) return attn_range_error();
 	return TG_OK;
 }
 
@@ -1749,7 +1766,10 @@ int tg_block_attention(tg_session *s, int layer, float *x, int rows) {
 	prefill_block_end(p, p.o_parts, Ld.apost, Ld.mpre, false, false);
 	TG_HIP(hipGetLastError());
 	TG_HIP(hipMemcpyAsync(x, p.x, bytes, hipMemcpyDeviceToHost, g_stream));
-	return set_counters_after_prefill(s, rows);
+	int flag = 0;
+	TG_HIP(hipMemcpyAsync(&flag, s->ctr + 5, sizeof(int), hipMemcpyDeviceToHost, g_stream));
+	if (int rc = set_counters_after_prefill(s, rows)) return rc;  // synchronises
+	return flag ? attn_range_error() : TG_OK;
 }
 
 int tg_block_mlp(tg_session *s, int layer, float *x, int rows) {

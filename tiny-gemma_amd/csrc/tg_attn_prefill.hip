@@ -234,39 +234,86 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 // and 16 queries); Q is split once, P once per tile and wave.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-struct Planes {
-	bf16x8 h, m, l;
+// Operand formats of the split path.
+//   FmtBf16x3: three bf16 planes, six products, as described above.  bf16 has fp32's exponent range: no input can
+//              fall outside it.
+//   FmtF16x2 : x = h + l with h = fp16(x), l = fp16(x - h): 11 + 11 significant bits, three products (hh, hl, lh; the
+//              dropped ll is below 2^-22 of the product), half the matrix instructions and two thirds of the LDS traffic
+//              of the bf16 form.  The matrix cores take fp16 subnormals as they are (checked on the MI355X: 2^-24 x
+//              16384 summed 32 times gives 2^-5), so small values only lose what lies below 2^-25 in absolute terms;
+//              an element of magnitude 0.25 or more keeps 22 bits, i.e. 1.2e-7 relative, next to fp32's 6e-8.  The price
+//              is the range: an operand beyond +-65504 does not fit.  q and k are RMS-normalised (|x| <= 16 |1 + w|)
+//              and p lies in [0, 1]; v is a projection of a normalised vector.  The kernels track the largest
+//              magnitude they convert and raise a flag if it does not fit, which the forward turns into an error.
+struct FmtBf16x3 {
+	typedef bf16x8 vec;
+	typedef bf16x2 vec2;
+	static constexpr int NP = 3;
+	static constexpr float QSCALE = 0.0625f, SSCALE = 1.0f;  // 1/sqrt(head_dim) goes onto q before the split (exact: a power of two)
+	static constexpr bool RANGE_CHECK = false;
 };
-__device__ __forceinline__ Planes split8(const float *x) {
-	Planes o;
+struct FmtF16x2 {
+	typedef f16x8 vec;
+	typedef f16x2 vec2;
+	static constexpr int NP = 2;
+	static constexpr float QSCALE = 1.0f, SSCALE = 0.0625f;  // ... or onto the scores: q stays where fp16 resolves it best
+	static constexpr bool RANGE_CHECK = true;
+};
+constexpr float F16_MAX = 65504.0f;
+
+template <typename F>
+struct PlanesT {
+	typename F::vec p[F::NP];  // leading part, then the successive remainders
+};
+template <typename F>
+__device__ __forceinline__ PlanesT<F> split8(const float *x) {
+	PlanesT<F> o;
 #pragma unroll
 	for (int i = 0; i < 8; i += 2) {
-		const f32x2 v = {x[i], x[i + 1]};
-		const bf16x2 a = __builtin_convertvector(v, bf16x2);  // round to nearest even
-		const f32x2 r1 = v - __builtin_convertvector(a, f32x2);
-		const bf16x2 b = __builtin_convertvector(r1, bf16x2);
-		const f32x2 r2 = r1 - __builtin_convertvector(b, f32x2);
-		const bf16x2 c = __builtin_convertvector(r2, bf16x2);
-		o.h[i] = a[0];
-		o.h[i + 1] = a[1];
-		o.m[i] = b[0];
-		o.m[i + 1] = b[1];
-		o.l[i] = c[0];
-		o.l[i + 1] = c[1];
+		f32x2 r = {x[i], x[i + 1]};
+#pragma unroll
+		for (int pl = 0; pl < F::NP; pl++) {
+			const typename F::vec2 a = __builtin_convertvector(r, typename F::vec2);  // round to nearest even
+			o.p[pl][i] = a[0];
+			o.p[pl][i + 1] = a[1];
+			if (pl + 1 < F::NP) r = r - __builtin_convertvector(a, f32x2);  // exact
+		}
 	}
 	return o;
 }
-// acc += a . b with the six significant cross terms, smallest first
-__device__ __forceinline__ f32x4 mfma6(const Planes &a, const Planes &b, f32x4 acc) {
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.l, b.h, acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.l, acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.m, b.m, acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.m, b.h, acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.m, acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.h, b.h, acc, 0, 0, 0);
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+// acc += a . b with the significant cross terms, smallest first
+template <typename F>
+__device__ __forceinline__ f32x4 mfma_terms(const PlanesT<F> &a, const PlanesT<F> &b, f32x4 acc) {
+	if constexpr (F::NP == 3) {
+		acc = mfma16(a.p[2], b.p[0], acc);
+		acc = mfma16(a.p[0], b.p[2], acc);
+		acc = mfma16(a.p[1], b.p[1], acc);
+	}
+	acc = mfma16(a.p[1], b.p[0], acc);
+	acc = mfma16(a.p[0], b.p[1], acc);
+	acc = mfma16(a.p[0], b.p[0], acc);
 	return acc;
+}
+// largest magnitude among 8 values about to be converted (formats with a limited range only)
+template <typename F>
+__device__ __forceinline__ void track_range(unsigned &rmax, const float *x) {
+	// largest magnitude as a bit pattern: unsigned order is magnitude order, and every NaN sorts above infinity
+	if constexpr (F::RANGE_CHECK) {
+#pragma unroll
+		for (int i = 0; i < 8; i++) rmax = max(rmax, __float_as_uint(x[i]) & 0x7fffffffu);
+	}
+}
+template <typename F>
+__device__ __forceinline__ void report_range(unsigned rmax, int *range_flag) {
+	if constexpr (F::RANGE_CHECK) {
+		if (range_flag != nullptr && rmax > __float_as_uint(F16_MAX)) *range_flag = 1;  // too large, infinite or NaN
+	}
 }
 
 constexpr int NT32 = HD / 32;  // k steps of a score product
@@ -275,14 +322,17 @@ constexpr int NT32 = HD / 32;  // k steps of a score product
 // with its own four waves (heads).  QG = 2: a K/V tile is fetched, split and staged once for 32 queries x 4 heads,
 // and the two waves a SIMD then holds overlap each other's LDS reads, matrix and vector work; the launcher takes it
 // for prompts long enough to keep the compute units busy with such workgroups, else QG = 1.
-template <int QG>
-__global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
-                                                                 int ldkv, int ldo, int is_sw, int window, const int4 *items,
-                                                                 float *part_o, float *part_ml) {
+template <int QG, typename F>
+__global__ __launch_bounds__(256 * QG) void attn_prefill_split_kernel(float *o, const float *q, const float *k, const float *v, int S, int ldq,
+                                                                int ldkv, int ldo, int is_sw, int window, const int4 *items,
+                                                                float *part_o, float *part_ml, int *range_flag) {
+	typedef typename F::vec vec;
+	typedef PlanesT<F> Planes;
 	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 	// Kb[plane][t][key][g]: dims 32t + 8g .. + 7 of a key; Vb[plane][g][dim]: the 8 keys of group g at one dim
-	bf16x8(*Kb)[NT32][TK][4] = reinterpret_cast<bf16x8(*)[NT32][TK][4]>(smem);
-	bf16x8(*Vb)[4][HD] = reinterpret_cast<bf16x8(*)[4][HD]>(smem + sizeof(bf16x8) * 3 * NT32 * TK * 4);
+	vec(*Kb)[NT32][TK][4] = reinterpret_cast<vec(*)[NT32][TK][4]>(smem);
+	vec(*Vb)[4][HD] = reinterpret_cast<vec(*)[4][HD]>(smem + sizeof(vec) * F::NP * NT32 * TK * 4);
+	unsigned rmax = 0u;
 	constexpr int BQ = 16 * QG;   // query positions per workgroup
 	constexpr int SU = 4 / QG;    // staging units per thread and operand
 
@@ -343,10 +393,11 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 			float x[8];
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
-				x[e] = x0[e] * 0.0625f;
-				x[4 + e] = x1[e] * 0.0625f;
+				x[e] = x0[e] * F::QSCALE;
+				x[4 + e] = x1[e] * F::QSCALE;
 			}
-			qp[t] = split8(x);
+			track_range<F>(rmax, x);
+			qp[t] = split8<F>(x);
 		}
 	}
 
@@ -365,18 +416,18 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 				x[e] = kpre[u][0][e];
 				x[4 + e] = kpre[u][1][e];
 			}
-			const Planes pl = split8(x);
+			track_range<F>(rmax, x);
+			const Planes pl = split8<F>(x);
 			const int t = sk_t0 + 2 * QG * u;
-			Kb[0][t][sk_key][sk_g] = pl.h;
-			Kb[1][t][sk_key][sk_g] = pl.m;
-			Kb[2][t][sk_key][sk_g] = pl.l;
+#pragma unroll
+			for (int pn = 0; pn < F::NP; pn++) Kb[pn][t][sk_key][sk_g] = pl.p[pn];
 		}
 #pragma unroll
 		for (int u = 0; u < SU; u++) {
-			const Planes pl = split8(vpre[u]);
-			Vb[0][sv_g][64 * QG * u + sv_d] = pl.h;
-			Vb[1][sv_g][64 * QG * u + sv_d] = pl.m;
-			Vb[2][sv_g][64 * QG * u + sv_d] = pl.l;
+			track_range<F>(rmax, vpre[u]);
+			const Planes pl = split8<F>(vpre[u]);
+#pragma unroll
+			for (int pn = 0; pn < F::NP; pn++) Vb[pn][sv_g][64 * QG * u + sv_d] = pl.p[pn];
 		}
 		tg_lds_barrier();
 		if (tile + 1 < ntiles) fetch(tile + 1);  // in flight during the products
@@ -392,13 +443,12 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 #pragma unroll
 			for (int hf = 0; hf < 2; hf++) {
 				Planes kf;
-				kf.h = Kb[0][t][16 * hf + c][g];
-				kf.m = Kb[1][t][16 * hf + c][g];
-				kf.l = Kb[2][t][16 * hf + c][g];
-				sa[hf][t & 1] = mfma6(kf, qp[t], sa[hf][t & 1]);
+#pragma unroll
+				for (int pn = 0; pn < F::NP; pn++) kf.p[pn] = Kb[pn][t][16 * hf + c][g];
+				sa[hf][t & 1] = mfma_terms<F>(kf, qp[t], sa[hf][t & 1]);
 			}
 		}
-		f32x4 s0 = sa[0][0] + sa[0][1], s1 = sa[1][0] + sa[1][1];
+		f32x4 s0 = (sa[0][0] + sa[0][1]) * F::SSCALE, s1 = (sa[1][0] + sa[1][1]) * F::SSCALE;
 		// ---- mask + online softmax for query c ----
 		const int j0 = kb + tile * TK + 4 * g;
 		float tmax = -INFINITY;
@@ -435,17 +485,17 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 			for (int i = 0; i < 4; i++) oacc[dt][i] *= ar[i];
 		}
 		// ---- O += P V ----
-		const Planes pp = split8(pv);
+		const Planes pp = split8<F>(pv);
 #pragma unroll
 		for (int dt = 0; dt < HD / 16; dt++) {
 			Planes vf;
-			vf.h = Vb[0][g][16 * dt + c];
-			vf.m = Vb[1][g][16 * dt + c];
-			vf.l = Vb[2][g][16 * dt + c];
-			oacc[dt] = mfma6(pp, vf, oacc[dt]);
+#pragma unroll
+			for (int pn = 0; pn < F::NP; pn++) vf.p[pn] = Vb[pn][g][16 * dt + c];
+			oacc[dt] = mfma_terms<F>(pp, vf, oacc[dt]);
 		}
 	}
 
+	report_range<F>(rmax, range_flag);
 	if (slot >= 0) {
 		float *po = part_o + (size_t)slot * BQ * NH * HD;
 #pragma unroll
@@ -474,7 +524,10 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_bf16x3_kernel(float *o,
 		}
 	}
 }
-constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD);  // 96 KB
+template <typename F>
+constexpr size_t split_lds_bytes() {
+	return sizeof(typename F::vec) * F::NP * (NT32 * TK * 4 + 4 * HD);  // 96 KB with three planes, 64 KB with two
+}
 
 // ---- the same kernel fed from pre-split planes by a producer wave ------------------------------------------------
 // In the kernel above every workgroup splits every K/V tile it uses into bf16 planes itself while staging it:
@@ -486,15 +539,28 @@ constexpr size_t BF_LDS_BYTES = sizeof(bf16x8) * (3 * NT32 * TK * 4 + 3 * 4 * HD
 // P.V); LDS holds a ring of three of them (144 KB): every wave requests its share of image i + 2 when phase i starts,
 // into the buffer phase i - 1 has just released, so every copy has two phases to arrive.  One workgroup barrier per
 // phase keeps the waves in step.
-constexpr size_t PLANE_IMG = sizeof(bf16x8) * 3 * NT32 * TK * 4;  // bytes of a K image = bytes of a V image (48 KB)
-constexpr size_t PLANE_RING_BYTES = 3 * PLANE_IMG;
-static_assert(PLANE_IMG == sizeof(bf16x8) * 3 * 4 * HD, "K and V images have the same size");
+constexpr size_t PLANE_BYTES = 16 * NT32 * TK * 4;  // one plane of a K image = one plane of a V image (16 KB)
+static_assert(PLANE_BYTES == 16 * 4 * HD, "K and V images have the same size");
+template <typename F>
+constexpr size_t plane_img() {
+	return F::NP * PLANE_BYTES;  // bytes of a K image = bytes of a V image: 48 KB with three planes, 32 KB with two
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_in_flight() {  // until at most N of this wave's vector memory loads are outstanding
+	asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 // One workgroup per 32-key tile: planes[tile] = K image, then V image.  Keys past S are written as zeros.
-__global__ __launch_bounds__(PNT) void attn_planes_kernel(unsigned char *planes, const float *k, const float *v, int S, int ldkv) {
+template <typename F>
+__global__ __launch_bounds__(PNT) void attn_planes_kernel(unsigned char *planes, const float *k, const float *v, int S, int ldkv,
+                                                         int *range_flag) {
+	typedef typename F::vec vec;
+	typedef PlanesT<F> Planes;
+	constexpr size_t PLANE_IMG = plane_img<F>();
 	const int tile = blockIdx.x, tid = threadIdx.x;
-	bf16x8 *Kimg = reinterpret_cast<bf16x8 *>(planes + (size_t)tile * 2 * PLANE_IMG);
-	bf16x8 *Vimg = reinterpret_cast<bf16x8 *>(planes + (size_t)tile * 2 * PLANE_IMG + PLANE_IMG);
+	vec *Kimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * PLANE_IMG);
+	vec *Vimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * PLANE_IMG + PLANE_IMG);
+	unsigned rmax = 0u;
 	// K: unit = (t, key, g): dims 32t + 8g .. + 7 of a key -> Kb[plane][t][key][g]
 #pragma unroll
 	for (int u = 0; u < 4; u++) {
@@ -508,11 +574,11 @@ __global__ __launch_bounds__(PNT) void attn_planes_kernel(unsigned char *planes,
 			x[e] = j < S ? a[e] : 0.0f;
 			x[4 + e] = j < S ? b[e] : 0.0f;
 		}
-		const Planes pl = split8(x);
+		track_range<F>(rmax, x);
+		const Planes pl = split8<F>(x);
 		const size_t at = ((size_t)t * TK + key) * 4 + g;
-		Kimg[at] = pl.h;
-		Kimg[(size_t)NT32 * TK * 4 + at] = pl.m;
-		Kimg[(size_t)2 * NT32 * TK * 4 + at] = pl.l;
+#pragma unroll
+		for (int pn = 0; pn < F::NP; pn++) Kimg[(size_t)pn * NT32 * TK * 4 + at] = pl.p[pn];
 	}
 	// V: unit = (g, dim): keys 4g .. 4g+3 and 16+4g .. 16+4g+3 at one dim -> Vb[plane][g][dim]
 #pragma unroll
@@ -525,20 +591,21 @@ __global__ __launch_bounds__(PNT) void attn_planes_kernel(unsigned char *planes,
 			const float val = v[(size_t)(j < S ? j : S - 1) * ldkv + d];
 			x[sl] = j < S ? val : 0.0f;
 		}
-		const Planes pl = split8(x);
+		track_range<F>(rmax, x);
+		const Planes pl = split8<F>(x);
 		const size_t at = (size_t)g * HD + d;
-		Vimg[at] = pl.h;
-		Vimg[(size_t)4 * HD + at] = pl.m;
-		Vimg[(size_t)2 * 4 * HD + at] = pl.l;
+#pragma unroll
+		for (int pn = 0; pn < F::NP; pn++) Vimg[(size_t)pn * 4 * HD + at] = pl.p[pn];
 	}
+	report_range<F>(rmax, range_flag);
 }
 
 // A wave's share of the copy of one 48 KB image into LDS: loads of 64 lanes x 16 bytes, each landing at
 // (wave-uniform base) + 16 * lane; the NW waves of a workgroup take every NW-th kilobyte.
-template <int NW>
+template <int NW, int KB>
 __device__ __forceinline__ void copy_image_to_lds(const unsigned char *img, unsigned char *lds, int lane, int w) {
 #pragma unroll
-	for (int c = 0; c < (int)(PLANE_IMG / 1024) / NW; c++)
+	for (int c = 0; c < KB / NW; c++)
 		__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + (size_t)(c * NW + w) * 1024 + 16 * lane),
 		                                 (__attribute__((address_space(3))) void *)(lds + (c * NW + w) * 1024), 16, 0, 0);
 }
@@ -547,16 +614,19 @@ __device__ __forceinline__ void copy_image_to_lds(const unsigned char *img, unsi
 // writes straight into LDS will touch, so before every LDS read it can see it waits for ALL such loads in flight,
 // which would serialise the copy of a later image with the work on the current one.  These reads it does not see;
 // the wait for them is lds_wait(), which names the registers so that it stays between the reads and their use.
-template <int OFF>
-__device__ __forceinline__ bf16x8 lds_read16(unsigned addr) {
-	bf16x8 r;
+template <typename V, int OFF>
+__device__ __forceinline__ V lds_read16(unsigned addr) {
+	V r;
 	asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
 	return r;
 }
-__device__ __forceinline__ void lds_wait(Planes &a, Planes &b) {
-	asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.h), "+v"(a.m), "+v"(a.l), "+v"(b.h), "+v"(b.m), "+v"(b.l));
+__device__ __forceinline__ void lds_wait(PlanesT<FmtBf16x3> &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.p[0]), "+v"(a.p[1]), "+v"(a.p[2])); }
+__device__ __forceinline__ void lds_wait(PlanesT<FmtF16x2> &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.p[0]), "+v"(a.p[1])); }
+template <typename P>
+__device__ __forceinline__ void lds_wait(P &a, P &b) {  // LDS reads return in order: both have arrived after these two
+	lds_wait(a);
+	lds_wait(b);
 }
-__device__ __forceinline__ void lds_wait(Planes &a) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a.h), "+v"(a.m), "+v"(a.l)); }
 template <int... I, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
 	(f(std::integral_constant<int, I>{}), ...);
@@ -566,35 +636,36 @@ __device__ __forceinline__ void static_for(F &&f) {
 	static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 // byte offsets inside an image: Kb[plane][t][key][g], Vb[plane][g][dim], 16-byte elements
-constexpr int KOFF_PLANE = NT32 * TK * 4 * 16, KOFF_T = TK * 4 * 16, KOFF_HALF = 16 * 4 * 16;
-constexpr int VOFF_PLANE = 4 * HD * 16, VOFF_DT = 16 * 16;
-template <int T, int HF>
-__device__ __forceinline__ Planes read_k(unsigned kaddr) {
-	Planes f;
-	f.h = lds_read16<T * KOFF_T + HF * KOFF_HALF>(kaddr);
-	f.m = lds_read16<KOFF_PLANE + T * KOFF_T + HF * KOFF_HALF>(kaddr);
-	f.l = lds_read16<2 * KOFF_PLANE + T * KOFF_T + HF * KOFF_HALF>(kaddr);
+constexpr int KOFF_T = TK * 4 * 16, KOFF_HALF = 16 * 4 * 16, VOFF_DT = 16 * 16;
+template <typename F, int T, int HF>
+__device__ __forceinline__ PlanesT<F> read_k(unsigned kaddr) {
+	PlanesT<F> f;
+	f.p[0] = lds_read16<typename F::vec, T * KOFF_T + HF * KOFF_HALF>(kaddr);
+	f.p[1] = lds_read16<typename F::vec, (int)PLANE_BYTES + T * KOFF_T + HF * KOFF_HALF>(kaddr);
+	if constexpr (F::NP == 3) f.p[2] = lds_read16<typename F::vec, 2 * (int)PLANE_BYTES + T * KOFF_T + HF * KOFF_HALF>(kaddr);
 	return f;
 }
-template <int DT>
-__device__ __forceinline__ Planes read_v(unsigned vaddr) {
-	Planes f;
-	f.h = lds_read16<DT * VOFF_DT>(vaddr);
-	f.m = lds_read16<VOFF_PLANE + DT * VOFF_DT>(vaddr);
-	f.l = lds_read16<2 * VOFF_PLANE + DT * VOFF_DT>(vaddr);
+template <typename F, int DT>
+__device__ __forceinline__ PlanesT<F> read_v(unsigned vaddr) {
+	PlanesT<F> f;
+	f.p[0] = lds_read16<typename F::vec, DT * VOFF_DT>(vaddr);
+	f.p[1] = lds_read16<typename F::vec, (int)PLANE_BYTES + DT * VOFF_DT>(vaddr);
+	if constexpr (F::NP == 3) f.p[2] = lds_read16<typename F::vec, 2 * (int)PLANE_BYTES + DT * VOFF_DT>(vaddr);
 	return f;
 }
 
-// Same arguments and outputs as attn_prefill_bf16x3_kernel, except that K and V come as plane images (attn_planes_kernel).
+// Same arguments and outputs as attn_prefill_split_kernel, except that K and V come as plane images (attn_planes_kernel).
 // Every wave computes (head = wave % 4, query group = wave / 4) and issues its share of the image copies.
-template <int QG>
+template <int QG, typename F>
 __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o, const float *q, const unsigned char *planes, int S, int ldq,
                                                                      int ldo, int is_sw, int window, const int4 *items, float *part_o,
-                                                                     float *part_ml) {
+                                                                     float *part_ml, int *range_flag) {
+	typedef PlanesT<F> Planes;
 	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // ring of three images
-	constexpr int BQ = 16 * QG, NW = 4 * QG;
-	constexpr int SHARE = (int)(PLANE_IMG / 1024) / NW;  // loads per wave and image: 12 or 6
-	static_assert(SHARE == 12 || SHARE == 6, "the wait counts below are written for these");
+	constexpr size_t PLANE_IMG = plane_img<F>();
+	constexpr int BQ = 16 * QG, NW = 4 * QG, IMG_KB = (int)(PLANE_IMG / 1024);
+	constexpr int SHARE = IMG_KB / NW;  // loads per wave and image (12, 8, 6 or 4)
+	unsigned rmax = 0u;
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, head = w & 3, qh = w >> 2, c = lane & 15, g = lane >> 4;
 	int q0 = plain_query_tile(is_sw) * BQ, slot = -1;
@@ -631,10 +702,11 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 			float x[8];
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
-				x[e] = x0[e] * 0.0625f;
-				x[4 + e] = x1[e] * 0.0625f;
+				x[e] = x0[e] * F::QSCALE;
+				x[4 + e] = x1[e] * F::QSCALE;
 			}
-			qp[t] = split8(x);
+			track_range<F>(rmax, x);
+			qp[t] = split8<F>(x);
 		}
 	}
 	f32x4 oacc[HD / 16];  // oacc[dt][i] = O[query 4 g + i][16 dt + c]
@@ -645,10 +717,9 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 	// The Q loads have been consumed above: from here on the only loads this wave has in flight are image copies, in
 	// the order it issues them, so "at most SHARE outstanding" means "all but the youngest image's share have arrived".
 	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-	copy_image_to_lds<NW>(img0, smem, lane, w);
-	copy_image_to_lds<NW>(img0 + PLANE_IMG, smem + PLANE_IMG, lane, w);
-	if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-	else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+	copy_image_to_lds<NW, IMG_KB>(img0, smem, lane, w);
+	copy_image_to_lds<NW, IMG_KB>(img0 + PLANE_IMG, smem + PLANE_IMG, lane, w);
+	wait_loads_in_flight<SHARE>();
 	tg_lds_barrier();  // image 0 is complete
 
 	const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -662,7 +733,7 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 		const bool mine = kb + tile * TK <= q0w + 15;
 
 		// ---- phase 2 * tile: scores.  Image 2 * tile + 2 (the next K) goes into the free buffer meanwhile ----
-		if (2 * tile + 2 < nimg) copy_image_to_lds<NW>(img0 + (size_t)(2 * tile + 2) * PLANE_IMG, smem + fbuf * PLANE_IMG, lane, w);
+		if (2 * tile + 2 < nimg) copy_image_to_lds<NW, IMG_KB>(img0 + (size_t)(2 * tile + 2) * PLANE_IMG, smem + fbuf * PLANE_IMG, lane, w);
 		f32x4 s0 = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
 		if (mine) {
 			// the two groups of 16 keys; even and odd k steps in separate accumulators; the fragments of step t + 1 are
@@ -670,34 +741,33 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 			f32x4 sa[2][2];
 #pragma unroll
 			for (int hf = 0; hf < 2; hf++) sa[hf][0] = sa[hf][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-			Planes ka = read_k<0, 0>(kaddr), kc = read_k<0, 1>(kaddr);
+			Planes ka = read_k<F, 0, 0>(kaddr), kc = read_k<F, 0, 1>(kaddr);
 			static_for<NT32>([&](auto tc) {
 				constexpr int t = decltype(tc)::value;
 				lds_wait(ka, kc);
 				const Planes a = ka, b = kc;
 				if constexpr (t + 1 < NT32) {
-					ka = read_k<t + 1, 0>(kaddr);
-					kc = read_k<t + 1, 1>(kaddr);
+					ka = read_k<F, t + 1, 0>(kaddr);
+					kc = read_k<F, t + 1, 1>(kaddr);
 				}
-				sa[0][t & 1] = mfma6(a, qp[t], sa[0][t & 1]);
-				sa[1][t & 1] = mfma6(b, qp[t], sa[1][t & 1]);
+				sa[0][t & 1] = mfma_terms<F>(a, qp[t], sa[0][t & 1]);
+				sa[1][t & 1] = mfma_terms<F>(b, qp[t], sa[1][t & 1]);
 			});
-			s0 = sa[0][0] + sa[0][1];
-			s1 = sa[1][0] + sa[1][1];
+			s0 = (sa[0][0] + sa[0][1]) * F::SSCALE;
+			s1 = (sa[1][0] + sa[1][1]) * F::SSCALE;
 		}
 		// this wave's share of image 2 * tile + 1 (issued one phase ago) has arrived once at most the share just issued is outstanding
 		if (2 * tile + 2 < nimg) {
-			if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-			else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+			wait_loads_in_flight<SHARE>();
 		} else {
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 		}
 		tg_lds_barrier();  // the K image is released, the V image is complete
 
 		// ---- phase 2 * tile + 1: softmax and P.V.  Image 2 * tile + 3 (the next V) goes into the buffer the K image has left ----
-		if (2 * tile + 3 < nimg) copy_image_to_lds<NW>(img0 + (size_t)(2 * tile + 3) * PLANE_IMG, smem + kbuf * PLANE_IMG, lane, w);
+		if (2 * tile + 3 < nimg) copy_image_to_lds<NW, IMG_KB>(img0 + (size_t)(2 * tile + 3) * PLANE_IMG, smem + kbuf * PLANE_IMG, lane, w);
 		if (mine) {
-			Planes va = read_v<0>(vaddr);  // in flight during the softmax
+			Planes va = read_v<F, 0>(vaddr);  // in flight during the softmax
 			const int j0 = kb + tile * TK + 4 * g;
 			float tmax = -INFINITY;
 #pragma unroll
@@ -733,18 +803,17 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 				for (int i = 0; i < 4; i++) oacc[dt][i] *= ar[i];
 			}
 			// ---- O += P V ----
-			const Planes pp = split8(pv);
+			const Planes pp = split8<F>(pv);
 			static_for<HD / 16>([&](auto dc) {
 				constexpr int dt = decltype(dc)::value;
 				lds_wait(va);
 				const Planes vf = va;
-				if constexpr (dt + 1 < HD / 16) va = read_v<dt + 1>(vaddr);
-				oacc[dt] = mfma6(pp, vf, oacc[dt]);
+				if constexpr (dt + 1 < HD / 16) va = read_v<F, dt + 1>(vaddr);
+				oacc[dt] = mfma_terms<F>(pp, vf, oacc[dt]);
 			});
 		}
 		if (2 * tile + 3 < nimg) {
-			if (SHARE == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-			else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+			wait_loads_in_flight<SHARE>();
 		} else {
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 		}
@@ -752,6 +821,7 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 		kbuf = fbuf;
 	}
 
+	report_range<F>(rmax, range_flag);
 	if (slot >= 0) {
 		float *po = part_o + (size_t)slot * BQ * NH * HD;
 #pragma unroll
@@ -875,7 +945,9 @@ __global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o
 // 2000; 2: always), or every workgroup splits what it stages (0)
 int g_attn_prefill_planes = 1;
 constexpr int TG_ATTN_PLANES_MIN_TOKENS = 2048;
-size_t tg_attn_prefill_planes_bytes(int S) { return (size_t)((S + TK - 1) / TK) * 2 * PLANE_IMG; }
+size_t tg_attn_prefill_planes_bytes(int S) { return (size_t)((S + TK - 1) / TK) * 2 * plane_img<FmtBf16x3>(); }  // the larger format
+// split path: 1 (default) = two fp16 planes, three products; 0 = three bf16 planes, six products
+int g_attn_prefill_f16 = 1;
 
 int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
 
@@ -948,24 +1020,45 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 size_t tg_attn_prefill_part_floats(int nslots, int tq) { return (size_t)nslots * tq * NH * HD; }
 size_t tg_attn_prefill_ml_floats(int nslots, int tq) { return (size_t)nslots * tq * NH * 2; }
 
+namespace {
+// The launches of the split path in one operand format: plane images + copying kernel, or the staging kernel.
+template <typename F>
+void launch_split(dim3 grid, int tq, bool planes, float *o, const float *q, const float *k, const float *v, int S, int ldq, int ldkv, int ldo,
+                  int is_sw, int window, const int4 *items, float *po, float *pml, void *planes_ws, int *range_flag, hipStream_t s) {
+	static bool lds_set = false;
+	constexpr size_t ring = 3 * plane_img<F>(), staged = split_lds_bytes<F>();
+	if (!lds_set) {  // more than 64 KB of dynamic LDS needs the opt-in
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<1, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ring);
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<2, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ring);
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_split_kernel<1, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged);
+		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_split_kernel<2, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged);
+		lds_set = true;
+	}
+	if (planes) {
+		unsigned char *pw = (unsigned char *)planes_ws;
+		hipLaunchKernelGGL(attn_planes_kernel<F>, dim3((unsigned)((S + TK - 1) / TK)), dim3(PNT), 0, s, pw, k, v, S, ldkv, range_flag);
+		if (tq == 32)
+			hipLaunchKernelGGL((attn_prefill_planes_kernel<2, F>), grid, dim3(512), ring, s, o, q, pw, S, ldq, ldo, is_sw, window, items, po, pml,
+			                   range_flag);
+		else
+			hipLaunchKernelGGL((attn_prefill_planes_kernel<1, F>), grid, dim3(256), ring, s, o, q, pw, S, ldq, ldo, is_sw, window, items, po, pml,
+			                   range_flag);
+	} else if (tq == 32) {
+		hipLaunchKernelGGL((attn_prefill_split_kernel<2, F>), grid, dim3(512), staged, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items, po,
+		                   pml, range_flag);
+	} else {
+		hipLaunchKernelGGL((attn_prefill_split_kernel<1, F>), grid, dim3(256), staged, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items, po,
+		                   pml, range_flag);
+	}
+}
+}  // namespace
+
 // q/k/v: rows of S tokens (q already normalised and rotated, ldq floats apart; k, v ldkv apart); o [S][ldo]
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
                             int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
-                            bool finish_later, void *planes_ws) {
+                            bool finish_later, void *planes_ws, int *range_flag) {
 	(void)n_head;
 	(void)hd;
-	static bool lds_set = false;
-	if (g_attn_prefill_bf16x3 && !lds_set) {  // 96 KB of dynamic LDS needs the opt-in
-		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
-		                          (int)PLANE_RING_BYTES);
-		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_planes_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
-		                          (int)PLANE_RING_BYTES);
-		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
-		                          (int)BF_LDS_BYTES);
-		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_bf16x3_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
-		                          (int)BF_LDS_BYTES);
-		lds_set = true;
-	}
 	const bool whole = plan == nullptr;  // the caller passes the work list that fits the layer kind, or none
 	const int tq = tg_attn_prefill_query_tile(S, n_cu);  // a plan must have been built for this tile size
 	const dim3 grid(whole ? (unsigned)((S + tq - 1) / tq) : (unsigned)plan->nitems);
@@ -973,24 +1066,13 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
 	const bool planes = g_attn_prefill_bf16x3 && planes_ws != nullptr &&
 	                    (g_attn_prefill_planes == 2 || (g_attn_prefill_planes == 1 && S >= TG_ATTN_PLANES_MIN_TOKENS));
-	if (planes) {
-		unsigned char *pw = (unsigned char *)planes_ws;
-		hipLaunchKernelGGL(attn_planes_kernel, dim3((unsigned)((S + TK - 1) / TK)), dim3(PNT), 0, s, pw, k, v, S, ldkv);
-		if (tq == 32)
-			hipLaunchKernelGGL(attn_prefill_planes_kernel<2>, grid, dim3(512), PLANE_RING_BYTES, s, o, q, pw, S, ldq, ldo, is_sw, window, items,
-			                   po, pml);
-		else
-			hipLaunchKernelGGL(attn_prefill_planes_kernel<1>, grid, dim3(256), PLANE_RING_BYTES, s, o, q, pw, S, ldq, ldo, is_sw, window, items,
-			                   po, pml);
-	} else if (g_attn_prefill_bf16x3 && tq == 32)
-		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<2>, grid, dim3(512), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
-		                   window, items, po, pml);
-	else if (g_attn_prefill_bf16x3)
-		hipLaunchKernelGGL(attn_prefill_bf16x3_kernel<1>, grid, dim3(256), BF_LDS_BYTES, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw,
-		                   window, items, po, pml);
-	else
+	if (!g_attn_prefill_bf16x3)
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items,
 		                   po, pml);
+	else if (g_attn_prefill_f16)
+		launch_split<FmtF16x2>(grid, tq, planes, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items, po, pml, planes_ws, range_flag, s);
+	else
+		launch_split<FmtBf16x3>(grid, tq, planes, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items, po, pml, planes_ws, range_flag, s);
 	if (whole || finish_later) return;
 	hipLaunchKernelGGL(attn_prefill_merge_kernel, dim3((unsigned)(plan->nsplit * tq)), dim3(PNT), 0, s, o, S, ldo, plan->split,
 	                   plan->part_o, plan->part_ml, tq);

@@ -188,7 +188,9 @@ size_t tg_attn_prefill_part_floats(int nslots, int tq);
 size_t tg_attn_prefill_ml_floats(int nslots, int tq);
 void tg_launch_attn_prefill(float *o, const float *q, const float *k, const float *v, int S, int n_head, int hd, int ldq, int ldkv,
                             int ldo, int is_sw, int window, const TgAttnPrefillPlan *plan, int n_cu, hipStream_t s,
-                            bool finish_later = false, void *planes_ws = nullptr);
+                            bool finish_later = false, void *planes_ws = nullptr, int *range_flag = nullptr);
+// range_flag (device, may be null): set to 1 when an operand does not fit the fp16 planes of the split path
+extern int g_attn_prefill_f16;
 // planes_ws: tg_attn_prefill_planes_bytes(S) bytes of scratch for the pre-split K/V plane images of the split-bf16 path
 // (null: every workgroup splits the tiles it stages itself)
 extern int g_attn_prefill_planes;
