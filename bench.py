@@ -158,8 +158,9 @@ def main():
     ap.add_argument("--gemv-max-blocks", type=int, default=None, help="tuning knob: workgroups per GEMV launch (0 = one per tile)")
     ap.add_argument("--prefetch-blocks", type=int, default=None, help="tuning knob: weight-prefetch workgroups per launch")
     ap.add_argument("--prefetch-plan", type=int, default=None, help="tuning knob")
-    ap.add_argument("--counter-run", action="store_true",
-                    help="for rocprofv3 --pmc: prefill, a few decode steps and 4 launches of a 256 MiB copy kernel; no timing")
+    ap.add_argument("--counter-run", nargs="?", const="decode", default=None, choices=["decode", "gemm"],
+                    help="for rocprofv3 --pmc, no timing.  decode (default): prefill, a few decode steps and 4 launches of a "
+                         "256 MiB copy kernel; gemm: 4 launches of the prefill GEMM at 4096 x 1152 x 6912 and nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is single-GPU (batch-1 decode has no data parallelism to spread); run with --gpus 1",
@@ -181,6 +182,17 @@ def main():
         tg.lib().tg_set_gemv_max_blocks(args.gemv_max_blocks)
     n_prompt, step_bytes, lm_bytes = MODELS[args.model]
     cfg = tg.named_config(args.model)
+    if args.counter_run == "gemm":
+        gm, gk, gn = 4096, cfg.hidden_size, cfg.intermediate_size
+        grng = np.random.default_rng(7)
+        gw = tg.QWeight(grng.integers(-127, 128, (gk, gn), dtype=np.int8), grng.uniform(0.001, 0.02, gn).astype(np.float32))
+        ga = tg.DeviceBuffer.from_numpy(grng.standard_normal((gm, gk)).astype(np.float32))
+        gc = tg.DeviceBuffer(4 * gm * gn)
+        for _ in range(4):
+            gw.gemm(gc, ga, gm)
+        tg.synchronize()
+        print(json.dumps({"counter_run": "gemm", "shape": [gm, gk, gn], "launches": 4}))
+        return
     if n_prompt + args.warmup + args.steps + args.profile_steps + 600 > cfg.n_pos:
         print("bench.py: steps exceed the model's context (n_pos)", file=sys.stderr)
         sys.exit(2)
@@ -368,6 +380,25 @@ def main():
         }
         gw.free()
         del ga, gc
+        # what the integer matrix cores sustain when every compute unit issues nothing else (register operands, no
+        # memory traffic): 32 clocks per instruction always, but the clock the part holds depends on the operand values
+        cpm, mhz = C.c_double(), C.c_double()
+        ceiling = {}
+        for label, operands in (("zero", 0), ("int8_in_pm6", 2), ("uniform_int8", 1)):
+            tg.check(L.tg_debug_mfma_clock(256, 20000, operands, C.byref(cpm), C.byref(mhz)))
+            ceiling[label] = {"clocks_per_mfma": cpm.value, "clock_mhz": mhz.value,
+                              "TOPs": 1024 * 65536.0 / cpm.value * mhz.value / 1e6}
+        tg.check(L.tg_debug_mfma_clock(8, 20000, 1, C.byref(cpm), C.byref(mhz)))
+        ceiling["uniform_int8_8_workgroups_only"] = {"clocks_per_mfma": cpm.value, "clock_mhz": mhz.value}
+        pg = extra_rooflines["prefill_gemm"]
+        pg["mfma_ceiling"] = ceiling
+        pg["executed_TOPs"] = 3.0 * pg["achieved"]
+        pg["frac_of_sustained_int8_rate"] = 3.0 * pg["achieved"] / ceiling["uniform_int8"]["TOPs"]
+        pg["mfma_ceiling_note"] = ("tg_debug_mfma_clock: 256 workgroups x 4 waves issuing only v_mfma_i32_32x32x32_i8 on register operands; "
+                                   "TOPs = 1024 SIMDs x 65536 ops / clocks_per_mfma x clock.  With every compute unit busy the part lowers its "
+                                   "clock under the power limit, more so the more operand bits toggle: the nominal 5.0 POP/s needs 2.4 GHz, "
+                                   "which it only holds for all-zero operands or a mostly idle chip.  frac_of_sustained_int8_rate = executed "
+                                   "(3 x algorithmic) rate / the uniform_int8 figure")
 
     # ---- what a dependent launch and a device-wide barrier cost here; the same steps replayed from captured graphs ----
     launch_floor = None

@@ -231,6 +231,13 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
  * the figure is meaningless), so the kernel always ends. */
 int tg_debug_launch_chain(int n_launches, int workgroups, double *us_per_launch);
 int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins, double *us_per_barrier, int *timed_out);
+
+/* The rate the integer matrix cores sustain on this machine (no counterpart in the reference: measurement aid).
+ * `workgroups` x 4 waves issue nothing but v_mfma_i32_32x32x32_i8 on register operands for `iters` x 12 instructions
+ * each; operands: 0 = all zero, 1 = uniformly random int8, 2 = int8 in [-6, 6].  Returns the average shader clocks
+ * per instruction (32 when nothing stalls) and the average shader clock in MHz during the loop, which the part
+ * lowers under load depending on the operand values.  workgroups <= 4096, iters <= 2^20. */
+int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_per_mfma, double *clock_mhz);
 /* Host-side planning of a prefill, for inspection and tests; no counterpart in the reference, no GPU call.
  * tg_plan_attention_prefill: the work list of one attention layer of n_tokens on n_cu compute units, causal (window < 0)
  * or local (a query sees `window` keys before it and itself): *query_tile = query positions per workgroup; items =

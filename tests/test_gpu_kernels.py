@@ -341,3 +341,22 @@ def test_attention_prefill_short_prompts_cut_into_key_chunks(tg, attn_mode, S, c
         o = tg.attention_prefill(q, k, v, is_sw, ctx)
         assert np.isfinite(o).all()
         assert normrel(o, _dense_rows(q, k, v, rows, is_sw, ctx)) < 2e-6
+
+
+def test_machine_probes_return_sane_figures(tg):
+    """The three timing probes behind the C ABI run, end normally (every wait in them is bounded) and report figures
+    of the right order: a dependent launch costs microseconds, a barrier round did not time out, and the matrix cores
+    issue one 32x32x32 int8 instruction per 32 clocks at a clock between 1 and 2.6 GHz."""
+    import ctypes as C
+    L = tg.lib()
+    us, flag, cpm, mhz = C.c_double(), C.c_int32(), C.c_double(), C.c_double()
+    tg.check(L.tg_debug_launch_chain(200, 256, C.byref(us)))
+    assert 0.5 < us.value < 50.0
+    tg.check(L.tg_debug_grid_barrier(50, 64, 0, 1 << 16, C.byref(us), C.byref(flag)))
+    assert flag.value == 0 and 0.1 < us.value < 100.0
+    for operands in (0, 1, 2):
+        tg.check(L.tg_debug_mfma_clock(256, 2000, operands, C.byref(cpm), C.byref(mhz)))
+        print(f"mfma probe operands {operands}: {cpm.value:.2f} clocks per instruction at {mhz.value:.0f} MHz")
+        assert 31.9 < cpm.value < 36.0 and 1000.0 < mhz.value < 2600.0
+    assert L.tg_debug_mfma_clock(0, 10, 0, C.byref(cpm), C.byref(mhz)) == -4
+    assert L.tg_debug_mfma_clock(8, 10, 3, C.byref(cpm), C.byref(mhz)) == -4

@@ -1,7 +1,16 @@
-// Timing probes of the two machine facts the decode design rests on (tg_debug_launch_chain, tg_debug_grid_barrier):
-// what a dependent kernel launch costs on this part, and what a device-wide barrier inside one kernel costs.  A decode
-// step is a chain of ~130 small dependent launches; the alternative, one resident kernel per step with a barrier
-// wherever a launch boundary is now, only pays if the barrier is the cheaper of the two.
+// Timing probes of the machine facts the design rests on.
+//
+// tg_debug_launch_chain, tg_debug_grid_barrier: what a dependent kernel launch costs on this part, and what a
+// device-wide barrier inside one kernel costs.  A decode step is a chain of ~130 small dependent launches; the
+// alternative, one resident kernel per step with a barrier wherever a launch boundary is now, only pays if the
+// barrier is the cheaper of the two.
+//
+// tg_debug_mfma_clock: the rate the integer matrix cores really sustain.  The instruction rate is fixed (one
+// v_mfma_i32_32x32x32_i8 per 32 clocks and SIMD), the clock is not: with every compute unit issuing matrix
+// instructions the part runs into its power limit and lowers the shader clock, by an amount that depends on the
+// operand VALUES (how many bits toggle).  The probe runs nothing but matrix instructions on operands held in
+// registers (no memory traffic at all) and reports clocks per instruction and the clock itself, for operands that
+// are all zero, small, or uniformly random int8: the ceiling the prefill GEMM can be measured against.
 //
 // Every wait in here is bounded: a workgroup that does not see the others arrive within max_spins polls gives up,
 // sets a flag and goes on, so the kernel always drains.
@@ -61,6 +70,57 @@ __global__ __launch_bounds__(PNT) void grid_barrier_kernel(unsigned *counter, fl
 		}
 	}
 	if (tid < 16) sink[blockIdx.x * 16 + tid] = acc;
+}
+
+// Back-to-back matrix instructions on register operands: 12 independent accumulators (3 x 4, as in the GEMM's inner
+// step), 3 A and 4 B fragments per wave filled from a hash of (workgroup, thread, fragment).  operands: 0 = zero,
+// 1 = uniformly random bytes, 2 = bytes in [-6, 6].  out[2 b] = shader clocks, out[2 b + 1] = ticks of the constant
+// 100 MHz counter, both around the loop of workgroup b's first thread.
+__device__ __forceinline__ unsigned probe_hash(unsigned x) {
+	x ^= x >> 16;
+	x *= 0x7feb352du;
+	x ^= x >> 15;
+	x *= 0x846ca68bu;
+	x ^= x >> 16;
+	return x;
+}
+__global__ __launch_bounds__(PNT) void mfma_clock_kernel(long long *out, int *sink, int iters, int operands) {
+	typedef int i32x4 __attribute__((ext_vector_type(4)));
+	typedef int i32x16 __attribute__((ext_vector_type(16)));
+	i32x4 frag[7];
+#pragma unroll
+	for (int f = 0; f < 7; f++)
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			const unsigned h = probe_hash((((unsigned)blockIdx.x * PNT + threadIdx.x) * 7 + f) * 4 + e + 1u);
+			unsigned v = 0;
+			if (operands == 1) v = h;
+			if (operands == 2)
+				for (int b = 0; b < 4; b++) v |= (unsigned)(((int)((h >> (8 * b)) & 0xff) % 13 - 6) & 0xff) << (8 * b);
+			frag[f][e] = (int)v;
+		}
+	i32x16 acc[12];
+#pragma unroll
+	for (int i = 0; i < 12; i++)
+#pragma unroll
+		for (int e = 0; e < 16; e++) acc[i][e] = 0;
+	__syncthreads();
+	const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+	for (int it = 0; it < iters; it++) {
+#pragma unroll
+		for (int i = 0; i < 12; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[3 + (i & 3)], frag[i >> 2], acc[i], 0, 0, 0);
+	}
+	const long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+	int x = 0;
+#pragma unroll
+	for (int i = 0; i < 12; i++)
+#pragma unroll
+		for (int e = 0; e < 16; e++) x ^= acc[i][e];
+	if (x == 0x5a5a5a5a && iters < 0) sink[threadIdx.x] = x;  // keeps the loop alive; never taken
+	if (threadIdx.x == 0) {
+		out[2 * blockIdx.x] = c1 - c0;
+		out[2 * blockIdx.x + 1] = r1 - r0;
+	}
 }
 
 struct Timer {
@@ -157,6 +217,36 @@ int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins,
 	*timed_out = h_flag;
 	*us_per_barrier = (us_many - us_few) / rounds;
 	return TG_OK;
+}
+
+int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_per_mfma, double *clock_mhz) {
+	if (workgroups < 1 || workgroups > 4096 || iters < 1 || iters > (1 << 20) || operands < 0 || operands > 2 || !clocks_per_mfma || !clock_mhz)
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	hipStream_t s = tg_probe_stream();
+	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
+	long long *buf = nullptr;
+	TG_HIP(hipMalloc((void **)&buf, sizeof(long long) * 2 * (size_t)workgroups + sizeof(int) * PNT));
+	int *sink = (int *)(buf + 2 * (size_t)workgroups);
+	int rc = TG_OK;
+	// the clock settles over some hundred microseconds of load: the figures come from the last of three launches
+	for (int pass = 0; pass < 3; pass++) hipLaunchKernelGGL(mfma_clock_kernel, dim3((unsigned)workgroups), dim3(PNT), 0, s, buf, sink, iters, operands);
+	if (hipStreamSynchronize(s) != hipSuccess || hipGetLastError() != hipSuccess) rc = tg_fail(TG_ERR_HIP, "launch failed");
+	if (rc == TG_OK) {
+		std::vector<long long> h(2 * (size_t)workgroups);
+		if (hipMemcpy(h.data(), buf, sizeof(long long) * h.size(), hipMemcpyDeviceToHost) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+		double c = 0.0, r = 0.0;
+		for (int i = 0; i < workgroups; i++) {
+			c += (double)h[2 * (size_t)i];
+			r += (double)h[2 * (size_t)i + 1];
+		}
+		if (rc == TG_OK && r <= 0.0) rc = tg_fail(TG_ERR_STATE, "the constant-rate counter did not advance");
+		if (rc == TG_OK) {
+			*clocks_per_mfma = c / workgroups / ((double)iters * 12.0);
+			*clock_mhz = 100.0 * c / r;
+		}
+	}
+	(void)hipFree(buf);
+	return rc;
 }
 
 }  // extern "C"
