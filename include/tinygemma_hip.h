@@ -167,6 +167,9 @@ int tg_set_graphs(int enable);
  * pick (second stage of the argmax, token log, counters), which saves one launch per token; 0: every step ends with
  * its own finishing launch.  Same picks either way. */
 int tg_set_chain_picks(int enable);
+/* every tg_set_* knob back to its default (a test that fails between a set and its restore must not leak its
+ * setting into the tests after it) */
+int tg_reset_knobs(void);
 /* Debug taps of tg_forward_prefill (a copy of the residual stream after every block: every row of prompts of up
  * to 1024 tokens, the last row of longer ones; read back with tg_session_tap): off by default, they cost one
  * device copy per block. */

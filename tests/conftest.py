@@ -51,6 +51,17 @@ def tg():
     return mod
 
 
+@pytest.fixture(autouse=True)
+def _knobs_back_to_defaults(request):
+    """After every GPU test the library's tuning knobs are back at their defaults (taps on, as the `tg` fixture
+    sets them), whatever the test did or wherever it failed."""
+    yield
+    if "tg" in request.fixturenames:
+        lib = ge.load_package().lib()
+        lib.tg_reset_knobs()
+        lib.tg_set_taps(1)
+
+
 @pytest.fixture(scope="session")
 def weight_images(oracle):
     """Weight-file images of the test models, generated once per session by the seeded generator."""

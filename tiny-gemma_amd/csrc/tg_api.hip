@@ -1406,6 +1406,24 @@ int tg_set_chain_picks(int enable) {
 	return TG_OK;
 }
 
+int tg_reset_knobs() {
+	g_gemm_mfma = 1;
+	g_prefetch_plan = 0;
+	g_prefetch_blocks = 128;
+	g_gemv_max_blocks = 2048;
+	g_use_graphs = false;
+	g_gemm_split = true;
+	g_gemm_resident_wgs = g_n_cu;
+	g_attn_merge_chunk = 48;
+	g_attn_prefill_bf16x3 = 1;
+	g_attn_prefill_planes = 1;
+	g_attn_prefill_f16 = 1;
+	g_chain_picks = true;
+	g_keep_taps = false;
+	g_knob_epoch++;
+	return TG_OK;
+}
+
 int tg_set_graphs(int enable) {
 	if (enable && profiler_attached())
 		return tg_fail(TG_ERR_STATE, "graph replay is not available under a profiler (a kernel trace of replayed graphs ended the process); use plain launches");
