@@ -145,7 +145,13 @@ def test_gemm_k_parts_rule(pkg):
     assert f(178, 6912, 1152, 256) == 4      # few rows, 108 stages of K: 4 x 27
     assert f(178, 1024, 1152, 256) == 2      # 16 stages: 2 x 8
     assert f(100, 2048, 640, 256) == 4 and f(100, 1024, 640, 256) == 2
-    assert f(4096, 6912, 1152, 256) == 2     # 288 workgroups on 256 units: two half-K copies
-    assert f(4096, 1152, 6912, 256) == 1     # 18 stages do not split into whole pairs per half
-    assert f(8192, 6912, 1152, 256) == 1     # last round filled to 0.75
-    assert f(1000, 6912, 1152, 256) == 2
+    assert f(1000, 6912, 1152, 256) == 2     # 72 workgroups on 256 units: two half-K copies
+    assert f(4096, 6912, 1152, 256) == 1     # 288 tiles: taken by the kernel that runs two workgroups per unit, no split
+    try:                                     # the rule of the one-workgroup-per-unit kernels
+        assert pkg.lib().tg_set_gemm_lds(0) == 0
+        assert f(4096, 6912, 1152, 256) == 2     # 288 workgroups on 256 units: two half-K copies
+        assert f(4096, 1152, 6912, 256) == 1     # 18 stages do not split into whole pairs per half
+        assert f(8192, 6912, 1152, 256) == 1     # last round filled to 0.75
+        assert f(1000, 6912, 1152, 256) == 2
+    finally:
+        assert pkg.lib().tg_set_gemm_lds(2) == 0

@@ -381,6 +381,7 @@ int tg_init(int device) {
 	g_n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	TG_HIP(hipStreamCreate(&g_stream));
 	if (g_gemm_resident_wgs > 0) g_gemm_resident_wgs = g_n_cu;
+	g_gemm_lds_cus = g_n_cu;
 	if (int rc = static_scratch_init()) return rc;
 	g_device = device;
 	g_inited = true;
@@ -1367,6 +1368,12 @@ int tg_set_taps(int enable) {
 	return TG_OK;
 }
 
+int tg_set_gemm_lds(int half_tiles_per_cu) {
+	if (half_tiles_per_cu < 0 || half_tiles_per_cu > 64) return tg_fail(TG_ERR_BAD_ARG, "0 (off) or the threshold in half tiles per compute unit, up to 64");
+	g_gemm_lds = half_tiles_per_cu;
+	return TG_OK;
+}
+
 int tg_set_gemm_mode(int mfma) {
 	g_gemm_mfma = mfma != 0;
 	return TG_OK;
@@ -1414,6 +1421,7 @@ int tg_reset_knobs() {
 	g_use_graphs = false;
 	g_gemm_split = true;
 	g_gemm_resident_wgs = g_n_cu;
+	g_gemm_lds = 2;
 	g_attn_merge_chunk = 48;
 	g_attn_prefill_bf16x3 = 1;
 	g_attn_prefill_planes = 1;

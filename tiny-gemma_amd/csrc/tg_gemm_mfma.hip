@@ -34,8 +34,13 @@
 
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 int g_gemm_resident_wgs = 256;
+// n > 0: products with at least n / 2 output tiles per compute unit run on gemm_i8_lds_kernel (two workgroups per
+// compute unit, both operands through an LDS ring); 0: never
+int g_gemm_lds = 2;
+int g_gemm_lds_cus = 256;  // compute units of the device (set by tg_init)
 
 namespace {
 
@@ -549,6 +554,194 @@ __global__ __launch_bounds__(GNT) void gemm_i8_resident_kernel(float *C, const i
 	}
 }
 
+// ---- the same product with two workgroups per compute unit -----------------------------------------------------
+// The kernels above hold one wave per SIMD (192 accumulators + a register ring of prefetched operands), so nothing
+// covers a workgroup's start-up, its barriers or its epilogue (accumulators -> fp32 -> 64 KB of stores with the matrix
+// cores idle: a sixth of the time at K = 1152).  Here a wave fits in 256 registers and a second workgroup shares the
+// compute unit: while one converts and stores, the other issues matrix instructions.
+//
+//   * Nothing is prefetched into registers.  Both operands go global -> LDS directly (global_load_lds_dwordx4: no
+//     registers, no conversion) into a ring of four one-k-step slots per workgroup (slot = 4 waves x 3 planes of A,
+//     each wave copying and reading only its own 3 KB, + 4 KB of B shared by the four waves), three k steps ahead.
+//   * One set of operand fragments (7 x 16 bytes per lane), read per k step after the barrier; the LDS latency is
+//     covered by the other workgroup's wave on the same SIMD.
+//   * The compiler does not see which LDS bytes a direct copy writes and would wait for ALL copies in flight before any
+//     LDS read it can see; the fragment reads are therefore explicit ds_read_b128 instructions with their own waits.
+//   * Of the 12 accumulator tiles, the 8 of digit planes 0 and 1 live in the accumulation registers and the 4 of plane 2
+//     in ordinary vector registers, 128 + 64: with two waves per SIMD a wave has 256 registers of both kinds together.
+//     The compiler allots all matrix accumulators to one kind, so the matrix instructions are written out with the
+//     register class of each accumulator given.  It therefore does not know them as matrix instructions: the wait
+//     between the last of them and the first ordinary read of an accumulator is explicit (s_nop).
+//   * The copies of a k step are issued one at a time behind every third matrix instruction: a wave issues in order,
+//     and a burst of copies or LDS reads from eight waves fills the queue it goes into and holds the matrix
+//     instructions behind it back.
+// Same integer sums, same epilogue arithmetic: the result equals the other kernels' bit for bit.
+constexpr int LDS_NSLOT = 4, LDS_AW = 3072, LDS_BOFF = 4 * LDS_AW, LDS_SLOT = LDS_BOFF + 4096;
+
+template <int OFF>
+__device__ __forceinline__ i32x4 lds_read_frag(unsigned addr) {
+	i32x4 r;
+	asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+	return r;
+}
+struct LdsFrags {
+	i32x4 a[3], b[4];
+};
+// names the registers, so that it stays between the reads and their use
+__device__ __forceinline__ void lds_frags_wait(LdsFrags &f) {
+	asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.b[0]), "+v"(f.b[1]), "+v"(f.b[2]), "+v"(f.b[3]));
+}
+template <int N>
+__device__ __forceinline__ void wait_copies_in_flight() {  // until at most N of this wave's vector memory loads are outstanding
+	asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+template <bool IN_ACC_REGS>
+__device__ __forceinline__ void mfma_i8_asm(i32x16 &acc, const i32x4 &bf, const i32x4 &af) {
+	if constexpr (IN_ACC_REGS) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(bf), "v"(af));
+	else asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(bf), "v"(af));
+}
+template <int... I, typename F>
+__device__ __forceinline__ void gemm_static_for_impl(std::integer_sequence<int, I...>, F &&f) {
+	(f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void gemm_static_for(F &&f) {
+	gemm_static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <bool GEGLU, bool LUTLDS>
+__global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
+                                                             const float *scales, int M, int K, int ldc, const float *lut, float gmin,
+                                                             float geps, float ginv, int lut_size, float *rowmax_part, int ntiles,
+                                                             int mblocks) {
+	extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];  // LDS_NSLOT slots; the GeLU table afterwards
+	const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+	// (row block, column tile) of this workgroup: every XCD a contiguous share, row blocks fastest (as gemm_i8_kernel)
+	int tile, mblock;
+	{
+		const int total = ntiles * mblocks, lin = (int)blockIdx.x;
+		if ((total & 7) == 0) {
+			const int chunk = total >> 3, v = (lin & 7) * chunk + (lin >> 3);
+			if ((mblocks & 7) == 0) {
+				const int mbx = mblocks >> 3, xcd = lin & 7, i = v - xcd * chunk;
+				mblock = xcd * mbx + i % mbx;
+				tile = i / mbx;
+			} else {
+				mblock = v % mblocks;
+				tile = v / mblocks;
+			}
+		} else {
+			tile = lin % ntiles;
+			mblock = lin / ntiles;
+		}
+	}
+	const int mtile = mblock * 4 + w;
+	const int nstage = K >> 5, last = nstage - 1;  // one k step (32 rows of K) per stage; a multiple of 4
+	const unsigned char *bsrc = reinterpret_cast<const unsigned char *>(Wg) + (size_t)tile * (size_t)K * TG_CT + (size_t)w * 1024 + 16 * lane;
+	const unsigned char *asrc = reinterpret_cast<const unsigned char *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 1024 + 16 * lane;
+	// piece q of the copy of stage st into a slot: q = 0..2 the planes of this wave's 32 rows, q = 3 its quarter of B.
+	// Stages past the end copy the last stage again, into slots nobody reads any more.
+	auto issue = [&](int st, int slot, int q) __attribute__((always_inline)) {
+		st = st < last ? st : last;
+		if (q < 3)
+			__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(asrc + (size_t)st * LDS_AW + q * 1024),
+			                                 (__attribute__((address_space(3))) void *)(ring + slot * LDS_SLOT + w * LDS_AW + q * 1024), 16, 0, 0);
+		else
+			__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(bsrc + (size_t)st * 4096),
+			                                 (__attribute__((address_space(3))) void *)(ring + slot * LDS_SLOT + LDS_BOFF + w * 1024), 16, 0, 0);
+	};
+#pragma unroll
+	for (int st = 0; st < LDS_NSLOT - 1; st++)
+#pragma unroll
+		for (int q = 0; q < 4; q++) issue(st, st, q);
+
+	i32x16 acc[3][4];
+#pragma unroll
+	for (int p = 0; p < 3; p++)
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int i = 0; i < 16; i++) acc[p][j][i] = 0;
+
+	const unsigned lbase = (unsigned)(size_t)ring;
+	const unsigned aaddr = lbase + w * LDS_AW + 16 * lane, baddr = lbase + LDS_BOFF + (hb * TG_CT + c) * 16;
+	LdsFrags f;
+	auto stage = [&](int st, auto uc) __attribute__((always_inline)) {
+		constexpr int U = decltype(uc)::value, O = U * LDS_SLOT;
+		wait_copies_in_flight<4 * (LDS_NSLOT - 2)>();  // this wave's copies of stage st have landed
+		tg_lds_barrier();                              // everyone's have; everyone has read stage st - 1
+		f.a[0] = lds_read_frag<O>(aaddr);
+		f.a[1] = lds_read_frag<O + 1024>(aaddr);
+		f.a[2] = lds_read_frag<O + 2048>(aaddr);
+		f.b[0] = lds_read_frag<O>(baddr);
+		f.b[1] = lds_read_frag<O + 512>(baddr);
+		f.b[2] = lds_read_frag<O + 1024>(baddr);
+		f.b[3] = lds_read_frag<O + 1536>(baddr);
+		lds_frags_wait(f);
+		gemm_static_for<12>([&](auto ic) {
+			constexpr int i = decltype(ic)::value, p = i >> 2, j = i & 3;
+			mfma_i8_asm<(p < 2)>(acc[p][j], f.b[j], f.a[p]);
+			if constexpr (i % 3 == 2) issue(st + LDS_NSLOT - 1, (U + LDS_NSLOT - 1) % LDS_NSLOT, i / 3);  // into the slot of stage st - 1
+		});
+	};
+	for (int st0 = 0; st0 < nstage; st0 += 4) {
+		stage(st0, std::integral_constant<int, 0>{});
+		stage(st0 + 1, std::integral_constant<int, 1>{});
+		stage(st0 + 2, std::integral_constant<int, 2>{});
+		stage(st0 + 3, std::integral_constant<int, 3>{});
+	}
+	wait_copies_in_flight<0>();  // the surplus copies too: the table below reuses the ring
+	// the matrix pipeline finishes its last instruction (8 passes) before an accumulator is read by an ordinary instruction
+	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+	float *lut_lds = reinterpret_cast<float *>(ring);
+	if (GEGLU && LUTLDS) {
+		__syncthreads();  // every wave is done with the ring
+		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
+		__syncthreads();
+	}
+
+	// epilogue, as in gemm_i8_kernel: element i of lane l is output column 8*(i/4) + 4*(l/32) + i%4, row l%32 of a 32x32 tile
+	const int m = mtile * 32 + c;
+	const float rs = rowinv[m];
+	auto value = [&](int j, int i, float scale) {
+		const float v = fmaf((float)acc[2][j][i], 65536.0f, fmaf((float)acc[1][j][i], 256.0f, (float)acc[0][j][i]));
+		return (v * rs) * scale;
+	};
+	float omax = 0.0f;
+	if (m < M) {
+		float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 4 * hb;
+		const float *sc0 = scales + tile * TG_CT + 4 * hb;
+#pragma unroll
+		for (int j = 0; j < (GEGLU ? 2 : 4); j++) {
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				const f32x4 su = *reinterpret_cast<const f32x4 *>(sc0 + 32 * j + 8 * q);
+				f32x4 sg = su;
+				if (GEGLU) sg = *reinterpret_cast<const f32x4 *>(sc0 + 32 * (j + 2) + 8 * q);
+				f32x4 o;
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int i = 4 * q + e;
+					if (GEGLU) {
+						const float gate = value(j + 2, i, sg[e]);
+						o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
+						       value(j, i, su[e]);
+						omax = fmaxf(omax, fabsf(o[e]));
+					} else {
+						o[e] = value(j, i, su[e]);
+					}
+				}
+				*reinterpret_cast<f32x4 *>(crow + 32 * j + 8 * q) = o;
+			}
+		}
+	}
+	if (GEGLU && rowmax_part != nullptr) {
+		omax = fmaxf(omax, tg_red_partner<32>(omax));
+		if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
+	}
+}
+
 // ---- few rows (a short prompt): the same product with the reduction split over the four waves ----------------
 // With a few hundred rows (up to 448: measured crossover between 400 and 512) the kernel above has only a handful of
 // workgroups (two row blocks x 9 column tiles for the down
@@ -717,6 +910,11 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 	hipLaunchKernelGGL(quant_pack_kernel<false>, grid, dim3(GNT), 0, s, A, lda, M, K, rowfac, apack, (float *)nullptr, (float *)nullptr);
 }
 
+// whether a product of M rows, K deep, ntiles column tiles runs on gemm_i8_lds_kernel (K in whole groups of four k steps)
+static bool tg_gemm_lds_taken(int M, int K, int ntiles) {
+	return g_gemm_lds > 0 && (K & 127) == 0 && M > TG_GEMM_SKINNY_ROWS && 2 * ntiles * ((M + 127) / 128) >= g_gemm_lds * g_gemm_lds_cus;
+}
+
 // ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns;
 // rowmax_part (GEGLU only, may be null): [tg_gemm_mfma_rows(M)] floats cleared by the caller; max|C[m][:]| is folded into it
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
@@ -751,6 +949,27 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	// 1000-token prefill: up|gate with 13.5 and 3.4 tiles per unit -5 % and -3 %; Q|K|V, output and down projections
 	// with 1.1 to 2.3 tiles per unit +1 to +3 us each: the start-up of the item walk is not recovered).
 	// (The load cursors of the item walk need at least 8 stages of K per item: K = 256 stays on one workgroup per tile.)
+	if (tg_gemm_lds_taken(M, K, ntiles) && ksplit == 1) {
+		static bool lds_set = false;
+		constexpr int ring_bytes = LDS_NSLOT * LDS_SLOT;
+		if (!lds_set) {  // 64 KB of dynamic LDS
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			lds_set = true;
+		}
+		const dim3 grid((unsigned)ntiles * mblocks), block(GNT);
+		if (geglu && lutlds)
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, true>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, ntiles, (int)mblocks);
+		else if (geglu)
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, ntiles, (int)mblocks);
+		else
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<false, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
+			                   geps, ginv, lut_size, rmp, ntiles, (int)mblocks);
+		return;
+	}
 	if (g_gemm_resident_wgs > 0 && ntiles * (int)mblocks * ksplit >= 3 * g_gemm_resident_wgs && K / KSTAGE / ksplit >= 8) {
 		const int mb = (int)mblocks * ksplit, total = ntiles * mb, G = g_gemm_resident_wgs;
 		const int perm = (total % 8 == 0 && G % 8 == 0) ? 1 : 0;  // workgroups go to the 8 XCDs round-robin
@@ -791,6 +1010,7 @@ int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu) {
 		return 1;
 	}
 	if (M <= TG_GEMM_SKINNY_ROWS || nstage % 4 != 0) return 1;
+	if (tg_gemm_lds_taken(M, K, ntiles)) return 1;  // two workgroups per compute unit: no nearly empty last round to fill
 	const long wgs = (long)((M + 127) / 128) * ntiles;
 	auto eff = [&](long n) { return (double)n / (double)(((n + n_cu - 1) / n_cu) * n_cu); };
 	// measured: worth it only when the last round is nearly empty (288 workgroups on 256 compute units: -2 % prefill time);
