@@ -186,7 +186,8 @@ int tg_set_gemm_split(int enable);
  * tiles, the operand prefetch running on from one tile into the next; 0 = one workgroup per tile.  Same results. */
 int tg_set_gemm_resident(int enable);
 /* n > 0 (default 2): prefill products of more than 448 rows with at least n / 2 output tiles per compute unit run two workgroups per compute
- * unit with both operands staged through LDS (same bits as the other kernels); 0: one workgroup per compute unit always */
+ * unit with both operands staged through LDS (same bits as the other kernels); 0: one workgroup per compute unit always.
+ * n + 64: the same without the two half-K copies that products filling under 3/4 of the workgroup slots otherwise run as */
 int tg_set_gemm_lds(int half_tiles_per_cu);
 /* prefill attention: 1 (default) = 16-bit matrix cores on two fp16 or three bf16 planes of every fp32 operand (cross
  * terms summed in fp32: fp32-level accuracy at several times the fp32 matrix rate), workgroups of 32 query positions

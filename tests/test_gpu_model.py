@@ -482,6 +482,31 @@ def test_two_gemm_workgroups_per_unit_change_no_bit_of_a_long_prefill(tg, oracle
     assert tok_a == tok_b and np.array_equal(lg_a, lg_b)
 
 
+def test_half_k_copies_of_the_two_workgroup_kernel_equal_the_unsplit_products(tg, oracle):
+    """8000 tokens through two layers of the 270m shape: output and down projection have 63 x 5 = 315 tiles for 512
+    workgroup slots and run as two half-K copies of the grid, the following norm adds the two partial results
+    (tg_set_gemm_lds(2), the default) - against the same products unsplit (2 + 64): same id, logits equal to fp32
+    rounding of one extra addition, and really a different path."""
+    cfg = tg.named_config("270m", 2)
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 24))
+    sess = model.session(gsize=1 << 20)
+    prompt = gi.prompt_ids(36, 8000)
+    out = []
+    try:
+        for knob in (2, 66):
+            tg.check(tg.lib().tg_set_gemm_lds(knob))
+            sess.reset()
+            out.append(sess.prefill(prompt))
+    finally:
+        tg.check(tg.lib().tg_set_gemm_lds(2))
+    (tok_a, lg_a), (tok_b, lg_b) = out
+    rel = normrel(lg_a, lg_b)
+    print(f"half-K copies vs unsplit (two workgroups per unit): logits rel {rel:.2e}")
+    assert tok_a == tok_b and rel < 2e-5
+    assert not np.array_equal(lg_a, lg_b)
+
+
 def test_half_k_grid_copies_equal_the_plain_grid(tg, oracle, weight_images, tables):
     """Prefill with the output/down projections computed as two half-K copies added by the following norm
     (taken when the plain grid fills its last round badly: here 1000 rows x 5 column tiles) against the

@@ -146,7 +146,10 @@ def test_gemm_k_parts_rule(pkg):
     assert f(178, 1024, 1152, 256) == 2      # 16 stages: 2 x 8
     assert f(100, 2048, 640, 256) == 4 and f(100, 1024, 640, 256) == 2
     assert f(1000, 6912, 1152, 256) == 2     # 72 workgroups on 256 units: two half-K copies
-    assert f(4096, 6912, 1152, 256) == 1     # 288 tiles: taken by the kernel that runs two workgroups per unit, no split
+    assert f(4096, 6912, 1152, 256) == 2     # 288 tiles on 512 workgroup slots (two per unit): two half-K copies fill them
+    assert f(4096, 1152, 6912, 256) == 1     # 1728 tiles
+    assert f(8192, 6912, 1152, 256) == 1     # 576 tiles: more than 3/4 of the slots
+    assert f(4096, 1152, 1536, 256) == 1     # 384 tiles, but 36 k steps do not halve into whole groups of four
     try:                                     # the rule of the one-workgroup-per-unit kernels
         assert pkg.lib().tg_set_gemm_lds(0) == 0
         assert f(4096, 6912, 1152, 256) == 2     # 288 workgroups on 256 units: two half-K copies

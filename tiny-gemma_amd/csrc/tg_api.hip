@@ -1369,8 +1369,9 @@ int tg_set_taps(int enable) {
 }
 
 int tg_set_gemm_lds(int half_tiles_per_cu) {
-	if (half_tiles_per_cu < 0 || half_tiles_per_cu > 64) return tg_fail(TG_ERR_BAD_ARG, "0 (off) or the threshold in half tiles per compute unit, up to 64");
-	g_gemm_lds = half_tiles_per_cu;
+	if (half_tiles_per_cu < 0 || half_tiles_per_cu > 127) return tg_fail(TG_ERR_BAD_ARG, "0 (off) or the threshold in half tiles per compute unit, up to 63 (+ 64: no half-K copies)");
+	g_gemm_lds = half_tiles_per_cu & 63;
+	g_gemm_lds_ksplit = (half_tiles_per_cu & 64) ? 0 : 1;  // + 64: without the half-K copies (measurement aid)
 	return TG_OK;
 }
 
@@ -1422,6 +1423,7 @@ int tg_reset_knobs() {
 	g_gemm_split = true;
 	g_gemm_resident_wgs = g_n_cu;
 	g_gemm_lds = 2;
+	g_gemm_lds_ksplit = 1;
 	g_attn_merge_chunk = 48;
 	g_attn_prefill_bf16x3 = 1;
 	g_attn_prefill_planes = 1;

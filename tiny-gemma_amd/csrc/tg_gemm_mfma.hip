@@ -41,6 +41,7 @@ int g_gemm_resident_wgs = 256;
 // compute unit, both operands through an LDS ring); 0: never
 int g_gemm_lds = 2;
 int g_gemm_lds_cus = 256;  // compute units of the device (set by tg_init)
+int g_gemm_lds_ksplit = 1;  // experiment switch: two half-K copies where the tiles would fill under 3/4 of the workgroup slots
 
 namespace {
 
@@ -613,7 +614,7 @@ template <bool GEGLU, bool LUTLDS>
 __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
                                                              const float *scales, int M, int K, int ldc, const float *lut, float gmin,
                                                              float geps, float ginv, int lut_size, float *rowmax_part, int ntiles,
-                                                             int mblocks) {
+                                                             int mblocks, int ksplit, size_t csplit) {
 	extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];  // LDS_NSLOT slots; the GeLU table afterwards
 	const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hb = lane >> 5;
 	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -636,10 +637,18 @@ __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int
 			mblock = lin / ntiles;
 		}
 	}
+	// ksplit == 2 (plain epilogue): the grid holds every row block twice; copy z walks half z of K and writes its own
+	// partial result (C + z * csplit), which the consumer adds.  Taken where one workgroup per tile would leave most
+	// compute units with a single workgroup and a few with two, which then set the pace.
+	const int mreal = mblocks / ksplit, z = mblock / mreal;
+	mblock -= z * mreal;
 	const int mtile = mblock * 4 + w;
-	const int nstage = K >> 5, last = nstage - 1;  // one k step (32 rows of K) per stage; a multiple of 4
-	const unsigned char *bsrc = reinterpret_cast<const unsigned char *>(Wg) + (size_t)tile * (size_t)K * TG_CT + (size_t)w * 1024 + 16 * lane;
-	const unsigned char *asrc = reinterpret_cast<const unsigned char *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 1024 + 16 * lane;
+	const int nstage = (K >> 5) / ksplit, last = nstage - 1;  // one k step (32 rows of K) per stage; a multiple of 4
+	const unsigned char *bsrc = reinterpret_cast<const unsigned char *>(Wg) + (size_t)tile * (size_t)K * TG_CT + (size_t)z * nstage * 4096 +
+	                            (size_t)w * 1024 + 16 * lane;
+	const unsigned char *asrc = reinterpret_cast<const unsigned char *>(Apack) + (size_t)mtile * (size_t)(K >> 5) * 3 * 1024 +
+	                            (size_t)z * nstage * LDS_AW + 16 * lane;
+	C += (size_t)z * csplit;
 	// piece q of the copy of stage st into a slot: q = 0..2 the planes of this wave's 32 rows, q = 3 its quarter of B.
 	// Stages past the end copy the last stage again, into slots nobody reads any more.
 	auto issue = [&](int st, int slot, int q) __attribute__((always_inline)) {
@@ -949,7 +958,7 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	// 1000-token prefill: up|gate with 13.5 and 3.4 tiles per unit -5 % and -3 %; Q|K|V, output and down projections
 	// with 1.1 to 2.3 tiles per unit +1 to +3 us each: the start-up of the item walk is not recovered).
 	// (The load cursors of the item walk need at least 8 stages of K per item: K = 256 stays on one workgroup per tile.)
-	if (tg_gemm_lds_taken(M, K, ntiles) && ksplit == 1) {
+	if (tg_gemm_lds_taken(M, K, ntiles) && (K >> 5) % (4 * ksplit) == 0) {
 		static bool lds_set = false;
 		constexpr int ring_bytes = LDS_NSLOT * LDS_SLOT;
 		if (!lds_set) {  // 64 KB of dynamic LDS
@@ -958,16 +967,17 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
 			lds_set = true;
 		}
-		const dim3 grid((unsigned)ntiles * mblocks), block(GNT);
+		const int mb = (int)mblocks * ksplit;
+		const dim3 grid((unsigned)(ntiles * mb)), block(GNT);
 		if (geglu && lutlds)
 			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, true>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, ntiles, (int)mblocks);
+			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
 		else if (geglu)
 			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, ntiles, (int)mblocks);
+			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
 		else
 			hipLaunchKernelGGL((gemm_i8_lds_kernel<false, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
-			                   geps, ginv, lut_size, rmp, ntiles, (int)mblocks);
+			                   geps, ginv, lut_size, rmp, ntiles, mb, ksplit, csplit);
 		return;
 	}
 	if (g_gemm_resident_wgs > 0 && ntiles * (int)mblocks * ksplit >= 3 * g_gemm_resident_wgs && K / KSTAGE / ksplit >= 8) {
@@ -1010,7 +1020,14 @@ int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu) {
 		return 1;
 	}
 	if (M <= TG_GEMM_SKINNY_ROWS || nstage % 4 != 0) return 1;
-	if (tg_gemm_lds_taken(M, K, ntiles)) return 1;  // two workgroups per compute unit: no nearly empty last round to fill
+	if (tg_gemm_lds_taken(M, K, ntiles)) {
+		// Two workgroups per compute unit.  With more tiles than compute units but well under two per unit, most units
+		// would hold one workgroup and a few two, and those few set the pace: two half-K copies fill both slots of
+		// every unit (halves of whole groups of four k steps, at least 8 k steps each).
+		const long tiles = (long)((M + 127) / 128) * ntiles;
+		const int ksteps = K >> 5;
+		return (g_gemm_lds_ksplit && 4 * tiles <= 3 * 2 * (long)n_cu && ksteps % 8 == 0 && ksteps / 2 >= 8) ? 2 : 1;
+	}
 	const long wgs = (long)((M + 127) / 128) * ntiles;
 	auto eff = [&](long n) { return (double)n / (double)(((n + n_cu - 1) / n_cu) * n_cu); };
 	// measured: worth it only when the last round is nearly empty (288 workgroups on 256 compute units: -2 % prefill time);
