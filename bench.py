@@ -372,7 +372,7 @@ def main():
         g_us = ev.elapsed_ms(e0, e1) * 1e3 / 20
         g_flops = 2.0 * gm * gk * gn
         extra_rooflines["prefill_gemm"] = {
-            "kernel": "gemm_i8_resident_kernel (+ row_scale_kernel, quant_pack_kernel)", "bound": "mfma", "unit": "TFLOP/s", "peak": INT8_PEAK_TOPS,
+            "kernel": "gemm_i8_lds_kernel (+ row_scale_kernel, quant_pack_kernel)", "bound": "mfma", "unit": "TFLOP/s", "peak": INT8_PEAK_TOPS,
             "shape": [gm, gk, gn], "algorithmic_flops_per_launch": g_flops, "avg_launch_us": g_us,
             "achieved": g_flops / g_us / 1e6, "frac": g_flops / g_us / 1e6 / INT8_PEAK_TOPS,
             "note": "tg_qgemm_dev, 20 back-to-back launches incl. the quantising pre-pass; algorithmic 2*M*K*N flops against the dense int8 "
