@@ -955,10 +955,11 @@ int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 
 // `window` keys before it and itself).  Returns false when no query tile needs splitting (then the plain launch is
 // already balanced).  items: one int4 per workgroup {query tile, first key tile, end key tile, slot or -1},
 // heaviest first; split: one int4 per split query tile; nslots: chunks that go through scratch.
-// 32 query positions per workgroup once that leaves a workgroup for every other compute unit (measured crossover:
-// between 2048 and 4096 tokens on 256 compute units)
+// 32 query positions per workgroup (two waves per SIMD, a K/V tile fetched once for twice the queries) once that leaves
+// a workgroup for every eighth compute unit; the work lists cut the key ranges so that the other units get items too.
+// Measured crossover on 256 compute units, whole prefills: 600 tokens +1.6 %, 1000 tokens -2 %, 1536 -4.6 %, 2047 -5.5 %.
 int tg_attn_prefill_query_tile(int S, int n_cu) {
-	return (g_attn_prefill_bf16x3 == 2 || (g_attn_prefill_bf16x3 == 1 && (S + 31) / 32 >= n_cu / 2)) ? 32 : TQ;
+	return (g_attn_prefill_bf16x3 == 2 || (g_attn_prefill_bf16x3 == 1 && (S + 31) / 32 >= n_cu / 8)) ? 32 : TQ;
 }
 
 bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
