@@ -921,7 +921,9 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 
 // whether a product of M rows, K deep, ntiles column tiles runs on gemm_i8_lds_kernel (K in whole groups of four k steps)
 static bool tg_gemm_lds_taken(int M, int K, int ntiles) {
-	return g_gemm_lds > 0 && (K & 127) == 0 && M > TG_GEMM_SKINNY_ROWS && 2 * ntiles * ((M + 127) / 128) >= g_gemm_lds * g_gemm_lds_cus;
+	const int tiles = ntiles * ((M + 127) / 128);
+	if (M <= TG_GEMM_SKINNY_ROWS && tiles < TG_GEMM_SKINNY_BLOCKS) return false;  // the few-row kernel's case
+	return g_gemm_lds > 0 && (K & 127) == 0 && 2 * tiles >= g_gemm_lds * g_gemm_lds_cus;
 }
 
 // ntiles tiles of 128 (virtual) columns; epi GEGLU: every tile is 64 up | 64 gate columns and C has ntiles * 64 columns;
