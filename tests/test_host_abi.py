@@ -147,6 +147,7 @@ def test_gemm_k_parts_rule(pkg):
     assert f(100, 2048, 640, 256) == 4 and f(100, 1024, 640, 256) == 2
     assert f(1000, 6912, 1152, 256) == 2     # 72 workgroups on 256 units: two half-K copies
     assert f(4096, 6912, 1152, 256) == 2     # 288 tiles on 512 workgroup slots (two per unit): two half-K copies fill them
+    assert f(4096, 1024, 1152, 256) == 1     # the same tiles with a short K: a second start-up costs more than idle slots
     assert f(4096, 1152, 6912, 256) == 1     # 1728 tiles
     assert f(8192, 6912, 1152, 256) == 1     # 576 tiles: more than 3/4 of the slots
     assert f(4096, 1152, 1536, 256) == 1     # 384 tiles, but 36 k steps do not halve into whole groups of four

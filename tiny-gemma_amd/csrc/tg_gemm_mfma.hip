@@ -1025,10 +1025,12 @@ int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu) {
 	if (tg_gemm_lds_taken(M, K, ntiles)) {
 		// Two workgroups per compute unit.  With more tiles than compute units but well under two per unit, most units
 		// would hold one workgroup and a few two, and those few set the pace: two half-K copies fill both slots of
-		// every unit (halves of whole groups of four k steps, at least 8 k steps each).
+		// every unit (halves of whole groups of four k steps).  Only for a long K: each copy has its own start-up and
+		// writes its own partial result, which at K = 1024 costs more than the idle slots (output projection at 4096
+		// rows: 26.5 us unsplit, 32.7 us as two copies; down projection, K = 6912: 123 -> 108 us).
 		const long tiles = (long)((M + 127) / 128) * ntiles;
 		const int ksteps = K >> 5;
-		return (g_gemm_lds_ksplit && 4 * tiles <= 3 * 2 * (long)n_cu && ksteps % 8 == 0 && ksteps / 2 >= 8) ? 2 : 1;
+		return (g_gemm_lds_ksplit && 4 * tiles <= 3 * 2 * (long)n_cu && ksteps % 8 == 0 && ksteps / 2 >= 32) ? 2 : 1;
 	}
 	const long wgs = (long)((M + 127) / 128) * ntiles;
 	auto eff = [&](long n) { return (double)n / (double)(((n + n_cu - 1) / n_cu) * n_cu); };
