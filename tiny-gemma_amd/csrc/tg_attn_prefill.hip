@@ -316,6 +316,13 @@ __device__ __forceinline__ void report_range(unsigned rmax, int *range_flag) {
 	}
 }
 
+// e^x for the softmax weights of the split-precision kernels: v_exp_f32 on x * log2(e), two instructions instead of
+// the dozen of expf (range checks, extended-precision argument), which at nine exponentials per lane and key tile cost
+// as much as the P.V matrix instructions (16,384 tokens of the 270m shape: 1.0 of 19.4 ms).  The product is rounded
+// once: for x in [-10, 0], where the weights that matter lie, the exponent is off by at most 2^-21, i.e. the result by
+// 3.3e-7 relative, a few units in the last place like the vectorised expf of the reference build; e^-inf = 0.
+__device__ __forceinline__ float softmax_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+
 constexpr int NT32 = HD / 32;  // k steps of a score product
 
 // Same arguments and outputs as attn_prefill_mfma_kernel.  QG = groups of 16 query positions per workgroup, each
@@ -463,13 +470,13 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_split_kernel(float *o, 
 		tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
 		const float m_new = fmaxf(m_run, tmax);
 		const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // no valid key yet (see the fp32 kernel)
-		const float alpha = expf(m_run - m_ref);
+		const float alpha = softmax_exp(m_run - m_ref);
 		float psum = 0.0f;
 		float pv[8];  // the lane's 8 key slots: keys 4g + i, then 16 + 4g + i
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
-			pv[i] = expf(s0[i] - m_ref);
-			pv[4 + i] = expf(s1[i] - m_ref);
+			pv[i] = softmax_exp(s0[i] - m_ref);
+			pv[4 + i] = softmax_exp(s1[i] - m_ref);
 			psum += pv[i] + pv[4 + i];
 		}
 		psum += tg_red_partner<16>(psum);
@@ -781,13 +788,13 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 			tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
 			const float m_new = fmaxf(m_run, tmax);
 			const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // no valid key yet (see the fp32 kernel)
-			const float alpha = expf(m_run - m_ref);
+			const float alpha = softmax_exp(m_run - m_ref);
 			float psum = 0.0f;
 			float pv[8];  // the lane's 8 key slots: keys 4g + i, then 16 + 4g + i
 #pragma unroll
 			for (int i = 0; i < 4; i++) {
-				pv[i] = expf(s0[i] - m_ref);
-				pv[4 + i] = expf(s1[i] - m_ref);
+				pv[i] = softmax_exp(s0[i] - m_ref);
+				pv[4 + i] = softmax_exp(s1[i] - m_ref);
 				psum += pv[i] + pv[4 + i];
 			}
 			psum += tg_red_partner<16>(psum);
