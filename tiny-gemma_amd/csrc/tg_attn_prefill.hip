@@ -617,6 +617,14 @@ __device__ __forceinline__ void copy_image_to_lds(const unsigned char *img, unsi
 		                                 (__attribute__((address_space(3))) void *)(lds + (c * NW + w) * 1024), 16, 0, 0);
 }
 
+// One piece (kilobyte c * NW + w) of the same copy, for callers that spread the pieces between other instructions: a
+// wave issues in order, and a burst of copies from eight waves fills the queue they go into and holds what follows back.
+template <int NW>
+__device__ __forceinline__ void copy_image_piece(const unsigned char *img, unsigned char *lds, int lane, int w, int c) {
+	__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + (size_t)(c * NW + w) * 1024 + 16 * lane),
+	                                 (__attribute__((address_space(3))) void *)(lds + (c * NW + w) * 1024), 16, 0, 0);
+}
+
 // LDS reads of the matrix operands as the instruction itself.  The compiler cannot tell which LDS bytes a load that
 // writes straight into LDS will touch, so before every LDS read it can see it waits for ALL such loads in flight,
 // which would serialise the copy of a later image with the work on the current one.  These reads it does not see;
@@ -740,8 +748,11 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 		const bool mine = kb + tile * TK <= q0w + 15;
 
 		// ---- phase 2 * tile: scores.  Image 2 * tile + 2 (the next K) goes into the free buffer meanwhile ----
-		if (2 * tile + 2 < nimg) copy_image_to_lds<NW, IMG_KB>(img0 + (size_t)(2 * tile + 2) * PLANE_IMG, smem + fbuf * PLANE_IMG, lane, w);
+		const bool copy_k = 2 * tile + 2 < nimg, copy_v = 2 * tile + 3 < nimg;
+		const unsigned char *next_k = img0 + (size_t)(2 * tile + 2) * PLANE_IMG, *next_v = img0 + (size_t)(2 * tile + 3) * PLANE_IMG;
+		unsigned char *k_dst = smem + fbuf * PLANE_IMG, *v_dst = smem + kbuf * PLANE_IMG;
 		f32x4 s0 = f32x4{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+		if (!mine && copy_k) copy_image_to_lds<NW, IMG_KB>(next_k, k_dst, lane, w);
 		if (mine) {
 			// the two groups of 16 keys; even and odd k steps in separate accumulators; the fragments of step t + 1 are
 			// requested before the matrix instructions of step t
@@ -759,6 +770,13 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 				}
 				sa[0][t & 1] = mfma_terms<F>(a, qp[t], sa[0][t & 1]);
 				sa[1][t & 1] = mfma_terms<F>(b, qp[t], sa[1][t & 1]);
+				// this wave's pieces of the next K image, one (two where there are more pieces than k steps) behind each of the
+				// first k steps
+				constexpr int PK = (SHARE + NT32 - 1) / NT32;
+#pragma unroll
+				for (int pc = t * PK; pc < (t + 1) * PK && pc < SHARE; pc++) {
+					if (copy_k) copy_image_piece<NW>(next_k, k_dst, lane, w, pc);
+				}
 			});
 			s0 = (sa[0][0] + sa[0][1]) * F::SSCALE;
 			s1 = (sa[1][0] + sa[1][1]) * F::SSCALE;
@@ -772,7 +790,7 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 		tg_lds_barrier();  // the K image is released, the V image is complete
 
 		// ---- phase 2 * tile + 1: softmax and P.V.  Image 2 * tile + 3 (the next V) goes into the buffer the K image has left ----
-		if (2 * tile + 3 < nimg) copy_image_to_lds<NW, IMG_KB>(img0 + (size_t)(2 * tile + 3) * PLANE_IMG, smem + kbuf * PLANE_IMG, lane, w);
+		if (!mine && copy_v) copy_image_to_lds<NW, IMG_KB>(next_v, v_dst, lane, w);
 		if (mine) {
 			Planes va = read_v<F, 0>(vaddr);  // in flight during the softmax
 			const int j0 = kb + tile * TK + 4 * g;
@@ -817,6 +835,9 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 				const Planes vf = va;
 				if constexpr (dt + 1 < HD / 16) va = read_v<F, dt + 1>(vaddr);
 				oacc[dt] = mfma_terms<F>(pp, vf, oacc[dt]);
+				if constexpr (dt < SHARE) {  // the pieces of the next V image, likewise
+					if (copy_v) copy_image_piece<NW>(next_v, v_dst, lane, w, dt);
+				}
 			});
 		}
 		if (2 * tile + 3 < nimg) {
