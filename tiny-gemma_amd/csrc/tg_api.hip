@@ -1325,7 +1325,7 @@ int tg_set_attn_merge_chunk(int keys) {
 
 int tg_set_attn_prefill_mode(int mode) {
 	if (mode < 0 || mode > 3) return tg_fail(TG_ERR_BAD_ARG, "mode: 0, 1, 2 or 3");
-	g_attn_prefill_bf16x3 = mode;
+	g_attn_prefill_split = mode;
 	return TG_OK;
 }
 
@@ -1425,7 +1425,7 @@ int tg_reset_knobs() {
 	g_gemm_lds = 2;
 	g_gemm_lds_ksplit = 1;
 	g_attn_merge_chunk = 48;
-	g_attn_prefill_bf16x3 = 1;
+	g_attn_prefill_split = 1;
 	g_attn_prefill_planes = 1;
 	g_attn_prefill_f16 = 1;
 	g_chain_picks = true;
@@ -1539,7 +1539,7 @@ struct PrefillCtx {
 	int *d_ids = nullptr;
 	float *x = nullptr, *xn = nullptr, *qkv = nullptr, *ao = nullptr, *t = nullptr, *hb = nullptr, *rowscale = nullptr, *amax = nullptr;
 	int8_t *apack = nullptr;
-	void *planes = nullptr;  // pre-split K/V plane images of the layer being processed (split-bf16 attention)
+	void *planes = nullptr;  // pre-split K/V plane images of the layer being processed (split-precision attention)
 	const TgAttnPrefillPlan *plan_global = nullptr, *plan_local = nullptr;
 	int o_parts = 1, d_parts = 1;
 	size_t tpart = 0;

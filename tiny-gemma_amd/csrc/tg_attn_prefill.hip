@@ -968,7 +968,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o
 
 }  // namespace
 
-// split-bf16 path: K/V split into plane images once per layer and copied straight into LDS (1: for prompts of
+// split-precision path: K/V split into plane images once per layer and copied straight into LDS (1: for prompts of
 // TG_ATTN_PLANES_MIN_TOKENS tokens or more, where it pays: measured break-even at ~1500 tokens, -8 % prefill time at
 // 2000; 2: always), or every workgroup splits what it stages (0)
 int g_attn_prefill_planes = 1;
@@ -977,7 +977,7 @@ size_t tg_attn_prefill_planes_bytes(int S) { return (size_t)((S + TK - 1) / TK) 
 // split path: 1 (default) = two fp16 planes, three products; 0 = three bf16 planes, six products
 int g_attn_prefill_f16 = 1;
 
-int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 matrix path; 2: the same, always with 32-query workgroups
+int g_attn_prefill_split = 1;  // 0: fp32 matrix path; 1 (default): split-precision matrix path (two fp16 or three bf16 planes); 2: the same, always with 32-query workgroups
 
 // Work list of a layer of S tokens, for tg_launch_attn_prefill: causal (window < 0) or local (a query sees the
 // `window` keys before it and itself).  Returns false when no query tile needs splitting (then the plain launch is
@@ -987,7 +987,7 @@ int g_attn_prefill_bf16x3 = 1;  // 0: fp32 matrix path; 1 (default): split-bf16 
 // a workgroup for every eighth compute unit; the work lists cut the key ranges so that the other units get items too.
 // Measured crossover on 256 compute units, whole prefills: 600 tokens +1.6 %, 1000 tokens -2 %, 1536 -4.6 %, 2047 -5.5 %.
 int tg_attn_prefill_query_tile(int S, int n_cu) {
-	return (g_attn_prefill_bf16x3 == 2 || (g_attn_prefill_bf16x3 == 1 && (S + 31) / 32 >= n_cu / 8)) ? 32 : TQ;
+	return (g_attn_prefill_split == 2 || (g_attn_prefill_split == 1 && (S + 31) / 32 >= n_cu / 8)) ? 32 : TQ;
 }
 
 bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots) {
@@ -1093,9 +1093,9 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
 	const dim3 grid(whole ? (unsigned)((S + tq - 1) / tq) : (unsigned)plan->nitems);
 	const int4 *items = whole ? nullptr : plan->items;
 	float *po = whole ? nullptr : plan->part_o, *pml = whole ? nullptr : plan->part_ml;
-	const bool planes = g_attn_prefill_bf16x3 && planes_ws != nullptr &&
+	const bool planes = g_attn_prefill_split && planes_ws != nullptr &&
 	                    (g_attn_prefill_planes == 2 || (g_attn_prefill_planes == 1 && S >= TG_ATTN_PLANES_MIN_TOKENS));
-	if (!g_attn_prefill_bf16x3)
+	if (!g_attn_prefill_split)
 		hipLaunchKernelGGL(attn_prefill_mfma_kernel, grid, dim3(PNT), 0, s, o, q, k, v, S, ldq, ldkv, ldo, is_sw, window, items,
 		                   po, pml);
 	else if (g_attn_prefill_f16)

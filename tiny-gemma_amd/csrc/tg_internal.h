@@ -180,7 +180,7 @@ struct TgAttnPrefillPlan {
 	int nitems, nsplit;
 	float *part_o, *part_ml;
 };
-extern int g_attn_prefill_bf16x3;  // prefill attention: 0 = fp32 matrix path, 1 = split-bf16 matrix path, 2 = the same with 32-query workgroups at any length
+extern int g_attn_prefill_split;  // prefill attention: 0 = fp32 matrix path, 1 = split-precision matrix path (two fp16 or three bf16 planes), 2 = the same with 32-query workgroups at any length
 int tg_attn_prefill_query_tile(int S, int n_cu);  // query positions per workgroup of the kernel a launch will take
 // window < 0: causal layer; else a local layer whose queries see `window` keys before them and themselves
 bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots);
@@ -191,7 +191,7 @@ void tg_launch_attn_prefill(float *o, const float *q, const float *k, const floa
                             bool finish_later = false, void *planes_ws = nullptr, int *range_flag = nullptr);
 // range_flag (device, may be null): set to 1 when an operand does not fit the fp16 planes of the split path
 extern int g_attn_prefill_f16;
-// planes_ws: tg_attn_prefill_planes_bytes(S) bytes of scratch for the pre-split K/V plane images of the split-bf16 path
+// planes_ws: tg_attn_prefill_planes_bytes(S) bytes of scratch for the pre-split K/V plane images of the split-precision path
 // (null: every workgroup splits the tiles it stages itself)
 extern int g_attn_prefill_planes;
 size_t tg_attn_prefill_planes_bytes(int S);
