@@ -182,9 +182,6 @@ int tg_set_gemm_mode(int mfma);
  * partial results where that keeps more compute units busy (a badly filled last round of workgroups at a few thousand
  * tokens; the long-K products of a short prompt); the following norm adds the parts.  0 = never */
 int tg_set_gemm_split(int enable);
-/* prefill, int8 matrix path: 1 (default) = one resident workgroup per compute unit walks its share of the output
- * tiles, the operand prefetch running on from one tile into the next; 0 = one workgroup per tile.  Same results. */
-int tg_set_gemm_resident(int enable);
 /* n > 0 (default 2): prefill products of more than 448 rows with at least n / 2 output tiles per compute unit run two workgroups per compute
  * unit with both operands staged through LDS (same bits as the other kernels); 0: one workgroup per compute unit always.
  * n + 64: the same without the two half-K copies that products filling under 3/4 of the workgroup slots otherwise run as */

@@ -177,40 +177,14 @@ def test_qgemm_mfma_equals_digit_plane_closed_form(tg, shape):
     assert np.array_equal(Cm, _digit_plane_closed_form(A, W, s))
 
 
-@pytest.mark.parametrize("shape", [(2048, 1152, 6912, 21), (1920, 1152, 6912, 22), (2300, 1024, 6912, 23), (6200, 640, 2048, 24),
-                                   (2048, 256, 6912, 25)])
-def test_qgemm_resident_workgroups_equal_one_per_tile_and_the_closed_form(tg, shape):
-    """From three output tiles per compute unit on, one resident workgroup per unit walks the tiles with the operand
-    prefetch running across tile boundaries.  Same bits as one workgroup per tile and as the closed form.  The
-    shapes cover the item walk's cases: 18 stages of K (tile boundaries alternate between the middle and the end of
-    a group of four stages) and 16; row blocks a multiple of 8 (split by XCD), 49 (XCD mapping on the flat list), and
-    tile counts that are no multiple of 8 (no XCD mapping); a last row block that is partly padding.  K = 256 has too
-    few stages for the tile walk and must stay on one workgroup per tile whatever the switch says."""
-    m, i, n, seed = shape
-    A, W, s = gi.gemm_inputs(m, i, n, seed)
-    A[1] *= np.float32(1e-4)
-    out = []
-    try:
-        tg.check(tg.lib().tg_set_gemm_lds(0))  # else the two-workgroups kernel takes these shapes
-        for resident in (1, 0):
-            tg.check(tg.lib().tg_set_gemm_resident(resident))
-            Cm = np.full((m, n), np.nan, np.float32)
-            tg.launch_qgemm(Cm, A, W, s, m, i, n)
-            out.append(Cm)
-    finally:
-        tg.check(tg.lib().tg_set_gemm_resident(1))
-        tg.check(tg.lib().tg_set_gemm_lds(2))
-    assert np.array_equal(out[0], out[1])
-    assert np.array_equal(out[0], _digit_plane_closed_form(A, W, s))
-
-
 @pytest.mark.parametrize("shape", [(2048, 1152, 6912, 31), (1920, 1152, 6912, 32), (2300, 1024, 6912, 33), (6200, 640, 2048, 34),
                                    (2048, 256, 6912, 35), (2048, 2048, 6912, 36)])
 def test_qgemm_two_workgroups_per_unit_equal_the_other_kernels_and_the_closed_form(tg, shape):
     """The default kernel for products of more than 448 rows with at least one output tile per compute unit
     (tg_set_gemm_lds(n): from n / 2 tiles per unit; 0 = never): two workgroups share a compute unit, both operands go
     through an LDS ring and a third of the accumulators sit in ordinary vector registers.  Same integer
-    sums and epilogue: the result must equal the default kernels' and the closed form bit for bit.  Shapes: K of 9,
+    sums and epilogue: the result must equal the one-workgroup-per-tile kernel's (tg_set_gemm_lds(0)) and the closed
+    form bit for bit.  Shapes: K of 9,
     8, 5, 2 and 16 groups of four k steps; row blocks a multiple of 8, 15 (a tile count that is no multiple of 8: no
     XCD mapping), 18 and 49; a last row block that is partly padding."""
     m, i, n, seed = shape

@@ -437,29 +437,6 @@ def test_short_prompt_k_parts_equal_the_unsplit_products(tg, oracle):
     assert not np.array_equal(lg_a, lg_b)
 
 
-def test_resident_gemm_workgroups_change_no_bit_of_a_long_prefill(tg, oracle):
-    """3000 tokens through two layers of the 270m shape: the up|gate product has 24 x 32 output tiles, three per
-    compute unit, and runs on resident workgroups (fused gelu(gate) * up epilogue inside the tile walk).  Same
-    arithmetic as one workgroup per tile: the logits must not differ in a single bit."""
-    cfg = tg.named_config("270m", 2)
-    model = tg.Transformer(cfg)
-    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 22))
-    sess = model.session(gsize=1024)
-    prompt = gi.prompt_ids(34, 3000)
-    out = []
-    try:
-        tg.check(tg.lib().tg_set_gemm_lds(0))  # else the two-workgroups kernel takes these shapes
-        for resident in (1, 0):
-            tg.check(tg.lib().tg_set_gemm_resident(resident))
-            sess.reset()
-            out.append(sess.prefill(prompt))
-    finally:
-        tg.check(tg.lib().tg_set_gemm_resident(1))
-        tg.check(tg.lib().tg_set_gemm_lds(2))
-    (tok_a, lg_a), (tok_b, lg_b) = out
-    assert tok_a == tok_b and np.array_equal(lg_a, lg_b)
-
-
 @pytest.mark.parametrize("gsize", [1024, 8192])
 def test_two_gemm_workgroups_per_unit_change_no_bit_of_a_long_prefill(tg, oracle, gsize):
     """3000 tokens through two layers of the 270m shape with tg_set_gemm_lds(1): the up|gate product (fused

@@ -380,7 +380,6 @@ int tg_init(int device) {
 	snprintf(g_devname, sizeof(g_devname), "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
 	g_n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	TG_HIP(hipStreamCreate(&g_stream));
-	if (g_gemm_resident_wgs > 0) g_gemm_resident_wgs = g_n_cu;
 	g_gemm_lds_cus = g_n_cu;
 	if (int rc = static_scratch_init()) return rc;
 	g_device = device;
@@ -1358,11 +1357,6 @@ int tg_session_release_workspace(tg_session *s) {
 	return TG_OK;
 }
 
-int tg_set_gemm_resident(int enable) {
-	g_gemm_resident_wgs = enable ? g_n_cu : 0;
-	return TG_OK;
-}
-
 int tg_set_taps(int enable) {
 	g_keep_taps = enable != 0;
 	return TG_OK;
@@ -1421,7 +1415,6 @@ int tg_reset_knobs() {
 	g_gemv_max_blocks = 2048;
 	g_use_graphs = false;
 	g_gemm_split = true;
-	g_gemm_resident_wgs = g_n_cu;
 	g_gemm_lds = 2;
 	g_gemm_lds_ksplit = 1;
 	g_attn_merge_chunk = 48;

@@ -36,7 +36,6 @@
 #include <type_traits>
 #include <utility>
 
-int g_gemm_resident_wgs = 256;
 // n > 0: products with at least n / 2 output tiles per compute unit run on gemm_i8_lds_kernel (two workgroups per
 // compute unit, both operands through an LDS ring); 0: never
 int g_gemm_lds = 2;
@@ -297,261 +296,6 @@ __global__ __launch_bounds__(GNT) void gemm_i8_kernel(float *C, const int8_t *Ap
 		// (non-negative floats order like their bit patterns; the caller cleared the array)
 		omax = fmaxf(omax, tg_red_partner<32>(omax));
 		if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
-	}
-}
-
-// ---- the same product with workgroups that stay resident ------------------------------------------------------
-// One workgroup per compute unit walks its share of the (row block, column tile) grid: item b, b + G, b + 2 G, ...
-// of the launch order above (G workgroups, a multiple of 8 when the XCD mapping is on, so a workgroup keeps its
-// XCD and the items in flight at any time are the ones the plain grid would run together).  The register ring of
-// prefetched operands does not know about tiles: its two load cursors walk straight from the last stage of one
-// item into the first stage of the next, so the next item's operands are already in flight (and its first weight
-// stage in LDS) while the epilogue of the current one runs.  With one wave per SIMD nothing else overlaps an
-// item's start-up latency.
-//
-// Ring slots and LDS buffers are compile-time indices with period 4 stages.  K / 64 is even but not always a
-// multiple of 4 (18 stages for K = 1152): then the boundary between two items falls alternately in the middle and
-// at the end of an unrolled group of four.
-//
-// Plain epilogue only: with the fused up|gate epilogue in the loop the register allocator permutes whole
-// accumulator tiles on every pass (some 150 register moves between matrix instructions that depend on them), which
-// costs more than the overlap gains; that product keeps one workgroup per tile.
-//
-// The ring (160 registers) stays live across the epilogue, so the epilogue must not be allowed what the compiler
-// does by default — copy all 192 accumulators into ordinary registers first.  It reads them one at a time with
-// an explicit v_accvgpr_read, in program order.
-__device__ __forceinline__ float acc_f32(int a) {
-	int r;
-	asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a));
-	return (float)r;
-}
-
-template <bool GEGLU, bool LUTLDS>
-__global__ __launch_bounds__(GNT) void gemm_i8_resident_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
-                                                               const float *scales, int M, int K, int ldc, const float *lut, float gmin,
-                                                               float geps, float ginv, int lut_size, float *rowmax_part, int Mpad,
-                                                               int ksplit, size_t csplit, int ntiles, int mblocks, int perm) {
-	__shared__ __attribute__((aligned(16))) i32x4 Bs[2][KSTAGE / 16][TG_CT];
-	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
-	__shared__ __attribute__((aligned(16))) float sc_lds[TG_CT];  // column scales of the item whose epilogue runs
-
-	const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hb = lane >> 5;
-	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int total = ntiles * mblocks, G = (int)gridDim.x;
-	const int nstage = K / KSTAGE / ksplit, mreal = mblocks / ksplit;
-	if (GEGLU && LUTLDS) {  // visible after the first barrier
-		for (int i = tid; i < lut_size; i += GNT) lut_lds[i] = lut[i];
-	}
-
-	// Items.  Position lin in launch order -> (column tile, row block) as in gemm_i8_kernel: with the XCD mapping
-	// (perm: total and G are multiples of 8) XCD x = lin % 8 owns positions x * total/8 + lin/8 of a list in which
-	// row blocks vary fastest (split by XCD first when their number is a multiple of 8).  In every case the pair is
-	// (quotient, remainder) of an index by a fixed divisor, and going from lin to lin + G adds a fixed step to the
-	// index: one division at the start, none afterwards.
-	const bool byxcd = perm && (mblocks & 7) == 0;
-	const int mbx = mblocks >> 3;
-	const int divisor = byxcd ? mbx : (perm ? mblocks : ntiles);
-	const int step = perm ? (G >> 3) : G, step_q = step / divisor, step_r = step - step_q * divisor;
-	struct Item {
-		int lin, q, r;
-	};
-	auto item_next = [&](const Item &it) __attribute__((always_inline)) {  // the workgroup's last item is its own successor
-		const bool more = it.lin + G < total;
-		int r = it.r + step_r, q = it.q + step_q;
-		const bool wrap = r >= divisor;
-		r = wrap ? r - divisor : r;
-		q = wrap ? q + 1 : q;
-		Item n;
-		n.lin = more ? it.lin + G : it.lin;
-		n.q = more ? q : it.q;
-		n.r = more ? r : it.r;
-		return n;
-	};
-	auto item_tile = [&](const Item &it) __attribute__((always_inline)) { return perm ? it.q : it.r; };
-	auto item_mblock = [&](const Item &it) __attribute__((always_inline)) {
-		return byxcd ? (it.lin & 7) * mbx + it.r : (perm ? it.r : it.q);
-	};
-	// z: which half of K (ksplit == 2), mtile: this wave's tile of 32 rows
-	auto item_z = [&](const Item &it) __attribute__((always_inline)) { return (ksplit == 2 && item_mblock(it) >= mreal) ? 1 : 0; };
-	auto item_mtile = [&](const Item &it) __attribute__((always_inline)) { return (item_mblock(it) - item_z(it) * mreal) * 4 + w; };
-	auto a_base = [&](const Item &it) __attribute__((always_inline)) {
-		return reinterpret_cast<const i32x4 *>(Apack) + (size_t)item_mtile(it) * (size_t)(K >> 5) * 3 * 64 + (size_t)item_z(it) * nstage * 6 * 64;
-	};
-	auto b_base = [&](const Item &it) __attribute__((always_inline)) {
-		return reinterpret_cast<const i32x4 *>(Wg + (size_t)item_tile(it) * (size_t)K * TG_CT) + (size_t)item_z(it) * nstage * 512;
-	};
-	Item cur;
-	{
-		const int lin = (int)blockIdx.x;
-		const int i = byxcd ? (lin >> 3) : (perm ? (lin & 7) * (total >> 3) + (lin >> 3) : lin);
-		cur.lin = lin;
-		cur.q = i / divisor;
-		cur.r = i - cur.q * divisor;
-	}
-	Item n1 = item_next(cur), n2 = item_next(n1);
-
-	// Load cursors: base of the cursor's stage (wave-uniform), stages left in its item, and the base of the item
-	// after it.  Advancing is branch-free (loads under branches would make the compiler wait for all of them);
-	// `next` is refreshed in the epilogue.  Behind the workgroup's last item a cursor walks that item again: the
-	// surplus loads of the ring stay inside the operands and land in slots nobody reads.
-	struct Cursor {
-		const i32x4 *p, *next;
-		int left;
-	};
-	Cursor ca, cb;
-	ca.p = a_base(cur);
-	cb.p = b_base(cur);
-	ca.next = a_base(n1);
-	cb.next = b_base(n1);
-	ca.left = cb.left = nstage - 1;
-	auto advance_a = [&]() __attribute__((always_inline)) {
-		const bool more = ca.left > 0;
-		ca.p = more ? ca.p + 6 * 64 : ca.next;
-		ca.left = more ? ca.left - 1 : nstage - 1;
-	};
-	auto advance_b = [&]() __attribute__((always_inline)) {
-		const bool more = cb.left > 0;
-		cb.p = more ? cb.p + 512 : cb.next;
-		cb.left = more ? cb.left - 1 : nstage - 1;
-	};
-	i32x4 *bdst = &Bs[0][0][0] + tid;
-	i32x4 areg[4][6];
-	i32x4 breg[4][2];
-	auto load_b = [&](i32x4 *r) __attribute__((always_inline)) {
-		r[0] = cb.p[tid];
-		r[1] = cb.p[tid + 256];
-		advance_b();
-	};
-	auto store_b = [&](int buf, const i32x4 *r) __attribute__((always_inline)) {
-		bdst[buf * 512] = r[0];
-		bdst[buf * 512 + 256] = r[1];
-	};
-	auto load_a = [&](i32x4 *r) __attribute__((always_inline)) {
-#pragma unroll
-		for (int i = 0; i < 6; i++) r[i] = ca.p[lane + i * 64];
-		advance_a();
-	};
-
-	i32x16 acc[3][4];
-	auto clear_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-		for (int p = 0; p < 3; p++)
-#pragma unroll
-			for (int j = 0; j < 4; j++)
-#pragma unroll
-				for (int i = 0; i < 16; i++) acc[p][j][i] = 0;
-	};
-	auto read_b = [&](int buf, int ks, i32x4 *bfrag) __attribute__((always_inline)) {
-#pragma unroll
-		for (int j = 0; j < 4; j++) bfrag[j] = Bs[buf][2 * ks + hb][32 * j + c];
-	};
-	auto mfma_step = [&](const i32x4 *a, const i32x4 *bfrag) __attribute__((always_inline)) {
-#pragma unroll
-		for (int p = 0; p < 3; p++)
-#pragma unroll
-			for (int j = 0; j < 4; j++) acc[p][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfrag[j], a[p], acc[p][j], 0, 0, 0);
-	};
-	i32x4 b0[4], b1[4];
-	// the stage of gemm_i8_kernel; u = stage index modulo 4 (ring slot and LDS buffer), the cursors know the rest
-	auto stage = [&](auto uc) __attribute__((always_inline)) {
-		constexpr int u = decltype(uc)::value;
-		load_a(areg[(u + 3) & 3]);
-		load_b(breg[u]);
-		store_b((u + 1) & 1, breg[(u + 1) & 3]);
-		read_b(u & 1, 1, b1);
-		mfma_step(areg[u], b0);
-		tg_lds_barrier();
-		read_b((u + 1) & 1, 0, b0);
-		mfma_step(areg[u] + 3, b1);
-	};
-
-	// Epilogue of item `cur`.  Both cursors are inside the next item by now (the ring runs 3 and 4 stages ahead, an
-	// item has at least 8): their `next` becomes the item after that.
-	auto epilogue = [&]() __attribute__((always_inline)) {
-		ca.next = a_base(n2);
-		cb.next = b_base(n2);
-		const int tile = item_tile(cur), m = item_mtile(cur) * 32 + c;
-		// The tile's 128 column scales go through LDS: held in registers (16 per lane and column block) they would not
-		// fit beside the ring.  The barrier also covers the wait for the matrix pipeline's last instruction.
-		if (tid < TG_CT) sc_lds[tid] = scales[tile * TG_CT + tid];
-		const float rs = rowinv[m];
-		float *crow = C + (size_t)item_z(cur) * csplit + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 4 * hb;
-		tg_lds_barrier();
-		// the matrix pipeline finishes its last instruction (8 passes) before the accumulators are read
-		asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-		// The four column blocks in order, one accumulator tile (three planes) at a time.  Fused up|gate: blocks 0, 1
-		// are the up columns, kept until their gate blocks 2, 3 come by.
-		float up[GEGLU ? 2 : 1][16];
-		float omax = 0.0f;
-#pragma unroll
-		for (int j = 0; j < 4; j++) {
-#pragma unroll
-			for (int q = 0; q < 4; q++) {
-				const f32x4 sc = *reinterpret_cast<const f32x4 *>(&sc_lds[32 * j + 8 * q + 4 * hb]);
-				f32x4 o;
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int i = 4 * q + e;
-					const float x = fmaf(acc_f32(acc[2][j][i]), 65536.0f, fmaf(acc_f32(acc[1][j][i]), 256.0f, acc_f32(acc[0][j][i])));
-					o[e] = (x * rs) * sc[e];
-					if (GEGLU && j < 2) up[j][i] = o[e];
-					if (GEGLU && j >= 2) {
-						o[e] = (LUTLDS ? gelu_lut(o[e], lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(o[e], lut, gmin, geps, ginv, lut_size)) * up[j - 2][i];
-						omax = fmaxf(omax, fabsf(o[e]));
-					}
-				}
-				if ((!GEGLU || j >= 2) && m < M) *reinterpret_cast<f32x4 *>(crow + 32 * (GEGLU ? j - 2 : j) + 8 * q) = o;
-			}
-		}
-		if (GEGLU && rowmax_part != nullptr) {
-			omax = fmaxf(omax, tg_red_partner<32>(omax));
-			if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
-		}
-		cur = n1;
-		n1 = n2;
-		n2 = item_next(n2);
-		// Leave with nothing outstanding (vmcnt(0); the ring's loads have long landed, this waits for the stores):
-		// otherwise the wait-count bookkeeping carries "maybe pending" registers of this rarely taken path into the
-		// main loop and drains the ring there on every pass.
-		__builtin_amdgcn_s_waitcnt(0x0F70);
-	};
-
-	load_b(breg[0]);
-	load_a(areg[0]);
-	load_b(breg[1]);
-	load_a(areg[1]);
-	load_b(breg[2]);
-	load_a(areg[2]);
-	load_b(breg[3]);
-	store_b(0, breg[0]);
-	tg_lds_barrier();
-	read_b(0, 0, b0);
-
-	// One pass of the loop is a group of four stages.  Items end after the group's fourth stage, or, when the stage
-	// count is 4 n + 2, alternately after the second stage of group n and after the fourth of group 2 n.
-	const int ngroups = nstage >> 2;
-	const bool paired = (nstage & 2) != 0;
-	const int period = paired ? 2 * ngroups + 1 : ngroups;
-	int gi = 0, left = (total - (int)blockIdx.x + G - 1) / G;  // items this workgroup still has to finish
-	clear_acc();
-	for (;;) {
-		stage(std::integral_constant<int, 0>{});
-		stage(std::integral_constant<int, 1>{});
-		if (paired && gi == ngroups) {
-			epilogue();
-			if (--left == 0) break;
-			clear_acc();
-		}
-		stage(std::integral_constant<int, 2>{});
-		stage(std::integral_constant<int, 3>{});
-		if (gi == period - 1) {
-			epilogue();
-			if (--left == 0) break;
-			clear_acc();
-			gi = 0;
-		} else {
-			gi++;
-		}
 	}
 }
 
@@ -956,47 +700,6 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	// kparts == 2 (STORE only; see tg_gemm_mfma_k_parts): two half-K copies of the grid, the second writes C + part_stride
 	const int ksplit = (kparts == 2 && !geglu) ? 2 : 1;
 	const size_t csplit = ksplit == 2 ? part_stride : 0;
-	// Resident workgroups pay off from three tiles per compute unit on (measured per product inside a 4096-token and a
-	// 1000-token prefill: up|gate with 13.5 and 3.4 tiles per unit -5 % and -3 %; Q|K|V, output and down projections
-	// with 1.1 to 2.3 tiles per unit +1 to +3 us each: the start-up of the item walk is not recovered).
-	// (The load cursors of the item walk need at least 8 stages of K per item: K = 256 stays on one workgroup per tile.)
-	if (tg_gemm_lds_taken(M, K, ntiles) && (K >> 5) % (4 * ksplit) == 0) {
-		static bool lds_set = false;
-		constexpr int ring_bytes = LDS_NSLOT * LDS_SLOT;
-		if (!lds_set) {  // 64 KB of dynamic LDS
-			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
-			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
-			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
-			lds_set = true;
-		}
-		const int mb = (int)mblocks * ksplit;
-		const dim3 grid((unsigned)(ntiles * mb)), block(GNT);
-		if (geglu && lutlds)
-			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, true>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
-		else if (geglu)
-			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
-		else
-			hipLaunchKernelGGL((gemm_i8_lds_kernel<false, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
-			                   geps, ginv, lut_size, rmp, ntiles, mb, ksplit, csplit);
-		return;
-	}
-	if (g_gemm_resident_wgs > 0 && ntiles * (int)mblocks * ksplit >= 3 * g_gemm_resident_wgs && K / KSTAGE / ksplit >= 8) {
-		const int mb = (int)mblocks * ksplit, total = ntiles * mb, G = g_gemm_resident_wgs;
-		const int perm = (total % 8 == 0 && G % 8 == 0) ? 1 : 0;  // workgroups go to the 8 XCDs round-robin
-		const dim3 grid((unsigned)G), block(GNT);
-		if (geglu && lutlds)
-			hipLaunchKernelGGL((gemm_i8_resident_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, Mpad, 1, (size_t)0, ntiles, mb, perm);
-		else if (geglu)
-			hipLaunchKernelGGL((gemm_i8_resident_kernel<true, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
-			                   ginv, lut_size, rmp, Mpad, 1, (size_t)0, ntiles, mb, perm);
-		else
-			hipLaunchKernelGGL((gemm_i8_resident_kernel<false, false>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
-			                   geps, ginv, lut_size, rmp, Mpad, ksplit, csplit, ntiles, mb, perm);
-		return;
-	}
 	const dim3 grid((unsigned)ntiles, mblocks * (unsigned)ksplit), block(GNT);
 	if (geglu && lutlds)
 		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,

@@ -227,8 +227,6 @@ void tg_launch_quant_pack(const float *A, int lda, int M, int K, int8_t *apack, 
 void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, const int8_t *Wg, const float *scales, int M, int K,
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
                          int kparts, size_t part_stride, hipStream_t s);
-// workgroups of the resident form of the MFMA GEMM (one per compute unit; set at init), 0: one workgroup per tile
-extern int g_gemm_resident_wgs;
 extern int g_gemm_lds, g_gemm_lds_cus, g_gemm_lds_ksplit;
 // parts of K (1, 2, 4) a plain-epilogue product should run in; part p writes C + p * part_stride, the consumer adds them
 int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu);
