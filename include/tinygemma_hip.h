@@ -186,6 +186,9 @@ int tg_set_gemm_split(int enable);
  * unit with both operands staged through LDS (same bits as the other kernels); 0: one workgroup per compute unit always.
  * n + 64: the same without the two half-K copies that products filling under 3/4 of the workgroup slots otherwise run as */
 int tg_set_gemm_lds(int half_tiles_per_cu);
+/* launches of the int8-matrix GEMM so far, by kernel: the few-row kernel, one workgroup per tile, two workgroups per
+ * compute unit (tests read them to make sure a product ran on the kernel they mean to check) */
+int tg_debug_gemm_launches(long long *few_rows, long long *one_per_tile, long long *two_per_unit);
 /* prefill attention: 1 (default) = 16-bit matrix cores on two fp16 or three bf16 planes of every fp32 operand (cross
  * terms summed in fp32: fp32-level accuracy at several times the fp32 matrix rate), workgroups of 32 query positions
  * for long prompts (4096 tokens and up on 256 compute units), else of 16; 2 = the same with 32 at any length;

@@ -191,15 +191,18 @@ def test_qgemm_two_workgroups_per_unit_equal_the_other_kernels_and_the_closed_fo
     A, W, s = gi.gemm_inputs(m, i, n, seed)
     A[1] *= np.float32(1e-4)
     A[m - 1] *= np.float32(3e3)
-    out = []
+    out, ran = [], []
     try:
         for lds in (1, 0):
             tg.check(tg.lib().tg_set_gemm_lds(lds))
             Cm = np.full((m, n), np.nan, np.float32)
+            before = tg.gemm_launches()
             tg.launch_qgemm(Cm, A, W, s, m, i, n)
+            ran.append(tuple(b - a for a, b in zip(before, tg.gemm_launches())))
             out.append(Cm)
     finally:
         tg.check(tg.lib().tg_set_gemm_lds(2))
+    assert ran == [(0, 0, 1), (0, 1, 0)]     # the two calls really ran on the two kernels
     assert np.array_equal(out[0], out[1])
     assert np.array_equal(out[0], _digit_plane_closed_form(A, W, s))
 

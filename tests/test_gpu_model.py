@@ -447,14 +447,19 @@ def test_two_gemm_workgroups_per_unit_change_no_bit_of_a_long_prefill(tg, oracle
     model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 2), 22))
     sess = model.session(gsize=gsize)
     prompt = gi.prompt_ids(34, 3000)
-    out = []
+    out, ran = [], []
     try:
         for lds in (1, 0):
             tg.check(tg.lib().tg_set_gemm_lds(lds))
             sess.reset()
+            before = tg.gemm_launches()
             out.append(sess.prefill(prompt))
+            ran.append(tuple(b - a for a, b in zip(before, tg.gemm_launches())))
     finally:
         tg.check(tg.lib().tg_set_gemm_lds(2))
+    # 2 layers x 4 products: Q|K|V (288 tiles) and up|gate (768) on the two-workgroups kernel, the output and down
+    # projections (120 tiles, under half a tile per compute unit) on one workgroup per tile either way
+    assert ran == [(0, 4, 4), (0, 8, 0)]
     (tok_a, lg_a), (tok_b, lg_b) = out
     assert tok_a == tok_b and np.array_equal(lg_a, lg_b)
 
@@ -474,7 +479,9 @@ def test_half_k_copies_of_the_two_workgroup_kernel_equal_the_unsplit_products(tg
         for knob in (2, 66):
             tg.check(tg.lib().tg_set_gemm_lds(knob))
             sess.reset()
+            before = tg.gemm_launches()
             out.append(sess.prefill(prompt))
+            assert tuple(b - a for a, b in zip(before, tg.gemm_launches())) == (0, 0, 8)  # all on the two-workgroups kernel
     finally:
         tg.check(tg.lib().tg_set_gemm_lds(2))
     (tok_a, lg_a), (tok_b, lg_b) = out

@@ -106,6 +106,7 @@ def lib():
     L.tg_qgemm_dev_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_debug_launch_chain.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
     L.tg_debug_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p]
+    L.tg_debug_gemm_launches.argtypes = [C.POINTER(C.c_longlong)] * 3
     L.tg_debug_mfma_clock.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.tg_decode_profile.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double), c_i32p]
     L.tg_debug_repeat_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
@@ -230,6 +231,13 @@ class QWeight:
             self.free()
         except Exception:  # noqa: BLE001
             pass
+
+
+def gemm_launches():
+    """(few-row kernel, one workgroup per tile, two workgroups per compute unit): GEMM launches so far, by kernel."""
+    a, b_, c = C.c_longlong(), C.c_longlong(), C.c_longlong()
+    check(lib().tg_debug_gemm_launches(C.byref(a), C.byref(b_), C.byref(c)))
+    return a.value, b_.value, c.value
 
 
 def synchronize():

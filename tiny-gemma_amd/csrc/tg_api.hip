@@ -1362,6 +1362,14 @@ int tg_set_taps(int enable) {
 	return TG_OK;
 }
 
+int tg_debug_gemm_launches(long long *few_rows, long long *one_per_tile, long long *two_per_unit) {
+	if (!few_rows || !one_per_tile || !two_per_unit) return tg_fail(TG_ERR_BAD_ARG, "null pointer");
+	*few_rows = g_gemm_launches[0];
+	*one_per_tile = g_gemm_launches[1];
+	*two_per_unit = g_gemm_launches[2];
+	return TG_OK;
+}
+
 int tg_set_gemm_lds(int half_tiles_per_cu) {
 	if (half_tiles_per_cu < 0 || half_tiles_per_cu > 127) return tg_fail(TG_ERR_BAD_ARG, "0 (off) or the threshold in half tiles per compute unit, up to 63 (+ 64: no half-K copies)");
 	g_gemm_lds = half_tiles_per_cu & 63;

@@ -40,6 +40,9 @@
 // compute unit, both operands through an LDS ring); 0: never
 int g_gemm_lds = 2;
 int g_gemm_lds_cus = 256;  // compute units of the device (set by tg_init)
+// launches so far of the few-row kernel, the one-workgroup-per-tile kernel and the two-workgroups-per-unit kernel
+// (tests read them to make sure a product really ran on the kernel they mean to check)
+long g_gemm_launches[3] = {0, 0, 0};
 int g_gemm_lds_ksplit = 1;  // experiment switch: two half-K copies where the tiles would fill under 3/4 of the workgroup slots
 
 namespace {
@@ -685,6 +688,7 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	float *rmp = geglu ? rowmax_part : nullptr;
 	// few rows and few column tiles: split K over the waves instead of leaving most compute units idle
 	if (M <= TG_GEMM_SKINNY_ROWS && (int)mblocks * ntiles < TG_GEMM_SKINNY_BLOCKS) {
+		g_gemm_launches[0]++;
 		const dim3 grid((unsigned)ntiles, (unsigned)((M + 31) / 32), (unsigned)(geglu ? 1 : kparts)), block(GNT);
 		if (geglu && lutlds)
 			hipLaunchKernelGGL((gemm_i8_skinny_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
@@ -700,6 +704,30 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
 	// kparts == 2 (STORE only; see tg_gemm_mfma_k_parts): two half-K copies of the grid, the second writes C + part_stride
 	const int ksplit = (kparts == 2 && !geglu) ? 2 : 1;
 	const size_t csplit = ksplit == 2 ? part_stride : 0;
+	if (tg_gemm_lds_taken(M, K, ntiles) && (K >> 5) % (4 * ksplit) == 0) {
+		g_gemm_launches[2]++;
+		static bool lds_set = false;
+		constexpr int ring_bytes = LDS_NSLOT * LDS_SLOT;
+		if (!lds_set) {  // 64 KB of dynamic LDS
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, true>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<true, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			(void)hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_lds_kernel<false, false>), hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);
+			lds_set = true;
+		}
+		const int mb = (int)mblocks * ksplit;
+		const dim3 grid((unsigned)(ntiles * mb)), block(GNT);
+		if (geglu && lutlds)
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, true>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
+		else if (geglu)
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<true, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps,
+			                   ginv, lut_size, rmp, ntiles, mb, 1, (size_t)0);
+		else
+			hipLaunchKernelGGL((gemm_i8_lds_kernel<false, false>), grid, block, ring_bytes, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin,
+			                   geps, ginv, lut_size, rmp, ntiles, mb, ksplit, csplit);
+		return;
+	}
+	g_gemm_launches[1]++;
 	const dim3 grid((unsigned)ntiles, mblocks * (unsigned)ksplit), block(GNT);
 	if (geglu && lutlds)
 		hipLaunchKernelGGL((gemm_i8_kernel<true, true>), grid, block, 0, s, C, apack, rowinv, Wg, scales, M, K, ldc, lut, gmin, geps, ginv,
