@@ -198,7 +198,9 @@ int tg_set_attn_prefill_mode(int mode);
  * planes (x = h + l, 22 significant bits), three products per fp32 product; 0 = three bf16 planes, six products
  * (24 bits).  The fp16 form runs half the matrix instructions; its operands must lie within +-65504 (q and k are
  * RMS-normalised, p is a probability, v a projection of a normalised vector): a value outside makes the forward
- * return TG_ERR_STATE instead of a wrong result, and the bf16 form, which has fp32's range, is the way out. */
+ * return TG_ERR_STATE instead of a wrong result, and the bf16 form, which has fp32's range, is the way out.
+ * With 1, launches that use the K/V plane images and 32-query workgroups run on 32x32x16 matrix instructions (two
+ * waves per head, each with half the head dimension); 2 = two fp16 planes on the 16x16x32 kernels only. */
 int tg_set_attn_prefill_format(int f16);
 /* prefill attention, modes 1-3: where the planes of K and V come from.  1 (default) = for prompts of 2048
  * tokens or more a pre-pass splits the K and V rows of a layer once and stores every 32-key tile as the image of the

@@ -263,7 +263,8 @@ ATTN_MODES = {
     "f16x2": (1, 1, 1),                 # the default: two fp16 planes, 16- or 32-query workgroups by prompt length
     "f16x2_32q": (2, 1, 1),
     "f16x2_16q_planes": (3, 2, 1),      # fed from pre-split plane images at any length (what 2048 tokens and more get)
-    "f16x2_32q_planes": (2, 2, 1),
+    "f16x2_32q_planes": (2, 2, 1),      # 32x32x16 matrix instructions, two waves per head (what long prompts get)
+    "f16x2_32q_planes_16x16": (2, 2, 2),  # the same images and workgroups on the 16x16x32 kernel
     "bf16x3": (1, 1, 0),                # three bf16 planes, six products
     "bf16x3_16q_planes": (3, 2, 0),
     "bf16x3_32q_planes": (2, 2, 0),

@@ -370,7 +370,8 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
     prompt = gi.prompt_ids(36, n_prompt)
     out = {}
     L = tg.lib()
-    combos = [(1, 0, 1), (0, 0, 1), (2, 0, 1), (3, 2, 1), (2, 2, 1), (1, 0, 0), (2, 2, 0)]   # (kernel mode, planes, fp16 format)
+    # (kernel mode, planes, operand format); (2, 2, 1) is the kernel on 32x32x16 matrix instructions
+    combos = [(1, 0, 1), (0, 0, 1), (2, 0, 1), (3, 2, 1), (2, 2, 1), (2, 2, 2), (1, 0, 0), (2, 2, 0)]
     try:
         for mode, planes, f16 in combos:
             tg.check(L.tg_set_attn_prefill_mode(mode))
@@ -386,7 +387,7 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
         assert out[key][0] == out[combos[0]][0]
         assert normrel(out[key][1], out[combos[0]][1]) < 2e-5
     # the plane images hold the same planes the staging code computes: not a bit differs
-    assert np.array_equal(out[(2, 2, 1)][1], out[(2, 0, 1)][1])
+    assert np.array_equal(out[(2, 2, 2)][1], out[(2, 0, 1)][1])
 
 
 def test_one_session_many_prompt_lengths(tg, oracle):

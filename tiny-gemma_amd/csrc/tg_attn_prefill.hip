@@ -28,6 +28,7 @@
 #include "tg_internal.h"
 
 #include <algorithm>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -629,6 +630,10 @@ __device__ __forceinline__ void copy_image_piece(const unsigned char *img, unsig
 // writes straight into LDS will touch, so before every LDS read it can see it waits for ALL such loads in flight,
 // which would serialise the copy of a later image with the work on the current one.  These reads it does not see;
 // the wait for them is lds_wait(), which names the registers so that it stays between the reads and their use.
+// Between such a read and its wait the compiler believes the register already holds the value: keep the two in one
+// basic block.  Where control flow merges in between it may copy the "value" to another register before the data has
+// arrived (seen with a read issued ahead of an if/else: a few lanes of the later-running waves got stale data).
+// tests/test_isa_hazards.py checks the compiled kernels for any instruction that touches such a register early.
 template <typename V, int OFF>
 __device__ __forceinline__ V lds_read16(unsigned addr) {
 	V r;
@@ -879,6 +884,362 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 	}
 }
 
+// ---- 32 query positions per matrix instruction ---------------------------------------------------------------------
+// In the kernels above a wave multiplies 16 queries with every K and V fragment it reads from LDS: 64 KB of fragments
+// per wave and key tile, with bank conflicts on the V reads in 13 % of the LDS cycles (SQ_LDS_BANK_CONFLICT).
+// v_mfma_f32_32x32x16_f16 takes fragments of the same size (64 lanes x 16 bytes) and does twice the work with them:
+// 32 keys x 32 queries x 16 dims.  A wave that owned 32 queries of a head alone would need 128 registers for its Q
+// planes and 128 for its output rows; here two waves share a head and split the HEAD DIMENSION: wave (head, dh) keeps
+// dims 128 dh .. + 127 of Q (64 registers) and of the output (64 registers), computes the scores' partial sums over
+// its dims, and the two swap those partial sums through LDS (4 KB each way, next to the 16 + 16 KB of fragments a
+// wave reads per tile, all of them conflict-free 1 KB rows).  A sum of two addends is the same in either order, so
+// both hold the same scores, weights and running sums, and each multiplies the weights with its half of V.  fp16
+// planes only (the bf16 form needs three planes of everything: 96 registers of Q).
+// Measured against the 16-query kernel on the same box (kernel trace): causal layer of 16,384 tokens 1,920-1,955 ->
+// 1,725-1,760 us, local layer 145-150 -> 137-142 us, local layer of 4,096 tokens 54-55 -> 50-52 us; the matrix cores
+// are busy 45 % of the kernel's clocks (41 %).
+//
+// Layout of v_mfma_f32_32x32x16_f16: lane (r = lane % 32, h = lane / 32) holds A[r][8h .. 8h + 7], B[8h .. 8h + 7][r]
+// and C[8j + 4h + i][r] in register 4j + i (j, i = 0..3).  Only the pairing of A and B slots matters, so
+//   scores:  A = K, lane holds dims 16 ks + 8h .. + 7 of key r, B = Q likewise for query r:
+//            C[8j + 4h + i][c] = S^T[key 8j + 4h + i][query c]: a lane holds 16 keys of query c = lane % 32;
+//   output:  B = P^T, step s = 0, 1 takes the lane's registers 8s .. 8s + 7 (keys 16s + 4h + i, then 16s + 8 + 4h + i);
+//            A = V^T with the same key order, lane r = dim: C[8j + 4h + i][c] = O^T[dim 32 dt + 8j + 4h + i][query c].
+// The output is kept transposed so that a lane owns one query in both products: its running maximum, running sum and
+// rescaling factor never leave the lane.
+// Plane images for this kernel (attn_planes_wide_kernel), 16-byte elements, every fragment 1 KB in lane order:
+//   Kw[plane][ks = 0..15][lane], Vw[plane][s = 0..1][dt = 0..7][lane].
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int WIDE_BQ = 32;                                        // query positions per workgroup
+constexpr size_t WIDE_IMG = 2 * PLANE_BYTES;                       // an image of two fp16 planes, 32 KB
+constexpr size_t WIDE_LDS = 4 * WIDE_IMG + 8 * 4096;               // ring of four images + the waves' partial scores: all 160 KB
+static_assert(PLANE_BYTES == (HD / 16) * 64 * 16 && PLANE_BYTES == 2 * (HD / 32) * 64 * 16, "one plane of Kw and of Vw");
+
+__global__ __launch_bounds__(PNT) void attn_planes_wide_kernel(unsigned char *planes, const float *k, const float *v, int S, int ldkv,
+                                                              int *range_flag) {
+	typedef FmtF16x2 F;
+	typedef F::vec vec;
+	const int tile = blockIdx.x, tid = threadIdx.x;
+	vec *Kimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * WIDE_IMG);
+	vec *Vimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * WIDE_IMG + WIDE_IMG);
+	unsigned rmax = 0u;
+	// K: unit = (key, piece of 8 dims): 32 consecutive threads read one key's 1 KB row
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		const int unit = tid + PNT * u, piece = unit & 31, key = unit >> 5;
+		const int j = tile * TK + key;
+		float x[8];
+		const float *src = k + (size_t)(j < S ? j : S - 1) * ldkv + 8 * piece;
+		const f32x4 a = *reinterpret_cast<const f32x4 *>(src), b = *reinterpret_cast<const f32x4 *>(src + 4);
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			x[e] = j < S ? a[e] : 0.0f;
+			x[4 + e] = j < S ? b[e] : 0.0f;
+		}
+		track_range<F>(rmax, x);
+		const PlanesT<F> pl = split8<F>(x);
+		const size_t at = (size_t)(piece >> 1) * 64 + (piece & 1) * 32 + key;  // ks = piece / 2, h = piece % 2
+#pragma unroll
+		for (int pn = 0; pn < 2; pn++) Kimg[pn * (PLANE_BYTES / 16) + at] = pl.p[pn];
+	}
+	// V: unit = (s, dt, lane): dim 32 dt + lane % 32, keys 16 s + 4 h + {0..3} and 16 s + 8 + 4 h + {0..3}
+#pragma unroll
+	for (int u = 0; u < 4; u++) {
+		const int unit = tid + PNT * u, lane = unit & 63, dt = (unit >> 6) & 7, s = unit >> 9;
+		const int d = 32 * dt + (lane & 31), h = lane >> 5;
+		float x[8];
+#pragma unroll
+		for (int sl = 0; sl < 8; sl++) {
+			const int j = tile * TK + 16 * s + 8 * (sl >> 2) + 4 * h + (sl & 3);
+			const float val = v[(size_t)(j < S ? j : S - 1) * ldkv + d];
+			x[sl] = j < S ? val : 0.0f;
+		}
+		track_range<F>(rmax, x);
+		const PlanesT<F> pl = split8<F>(x);
+#pragma unroll
+		for (int pn = 0; pn < 2; pn++) Vimg[pn * (PLANE_BYTES / 16) + unit] = pl.p[pn];
+	}
+	report_range<F>(rmax, range_flag);
+}
+
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+// acc += a . b: the three significant cross terms of two-plane operands, smallest first
+__device__ __forceinline__ f32x16 mfma32_terms(const PlanesT<FmtF16x2> &a, const PlanesT<FmtF16x2> &b, f32x16 acc) {
+	acc = mfma32(a.p[1], b.p[0], acc);
+	acc = mfma32(a.p[0], b.p[1], acc);
+	acc = mfma32(a.p[0], b.p[0], acc);
+	return acc;
+}
+// fragment at a compile-time offset from a per-lane base: both planes
+template <int OFF>
+__device__ __forceinline__ PlanesT<FmtF16x2> read_wide(unsigned addr) {
+	PlanesT<FmtF16x2> f;
+	f.p[0] = lds_read16<f16x8, OFF>(addr);
+	f.p[1] = lds_read16<f16x8, (int)PLANE_BYTES + OFF>(addr);
+	return f;
+}
+template <int OFF>
+__device__ __forceinline__ void lds_write16(unsigned addr, f32x4 v) {
+	asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+// until at most N of this wave's LDS instructions are outstanding (they complete in order): names the fragment that
+// must have arrived, so that the wait stays between its read and its use
+template <int N>
+__device__ __forceinline__ void lds_wait_but(PlanesT<FmtF16x2> &a) {
+	asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a.p[0]), "+v"(a.p[1]) : "n"(N));
+}
+constexpr int WIDE_AHEAD = 2;  // fragments requested ahead of the one in use (3 or 4: no faster, more registers)
+// The compiler inserts the wait states between a matrix instruction and a reader of its result only for readers it
+// knows; an LDS store written as text is not one.  24 wait states (a 32x32x16 result needs 19 before an LDS or memory
+// instruction may read it), tied to the registers so that they stay behind the matrix instructions.
+__device__ __forceinline__ void mfma_result_to_asm(f32x16 &acc) { asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc)); }
+
+// Same arguments and outputs as attn_prefill_planes_kernel<2, FmtF16x2>; plane images from attn_planes_wide_kernel.
+// Wave w: head = w / 2, dims 128 (w % 2) .. + 127; lane: c = lane % 32 (query), h = lane / 32.
+//
+// Time line.  Per key tile a wave goes through three phases, with a workgroup barrier after each:
+//   X1  its addend of the scores: 24 matrix instructions, 16 fragment reads, next to no vector work;
+//   X2  the partner's addend, mask, softmax, the weights as fp16 planes: about 200 vector instructions, no matrix work;
+//   Y   rescale the output (64 multiplies), then O^T += V^T P^T: 24 matrix instructions, 16 fragment reads.
+// A SIMD holds wave s and wave s + 4 and overlaps one wave's matrix instructions with the other's vector instructions
+// only if the two are in different phases (measured: 8 matrix instructions next to 64 multiplies take 360 clocks,
+// against 256 and 280 alone), so waves 4-7 (heads 2, 3) run one step behind waves 0-3: the SIMD sees X1 | Y, X2 | X1,
+// Y | X2.  A launch takes 3 ntiles + 1 steps.  Clocks between barriers, one workgroup of a long causal layer: 2,590,
+// 1,870 and 1,600 for the three kinds of step (the matrix instructions alone need 1,536, 768 and 768); with all
+// waves in one phase the kernel is 4 % slower.  Tried instead: the scores of tile t + 1 interleaved with the softmax
+// of tile t inside a wave, two phases per tile (5,700 clocks per tile on a single workgroup instead of 6,060, no
+// difference with all compute units busy); without the image copies a tile still takes 4,500 clocks.
+// Images: K of tile t is image 2t, V is image 2t + 1, image i lives in buffer i % 4.  In step 3t everyone requests its
+// share of K(t + 1), in step 3t + 1 of V(t + 1): the buffers they go to were last read in steps 3t - 2 and 3t, and
+// the images have three and four steps to arrive.  A wave's loads complete in the order it issued them, so "at most
+// n shares outstanding" is the test for the older ones.
+__global__ __launch_bounds__(512) void attn_prefill_wide_kernel(float *o, const float *q, const unsigned char *planes, int S, int ldq, int ldo,
+                                                                int is_sw, int window, const int4 *items, float *part_o, float *part_ml,
+                                                                int *range_flag) {
+	typedef FmtF16x2 F;
+	typedef PlanesT<F> Planes;
+	extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+	constexpr int BQ = WIDE_BQ, NW = 8, IMG_KB = (int)(WIDE_IMG / 1024), SHARE = IMG_KB / NW;  // 4 copy pieces per wave and image
+	constexpr int NKS = HD / 32, NDT = HD / 64;  // k steps of a wave's score product (8), output tiles of 32 dims it owns (4)
+	constexpr float EXP_SCALE = F::SSCALE * 1.44269504088896341f;  // 1/sqrt(head_dim) and log2(e) in one factor
+	static_assert(F::QSCALE == 1.0f, "the scores are scaled, not q");
+	unsigned rmax = 0u;
+
+	// the wave index as a scalar: what depends on it alone (roles, LDS regions, which copies a phase issues) then lives in scalar registers
+	const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int head = w >> 1, dh = w & 1, late = w >> 2, c = lane & 31, h = lane >> 5;
+	int q0 = plain_query_tile(is_sw) * BQ, slot = -1;
+	int4 item = int4{0, 0, 0, -1};
+	if (items != nullptr) {
+		item = items[blockIdx.x];
+		q0 = item.x * BQ;
+		slot = item.w;
+	}
+	int kb = (is_sw && q0 > window) ? ((q0 - window) / TK) * TK : 0;
+	int ke = (q0 + BQ < S) ? q0 + BQ : S;  // exclusive
+	if (items != nullptr) {
+		kb = item.y * TK;
+		ke = min(ke, item.z * TK);
+	}
+	const int ntiles = (ke - kb + TK - 1) / TK;
+	const unsigned char *img0 = planes + (size_t)(kb / TK) * 2 * WIDE_IMG;
+	const int nimg = 2 * ntiles;
+
+	const int qpos = q0 + c;
+	const int qrow = qpos < S ? qpos : S - 1;
+	const int klo = is_sw ? qpos - window : 0;
+
+	// Q planes: qp[ks] = dims 128 dh + 16 ks + 8 h .. + 7 of query c
+	Planes qp[NKS];
+	{
+		const float *qsrc = q + (size_t)qrow * ldq + head * HD + 128 * dh + 8 * h;
+#pragma unroll
+		for (int ks = 0; ks < NKS; ks++) {
+			const f32x4 x0 = *reinterpret_cast<const f32x4 *>(qsrc + 16 * ks), x1 = *reinterpret_cast<const f32x4 *>(qsrc + 16 * ks + 4);
+			float x[8];
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				x[e] = x0[e];
+				x[4 + e] = x1[e];
+			}
+			track_range<F>(rmax, x);
+			qp[ks] = split8<F>(x);
+		}
+	}
+	// The output is kept transposed, oacc[dt][4j + i] = O[query c][128 dh + 32 dt + 8j + 4h + i]: a lane then owns one
+	// query in the scores and in the output alike, and the running maximum, the running sum and the rescaling factor
+	// of that query never leave the lane.
+	f32x16 oacc[NDT], mine;
+#pragma unroll
+	for (int e = 0; e < 16; e++) mine[e] = 0.0f;
+#pragma unroll
+	for (int dt = 0; dt < NDT; dt++) oacc[dt] = mine;
+	float m_run = -INFINITY, l_run = 0.0f, alpha = 1.0f;  // the maximum in units of the unscaled scores
+	Planes pp[2];                                          // the weights of a tile, from its X2 to its Y
+
+	// from here on the only loads this wave has in flight are image copies, in the order it issues them
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	copy_image_to_lds<NW, IMG_KB>(img0, smem, lane, w);
+	copy_image_to_lds<NW, IMG_KB>(img0 + WIDE_IMG, smem + WIDE_IMG, lane, w);
+	wait_loads_in_flight<SHARE>();
+	tg_lds_barrier();  // image 0 is complete
+
+	const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+	const unsigned k_lane = (unsigned)(dh * NKS * 1024 + lane * 16), v_lane = (unsigned)(dh * NDT * 1024 + lane * 16);
+	const unsigned my_part = lds0 + 4u * (unsigned)WIDE_IMG + (unsigned)(w * 4096 + lane * 16);
+	const unsigned their_part = lds0 + 4u * (unsigned)WIDE_IMG + (unsigned)((w ^ 1) * 4096 + lane * 16);
+	// end of a step: all but the youngest `shares` of this wave's copies have arrived; the barrier completes the images
+	// and addends written by the other waves and releases what this step read
+	auto end_step = [&](int shares) {
+		if (shares == 2) {
+			wait_loads_in_flight<2 * SHARE>();
+		} else if (shares == 1) {
+			wait_loads_in_flight<SHARE>();
+		} else if (shares == 0) {
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+		}
+		tg_lds_barrier();
+	};
+	if (late) {  // step 0 of the late waves: only their share of K(1)
+		if (2 < nimg) copy_image_to_lds<NW, IMG_KB>(img0 + 2 * WIDE_IMG, smem + 2 * WIDE_IMG, lane, w);
+		end_step(-1);
+	}
+	for (int tile = 0; tile < ntiles; tile++) {
+		const bool more = tile + 1 < ntiles;  // images 2 tile + 2 and 2 tile + 3 exist
+		{
+			// ---- X1: this wave's addend of the scores, S^T = K Q^T over its 128 dims.  The early waves are in step 3 tile and
+			// request K(tile + 1), the late ones in step 3 tile + 1 and request V(tile + 1). ----
+			const int ci = 2 * tile + 2 + late;
+			const unsigned char *src = img0 + (size_t)ci * WIDE_IMG;
+			unsigned char *dst = smem + (size_t)(ci & 3) * WIDE_IMG;
+			const unsigned kaddr = lds0 + (unsigned)((2 * tile) & 3) * (unsigned)WIDE_IMG + k_lane;
+#pragma unroll
+			for (int e = 0; e < 16; e++) mine[e] = 0.0f;
+			Planes kf[WIDE_AHEAD];
+			static_for<WIDE_AHEAD>([&](auto tc) {
+				constexpr int t = decltype(tc)::value;
+				kf[t] = read_wide<t * 1024>(kaddr);
+			});
+			static_for<NKS>([&](auto tc) {
+				constexpr int t = decltype(tc)::value;
+				constexpr int later = (NKS - 1 - t < WIDE_AHEAD - 1) ? NKS - 1 - t : WIDE_AHEAD - 1;  // fragments requested after this one
+				lds_wait_but<2 * later>(kf[t % WIDE_AHEAD]);
+				mine = mfma32_terms(kf[t % WIDE_AHEAD], qp[t], mine);
+				if constexpr (t + WIDE_AHEAD < NKS) kf[t % WIDE_AHEAD] = read_wide<(t + WIDE_AHEAD) * 1024>(kaddr);
+				if constexpr (t < SHARE) {
+					if (more) copy_image_piece<NW>(src, dst, lane, w, t);
+				}
+			});
+			mfma_result_to_asm(mine);
+			static_for<4>([&](auto jc) {
+				constexpr int j = decltype(jc)::value;
+				lds_write16<j * 1024>(my_part, f32x4{mine[4 * j], mine[4 * j + 1], mine[4 * j + 2], mine[4 * j + 3]});
+			});
+			// late waves, step 3 tile + 1: V(tile) must be complete for the early waves' Y; K(tile + 1) and V(tile + 1) are younger
+			end_step(late ? (more ? 2 : 0) : -1);
+		}
+		{
+			// ---- X2: softmax.  The early waves (step 3 tile + 1) request V(tile + 1) here. ----
+			if (!late && more) copy_image_to_lds<NW, IMG_KB>(img0 + (size_t)(2 * tile + 3) * WIDE_IMG, smem + (size_t)((2 * tile + 3) & 3) * WIDE_IMG, lane, w);
+			const int t0 = kb + tile * TK;  // first key of the tile
+			f32x4 th[4];
+			static_for<4>([&](auto jc) {
+				constexpr int j = decltype(jc)::value;
+				th[j] = lds_read16<f32x4, j * 1024>(their_part);
+			});
+			asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(th[0]), "+v"(th[1]), "+v"(th[2]), "+v"(th[3]));
+			float sv[16];  // sv[4j + i]: key t0 + 8j + 4h + i of query c; a sum of two addends is the same in either order
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+#pragma unroll
+				for (int i = 0; i < 4; i++) sv[4 * j + i] = mine[4 * j + i] + th[j][i];
+			// only the tiles on the diagonal and at the far end of a window hold keys that some query must not see
+			if (t0 + TK - 1 > q0 || (is_sw && t0 < q0 + BQ - 1 - window)) {
+#pragma unroll
+				for (int j = 0; j < 4; j++)
+#pragma unroll
+					for (int i = 0; i < 4; i++) {
+						const int key = t0 + 8 * j + 4 * h + i;
+						if (key > qpos || key < klo) sv[4 * j + i] = -INFINITY;
+					}
+			}
+			float tmax = sv[0];
+#pragma unroll
+			for (int e = 1; e < 16; e++) tmax = fmaxf(tmax, sv[e]);
+			tmax = fmaxf(tmax, tg_red_partner<32>(tmax));
+			const float m_new = fmaxf(m_run, tmax);
+			const float m_ref = (m_new == -INFINITY) ? 0.0f : m_new;  // no valid key yet
+			alpha = __builtin_amdgcn_exp2f((m_run - m_ref) * EXP_SCALE);
+			float psum = 0.0f;
+#pragma unroll
+			for (int e = 0; e < 16; e++) {
+				sv[e] = __builtin_amdgcn_exp2f((sv[e] - m_ref) * EXP_SCALE);
+				psum += sv[e];
+			}
+			psum += tg_red_partner<32>(psum);
+			l_run = fmaf(l_run, alpha, psum);
+			m_run = m_new;
+			pp[0] = split8<F>(sv);
+			pp[1] = split8<F>(sv + 8);
+			// early waves, step 3 tile + 1: as above; late waves, step 3 tile + 2: K(tile + 1) must be complete, V(tile + 1) is younger
+			end_step(more ? (late ? 1 : 2) : 0);
+		}
+		{
+			// ---- Y: O^T = alpha O^T + V^T P^T.  The late waves (step 3 tile + 3) request K(tile + 2) here. ----
+			const int ci = 2 * tile + 4;
+			const bool copy = late && ci < nimg;
+			const unsigned char *src = img0 + (size_t)ci * WIDE_IMG;
+			unsigned char *dst = smem + (size_t)(ci & 3) * WIDE_IMG;
+			const unsigned vaddr = lds0 + (unsigned)((2 * tile + 1) & 3) * (unsigned)WIDE_IMG + v_lane;
+			Planes vf[WIDE_AHEAD];
+			static_for<WIDE_AHEAD>([&](auto tc) {
+				constexpr int t = decltype(tc)::value;
+				vf[t] = read_wide<(t / NDT) * 8192 + (t % NDT) * 1024>(vaddr);
+			});
+#pragma unroll
+			for (int dt = 0; dt < NDT; dt++) oacc[dt] = oacc[dt] * alpha;
+			static_for<2 * NDT>([&](auto sc) {
+				constexpr int st = decltype(sc)::value, s = st / NDT, dt = st % NDT;
+				constexpr int later = (2 * NDT - 1 - st < WIDE_AHEAD - 1) ? 2 * NDT - 1 - st : WIDE_AHEAD - 1;
+				constexpr int nx = st + WIDE_AHEAD;
+				lds_wait_but<2 * later>(vf[st % WIDE_AHEAD]);
+				oacc[dt] = mfma32_terms(vf[st % WIDE_AHEAD], pp[s], oacc[dt]);
+				if constexpr (nx < 2 * NDT) vf[st % WIDE_AHEAD] = read_wide<(nx / NDT) * 8192 + (nx % NDT) * 1024>(vaddr);
+				if constexpr (st < SHARE) {
+					if (copy) copy_image_piece<NW>(src, dst, lane, w, st);
+				}
+			});
+			// early waves, step 3 tile + 2: K(tile + 1) must be complete, V(tile + 1) is younger
+			end_step(late ? -1 : (more ? 1 : 0));
+		}
+	}
+	if (!late) end_step(-1);  // the last step of the early waves
+
+	report_range<F>(rmax, range_flag);
+	if (slot >= 0) {
+		float *po = part_o + (((size_t)slot * BQ + c) * NH + head) * HD + 128 * dh + 4 * h;
+#pragma unroll
+		for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+				*reinterpret_cast<f32x4 *>(po + 32 * dt + 8 * j) = f32x4{oacc[dt][4 * j], oacc[dt][4 * j + 1], oacc[dt][4 * j + 2], oacc[dt][4 * j + 3]};
+		if (h == 0 && dh == 0) {
+			float *pm = part_ml + (((size_t)slot * BQ + c) * NH + head) * 2;
+			pm[0] = m_run * F::SSCALE;  // in units of the scaled scores, like the other kernels
+			pm[1] = l_run;
+		}
+		return;
+	}
+	if (qpos < S) {
+		float *op = o + (size_t)qpos * ldo + head * HD + 128 * dh + 4 * h;
+#pragma unroll
+		for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+				*reinterpret_cast<f32x4 *>(op + 32 * dt + 8 * j) = f32x4{oacc[dt][4 * j] / l_run, oacc[dt][4 * j + 1] / l_run, oacc[dt][4 * j + 2] / l_run, oacc[dt][4 * j + 3] / l_run};
+	}
+}
+
 // One workgroup per query position of a split query tile; wave = head, lane = 4 consecutive dims.
 // split[b] = {query tile, first slot, number of chunks}.
 __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S, int ldo, const int4 *split, const float *part_o,
@@ -974,7 +1335,9 @@ __global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o
 int g_attn_prefill_planes = 1;
 constexpr int TG_ATTN_PLANES_MIN_TOKENS = 2048;
 size_t tg_attn_prefill_planes_bytes(int S) { return (size_t)((S + TK - 1) / TK) * 2 * plane_img<FmtBf16x3>(); }  // the larger format
-// split path: 1 (default) = two fp16 planes, three products; 0 = three bf16 planes, six products
+// split path: 1 (default) = two fp16 planes, three products, on 32x32x16 matrix instructions where the plane images
+// and 32-query workgroups are in use; 2 = the same planes on 16x16x32 instructions throughout; 0 = three bf16 planes,
+// six products
 int g_attn_prefill_f16 = 1;
 
 int g_attn_prefill_split = 1;  // 0: fp32 matrix path; 1 (default): split-precision matrix path (two fp16 or three bf16 planes); 2: the same, always with 32-query workgroups
@@ -1062,6 +1425,19 @@ void launch_split(dim3 grid, int tq, bool planes, float *o, const float *q, cons
 		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_split_kernel<1, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged);
 		(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_split_kernel<2, F>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)staged);
 		lds_set = true;
+	}
+	if constexpr (std::is_same<F, FmtF16x2>::value) {
+		if (planes && tq == WIDE_BQ && g_attn_prefill_f16 == 1) {  // 32 queries per matrix instruction
+			static bool wide_set = false;
+			if (!wide_set) {
+				(void)hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_wide_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)WIDE_LDS);
+				wide_set = true;
+			}
+			unsigned char *pw = (unsigned char *)planes_ws;
+			hipLaunchKernelGGL(attn_planes_wide_kernel, dim3((unsigned)((S + TK - 1) / TK)), dim3(PNT), 0, s, pw, k, v, S, ldkv, range_flag);
+			hipLaunchKernelGGL(attn_prefill_wide_kernel, grid, dim3(512), WIDE_LDS, s, o, q, pw, S, ldq, ldo, is_sw, window, items, po, pml, range_flag);
+			return;
+		}
 	}
 	if (planes) {
 		unsigned char *pw = (unsigned char *)planes_ws;
