@@ -388,6 +388,8 @@ def test_prefill_attention_modes_agree_inside_the_forward(tg, oracle, n_prompt):
         assert normrel(out[key][1], out[combos[0]][1]) < 2e-5
     # the plane images hold the same planes the staging code computes: not a bit differs
     assert np.array_equal(out[(2, 2, 2)][1], out[(2, 0, 1)][1])
+    # ... and the 32x32x16 kernel sums in another order: other last bits, which shows that it is the one that ran
+    assert not np.array_equal(out[(2, 2, 1)][1], out[(2, 2, 2)][1])
 
 
 def test_one_session_many_prompt_lengths(tg, oracle):
