@@ -923,9 +923,11 @@ __global__ __launch_bounds__(PNT) void attn_planes_wide_kernel(unsigned char *pl
 	vec *Kimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * WIDE_IMG);
 	vec *Vimg = reinterpret_cast<vec *>(planes + (size_t)tile * 2 * WIDE_IMG + WIDE_IMG);
 	unsigned rmax = 0u;
+	// one workgroup for the K image of a tile (blockIdx.y == 0), one for its V image: a prompt of 4096 tokens has only 128 tiles
 	// K: unit = (key, piece of 8 dims): 32 consecutive threads read one key's 1 KB row
 #pragma unroll
 	for (int u = 0; u < 4; u++) {
+		if (blockIdx.y != 0) break;
 		const int unit = tid + PNT * u, piece = unit & 31, key = unit >> 5;
 		const int j = tile * TK + key;
 		float x[8];
@@ -945,6 +947,7 @@ __global__ __launch_bounds__(PNT) void attn_planes_wide_kernel(unsigned char *pl
 	// V: unit = (s, dt, lane): dim 32 dt + lane % 32, keys 16 s + 4 h + {0..3} and 16 s + 8 + 4 h + {0..3}
 #pragma unroll
 	for (int u = 0; u < 4; u++) {
+		if (blockIdx.y != 1) break;
 		const int unit = tid + PNT * u, lane = unit & 63, dt = (unit >> 6) & 7, s = unit >> 9;
 		const int d = 32 * dt + (lane & 31), h = lane >> 5;
 		float x[8];
@@ -1434,7 +1437,7 @@ void launch_split(dim3 grid, int tq, bool planes, float *o, const float *q, cons
 				wide_set = true;
 			}
 			unsigned char *pw = (unsigned char *)planes_ws;
-			hipLaunchKernelGGL(attn_planes_wide_kernel, dim3((unsigned)((S + TK - 1) / TK)), dim3(PNT), 0, s, pw, k, v, S, ldkv, range_flag);
+			hipLaunchKernelGGL(attn_planes_wide_kernel, dim3((unsigned)((S + TK - 1) / TK), 2), dim3(PNT), 0, s, pw, k, v, S, ldkv, range_flag);
 			hipLaunchKernelGGL(attn_prefill_wide_kernel, grid, dim3(512), WIDE_LDS, s, o, q, pw, S, ldq, ldo, is_sw, window, items, po, pml, range_flag);
 			return;
 		}
