@@ -239,6 +239,9 @@ int tg_debug_repeat_kernel(tg_session *s, int kernel_class, int layer, int repea
  * accesses and no cache is written back or invalidated.  Every wait gives up after max_spins polls (*timed_out = 1:
  * the figure is meaningless), so the kernel always ends. */
 int tg_debug_launch_chain(int n_launches, int workgroups, double *us_per_launch);
+int tg_debug_handover(int rounds, int workgroups, int barrier, int data, int words_per_wg, int max_spins, double *us_per_round,
+                      int *timed_out, int *wrong_sums, int *xcd_of_wg);
+int tg_set_fused_decode(int enable, int gemv_workgroups, int max_spins);
 int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins, double *us_per_barrier, int *timed_out);
 
 /* The rate the integer matrix cores sustain on this machine (no counterpart in the reference: measurement aid).

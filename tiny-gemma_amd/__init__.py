@@ -14,7 +14,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libtinygemma_hip.so")
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip", "tg_repack.hip", "tg_probe.hip"]
+SOURCES = ["tg_api.hip", "tg_gemv.hip", "tg_attn.hip", "tg_attn_prefill.hip", "tg_rows.hip", "tg_gemm_mfma.hip", "tg_sample.hip", "tg_repack.hip", "tg_probe.hip", "tg_decode_fused.hip"]
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
                # leading scalar kernel arguments are preloaded into SGPRs by the dispatcher (no s_load round trip)
@@ -38,14 +38,33 @@ class Config(C.Structure):
                 ("n_kv", C.c_int), ("rope_theta", C.c_float), ("rope_theta_local", C.c_float), ("window_pattern", C.c_int)]
 
 
-def build_library(verbose=False):
-    """hipcc cross-compiles for gfx950 without a GPU."""
-    cmd = ["hipcc"] + HIPCC_FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB_PATH]
+def build_library(verbose=False, changed_only=False):
+    """hipcc cross-compiles for gfx950 without a GPU: one object per source, compiled in parallel, then one link.
+    changed_only: recompile only sources newer than their object (a development convenience; the default compiles all)."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    headers = [os.path.join(CSRC, h) for h in ("tg_internal.h", "tg_gemv_parts.h", "tg_attn_decode.h")] + [os.path.join(HERE, "..", "include", "tinygemma_hip.h")]
+
+    def compile_one(src):
+        path, obj = os.path.join(CSRC, src), os.path.join(objdir, src + ".o")
+        if changed_only and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in [path] + headers):
+            return obj
+        cmd = ["hipcc"] + flags + ["-c", path, "-o", obj]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed on " + src + ":\n" + r.stderr[-4000:])
+        if verbose:
+            print(" ".join(cmd))
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + r.stderr[-4000:])
-    if verbose:
-        print(" ".join(cmd))
+        raise RuntimeError("hipcc link failed:\n" + r.stderr[-4000:])
     return LIB_PATH
 
 
@@ -106,6 +125,7 @@ def lib():
     L.tg_qgemm_dev_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_debug_launch_chain.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
     L.tg_debug_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p]
+    L.tg_debug_handover.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p, c_i32p, c_i32p]
     L.tg_debug_gemm_launches.argtypes = [C.POINTER(C.c_longlong)] * 3
     L.tg_debug_mfma_clock.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.tg_decode_profile.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double), c_i32p]

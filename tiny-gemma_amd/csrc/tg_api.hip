@@ -42,6 +42,10 @@ bool g_gemm_split = true;       // prefill: products that would leave most compu
 int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_chain_picks = true;  // inside a batch of greedy decode steps the next step's first launch finishes the previous pick
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
+// Decode: all layers of a step in one launch of resident workgroups (tg_decode_fused.hip) instead of 5 launches per layer.
+// g_fused_ng: GEMV workgroups of that launch (0: one per compute unit, less the attention workgroups).
+int g_fused = 0, g_fused_ng = 0, g_fused_spins = 1 << 20;
+unsigned long long *g_fused_ts = nullptr;  // device buffer of tg_debug_fused_timestamps while it runs
 // Counts changes of the tuning knobs.  A captured decode step bakes the knobs of its capture into its launches
 // (prefetch workgroups, grid limits, attention geometry), so a session drops its captured graphs when this has moved.
 unsigned g_knob_epoch = 0;
@@ -200,6 +204,7 @@ int tg_fail(int code, const std::string &msg) {
 }
 
 hipStream_t tg_probe_stream() { return g_inited ? g_stream : nullptr; }  // for the timing probes of tg_probe.hip
+int tg_probe_n_cu() { return g_n_cu; }
 
 struct tg_qweight {
 	PackedMat p;
@@ -321,6 +326,16 @@ struct tg_session {
 	void *pf_ws = nullptr;
 	size_t pf_ws_bytes = 0;
 	AttnPlanDev pf_plan, pf_plan_local;
+	// one-kernel decode step (tg_decode_fused.hip): built on first use; fused_state 0 = not built yet, 1 = usable,
+	// -1 = not usable for this model or device, or a wait timed out (the session then stays on the launch path)
+	int fused_state = 0, fused_variant = -1;
+	unsigned fused_epoch = 0;      // g_knob_epoch that fused.ng and fused_variant were derived under
+	bool fused_unchecked = false;  // fused launches have been enqueued since the error word was last read
+	TgFused fused;                 // the launch-independent fields
+	TgFusedLayer *fused_layers = nullptr;
+	float *fused_xch = nullptr;
+	unsigned *fused_sync = nullptr;
+	unsigned fused_all = 0, fused_attn = 0;  // host mirrors of the arrival counters
 };
 
 namespace {
@@ -830,7 +845,8 @@ void tg_session_destroy(tg_session *s) {
 	s->graphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
-	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf, s->zeros, s->blk_x, s->blk_y};
+	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf, s->zeros, s->blk_x, s->blk_y, s->fused_layers,
+	              s->fused_xch, s->fused_sync};
 	for (void *p : ps)
 		if (p) (void)hipFree(p);
 	s->pf_plan.release();
@@ -985,6 +1001,165 @@ static int session_usable(const tg_session *s) {
 	if (!s) return tg_fail(TG_ERR_BAD_ARG, "null session");
 	if (!s->m || !s->m->loaded) return tg_fail(TG_ERR_STATE, "the session's model has no weights (destroyed, or a load failed)");
 	return TG_OK;
+}
+
+// ---- the one-kernel decode step ---------------------------------------------------------------------------
+static TgFusedMat fused_mat(const PackedMat &p) { return TgFusedMat{p.K, p.C, p.lc_shift, p.ntiles}; }
+
+// Keys per attention workgroup of the fused step: TG_FUSED_ATTN_WGS workgroups cover the context.  Up to
+// TG_ATTN_MERGE_MAX * g_attn_merge_chunk keys that is what the launch path does as well; 0: too many keys for it.
+static int fused_chunk(int valid) {
+	const int c = (valid + TG_FUSED_ATTN_WGS - 1) / TG_FUSED_ATTN_WGS;
+	const int c16 = (c + 15) / 16 * 16;
+	return c16 <= 256 ? c16 : 0;
+}
+
+// Builds the per-session tables of the fused step on first use.  Leaves fused_state at 1 (usable) or -1.
+static int fused_prepare(tg_session *s) {
+	if (s->fused_state != 0) return TG_OK;
+	s->fused_state = -1;
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	const int L = c.n_layers;
+	if (!tg_fused_supported(g_n_cu)) return TG_OK;
+	TgFused &f = s->fused;
+	memset(&f, 0, sizeof(f));
+	f.L = L;
+	f.hidden = c.hidden_size;
+	f.mqkv = fused_mat(m->L[0].qkv);
+	f.mo = fused_mat(m->L[0].o);
+	f.mug = fused_mat(m->L[0].ug);
+	f.md = fused_mat(m->L[0].d);
+	auto al = [](int floats) { return (floats + 63) / 64 * 64; };  // regions start on 256-byte boundaries
+	int off = 0;
+	f.off_qkv = off;
+	off += al(c.n_head * c.head_dim + 2 * c.head_dim);
+	f.off_pacc = off;
+	off += al(TG_FUSED_ATTN_WGS * c.n_head * c.head_dim);
+	f.off_pml = off;
+	off += al(TG_FUSED_ATTN_WGS * c.n_head * 2);
+	f.off_o = off;
+	off += al(c.hidden_size);
+	f.off_h = off;
+	off += al(c.intermediate_size);
+	f.off_d = off;
+	off += al(c.hidden_size);
+	f.layer_stride = (size_t)off;
+	std::vector<TgFusedLayer> hl((size_t)L);
+	for (int l = 0; l < L; l++) {
+		const LayerDev &Ld = m->L[(size_t)l];
+		TgFusedLayer &o = hl[(size_t)l];
+		o.Wqkv = Ld.qkv.W;
+		o.Wo = Ld.o.W;
+		o.Wug = Ld.ug.W;
+		o.Wd = Ld.d.W;
+		o.sqkv = Ld.qkv.scales;
+		o.so = Ld.o.scales;
+		o.sug = Ld.ug.scales;
+		o.sd = Ld.d.scales;
+		o.apre = Ld.apre;
+		o.apost = Ld.apost;
+		o.mpre = Ld.mpre;
+		o.mpost = Ld.mpost;
+		o.rms_q = Ld.rms_q;
+		o.rms_k = Ld.rms_k;
+		o.kc = s->kc[(size_t)l];
+		o.vc = s->vc[(size_t)l];
+		o.max_pos = s->max_pos[(size_t)l];
+		o.is_sw = Ld.is_sw ? 1 : 0;
+	}
+	TG_HIP(hipMalloc((void **)&s->fused_layers, sizeof(TgFusedLayer) * (size_t)L));
+	TG_HIP(hipMemcpy(s->fused_layers, hl.data(), sizeof(TgFusedLayer) * (size_t)L, hipMemcpyHostToDevice));
+	TG_HIP(hipMalloc((void **)&s->fused_xch, sizeof(float) * f.layer_stride * (size_t)L));
+	TG_HIP(hipMemset(s->fused_xch, 0, sizeof(float) * f.layer_stride * (size_t)L));
+	TG_HIP(hipMalloc((void **)&s->fused_sync, sizeof(unsigned) * TG_FUSED_SYNC_WORDS));
+	TG_HIP(hipMemset(s->fused_sync, 0, sizeof(unsigned) * TG_FUSED_SYNC_WORDS));
+	s->fused_all = s->fused_attn = 0;
+	f.layers = s->fused_layers;
+	f.wte = m->wte;
+	f.wte_scales = m->wte_scales;
+	f.vocab = c.n_vocab;
+	f.emb_scale = (float)sqrt((double)c.hidden_size);  // ops.hpp:586
+	f.cos_g = s->cos_g;
+	f.sin_g = s->sin_g;
+	f.cos_l = s->cos_l;
+	f.sin_l = s->sin_l;
+	f.lut = s->lut;
+	f.gmin = s->gmin;
+	f.geps = s->geps;
+	f.lut_size = s->lut_size;
+	f.xr = s->xr;
+	f.xch = s->fused_xch;
+	f.sync = s->fused_sync;
+	s->fused_state = 1;
+	s->fused_epoch = g_knob_epoch - 1;  // the workgroup count and the kernel variant are chosen by fused_usable
+	return TG_OK;
+}
+
+// Whether the next decode step of the session can run as one launch, and its attention geometry if so.
+static bool fused_usable(tg_session *s, int *chunk_local, int *chunk_global) {
+	if (!g_fused || s->fused_state != 1) return false;
+	if (s->fused_epoch != g_knob_epoch) {  // the knobs have moved: workgroups of the launch, kernel instantiation
+		s->fused_epoch = g_knob_epoch;
+		s->fused.ng = g_fused_ng > 0 ? g_fused_ng : g_n_cu - TG_FUSED_ATTN_WGS;
+		// one workgroup per compute unit, so that all of them are resident at once
+		s->fused_variant = s->fused.ng + TG_FUSED_ATTN_WGS <= g_n_cu ? tg_fused_variant(s->fused) : -1;
+	}
+	if (s->fused_variant < 0) return false;
+	const tg_config &c = s->m->cfg;
+	*chunk_local = fused_chunk(std::min(s->pos + 1, c.n_pos_local));
+	*chunk_global = fused_chunk(std::min(s->pos + 1, c.n_pos));
+	return *chunk_local > 0 && *chunk_global > 0;
+}
+
+// The layers of a decode step as one launch; the LM head follows as a launch of its own.
+static void launch_fused_layers(tg_session *s, int chunk_local, int chunk_global) {
+	tg_model *m = s->m;
+	const tg_config &c = m->cfg;
+	TgFused f = s->fused;
+	f.tok = s->ctr + 4;
+	if (s->pick_pending) {  // this launch finishes the previous step's greedy pick
+		f.am_val = s->blk_val;
+		f.am_idx = s->blk_idx;
+		f.am_n = m->lm.ntiles;
+		f.am_ctr = s->ctr;
+		f.am_log = s->tok_log;
+		s->pick_pending = false;
+	}
+	f.pos = s->pos;
+	f.bp_local = s->bp_local;
+	f.bp_global = s->bp_global;
+	f.chunk_local = chunk_local;
+	f.chunk_global = chunk_global;
+	f.all_base = s->fused_all;
+	f.attn_base = s->fused_attn;
+	f.max_spins = g_fused_spins;
+	f.ts = g_fused_ts;
+	tg_launch_decode_fused(f, s->fused_variant, g_stream);
+	// what the launch adds to the counters: 4 arrivals of every GEMV workgroup per layer, one of every attention
+	// workgroup that has keys
+	s->fused_all += 4u * (unsigned)c.n_layers * (unsigned)f.ng;
+	for (int l = 0; l < c.n_layers; l++) {
+		const int valid = std::min(s->pos + 1, s->max_pos[(size_t)l]);
+		const int ch = m->L[(size_t)l].is_sw ? chunk_local : chunk_global;
+		s->fused_attn += (unsigned)((valid + ch - 1) / ch);
+	}
+	s->fused_unchecked = true;
+}
+
+// After a stream synchronisation: did a wait inside a fused launch give up?  Then the results since the last check are
+// not valid; the session stays on the launch path from here on.
+static int fused_check(tg_session *s) {
+	if (!s->fused_unchecked) return TG_OK;
+	s->fused_unchecked = false;
+	unsigned err = 0;
+	TG_HIP(hipMemcpy(&err, s->fused_sync + 16 * 32, sizeof(unsigned), hipMemcpyDeviceToHost));
+	if (err == 0) return TG_OK;
+	s->fused_state = -1;
+	s->fused_all = s->fused_attn = 0;
+	TG_HIP(hipMemset(s->fused_sync, 0, sizeof(unsigned) * TG_FUSED_SYNC_WORDS));
+	return tg_fail(TG_ERR_STATE, "one-kernel decode step: a bounded wait between workgroups gave up (the workgroups were not all resident, or the device "
+	                             "is shared); the decode steps since the last read-back are not valid.  Reset the session; it now uses one launch per projection");
 }
 
 // ---- the launches of a decode step, one function per kernel (modules.hpp:135-220, 242-246) ----
@@ -1152,7 +1327,19 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 	if (prof) {                                    \
 		TG_HIP(prof->mark(k));                     \
 	}
-	for (int l = 0; l < L; l++) {
+	// all layers in one launch where that is possible (not when single kernels are timed or repeated, not in a captured step)
+	int fch_l = 0, fch_g = 0;
+	bool fused = false;
+	if (g_fused && !prof && !only && !full_grid) {
+		if (int rc = fused_prepare(s)) return rc;
+		fused = fused_usable(s, &fch_l, &fch_g);
+	}
+	const float *last_pend = s->d_out;
+	if (fused) {
+		launch_fused_layers(s, fch_l, fch_g);
+		last_pend = s->fused_xch + (size_t)(L - 1) * s->fused.layer_stride + s->fused.off_d;
+	}
+	for (int l = 0; l < L && !fused; l++) {
 		float *xr_in = s->xr + (size_t)(2 * l) * h, *xr_mid = s->xr + (size_t)(2 * l + 1) * h;
 		TG_MARK(TG_KC_QKV);
 		if (l == 0) {
@@ -1171,7 +1358,7 @@ static int enqueue_decode_step(tg_session *s, StepProfile *prof, bool full_grid,
 		TG_DO(TG_KC_DOWN, l, launch_down(s, l));
 	}
 	TG_MARK(TG_KC_LMHEAD);
-	TG_DO(TG_KC_LMHEAD, 0, launch_lmhead(s, s->d_out, m->L[(size_t)L - 1].mpost, s->xr + (size_t)(2 * L - 1) * h, s->xr + (size_t)(2 * L) * h));
+	TG_DO(TG_KC_LMHEAD, 0, launch_lmhead(s, last_pend, m->L[(size_t)L - 1].mpost, s->xr + (size_t)(2 * L - 1) * h, s->xr + (size_t)(2 * L) * h));
 	TG_MARK(TG_KC_ARGMAX);
 	if (!only) {
 		if (s->sampling)
@@ -1203,6 +1390,7 @@ int tg_forward_decode(tg_session *s, int32_t id, float *logits, int32_t *argmax)
 	int32_t tok = -1;
 	TG_HIP(hipMemcpyAsync(&tok, s->ctr + 4, sizeof(int), hipMemcpyDeviceToHost, g_stream));
 	TG_HIP(hipStreamSynchronize(g_stream));
+	if (int rc = fused_check(s)) return rc;
 	if (argmax) *argmax = tok;
 	if (s->taps) {  // taps now describe the decode step
 		s->taps = nullptr;
@@ -1417,7 +1605,37 @@ int tg_set_chain_picks(int enable) {
 	return TG_OK;
 }
 
+int tg_set_fused_decode(int enable, int gemv_workgroups, int max_spins) {
+	if (gemv_workgroups < 0 || max_spins < 0 || max_spins > (1 << 22)) return tg_fail(TG_ERR_BAD_ARG, "bad argument (max_spins <= 2^22)");
+	g_fused = enable != 0;
+	g_fused_ng = gemv_workgroups;
+	g_fused_spins = max_spins > 0 ? max_spins : 1 << 20;
+	g_knob_epoch++;
+	return TG_OK;
+}
+
+// One fused decode step of the session with timestamps: out[L][24] ticks of the 100 MHz counter (see TgFused::ts)
+int tg_debug_fused_timestamps(tg_session *s, unsigned long long *out, int n_layers) {
+	if (int rc = session_usable(s)) return rc;
+	const int L = s->m->cfg.n_layers;
+	if (!out || n_layers != L) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	unsigned long long *d = nullptr;
+	TG_HIP(hipMalloc((void **)&d, sizeof(unsigned long long) * 24 * (size_t)L));
+	TG_HIP(hipMemset(d, 0, sizeof(unsigned long long) * 24 * (size_t)L));
+	g_fused_ts = d;
+	int rc = tg_decode_enqueue(s, 1);
+	g_fused_ts = nullptr;
+	if (rc == TG_OK && hipStreamSynchronize(g_stream) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipStreamSynchronize failed");
+	if (rc == TG_OK) rc = fused_check(s);
+	if (rc == TG_OK && hipMemcpy(out, d, sizeof(unsigned long long) * 24 * (size_t)L, hipMemcpyDeviceToHost) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+	(void)hipFree(d);
+	return rc;
+}
+
 int tg_reset_knobs() {
+	g_fused = 0;
+	g_fused_ng = 0;
+	g_fused_spins = 1 << 20;
 	g_gemm_mfma = 1;
 	g_prefetch_plan = 0;
 	g_prefetch_blocks = 128;
@@ -1476,6 +1694,7 @@ int tg_decode_profile(tg_session *s, int n_steps, double *ms_sum, int *launches)
 int tg_session_read_ids(tg_session *s, int32_t *ids, int max_ids, int *n_out) {
 	if (!s || !ids) return tg_fail(TG_ERR_BAD_ARG, "null argument");
 	TG_HIP(hipStreamSynchronize(g_stream));
+	if (int rc = fused_check(s)) return rc;
 	const int n = std::min(max_ids, s->steps);
 	if (n > 0) TG_HIP(hipMemcpy(ids, s->tok_log, sizeof(int) * (size_t)n, hipMemcpyDeviceToHost));
 	if (n_out) *n_out = n;
@@ -1980,6 +2199,7 @@ int tg_session_tap(tg_session *s, int b, float *out, int rows) {
 	const tg_config &c = s->m->cfg;
 	if (b < 0 || b > 2 * c.n_layers) return tg_fail(TG_ERR_BAD_ARG, "no such block");
 	TG_HIP(hipStreamSynchronize(g_stream));
+	if (int rc = fused_check(s)) return rc;
 	const size_t h = (size_t)c.hidden_size;
 	if (s->taps) {
 		if (rows != s->tap_rows)
@@ -1997,6 +2217,7 @@ int tg_session_kv(tg_session *s, int layer, float *keys, float *values, int *pos
 	const tg_config &c = s->m->cfg;
 	if (layer < 0 || layer >= c.n_layers) return tg_fail(TG_ERR_BAD_ARG, "no such layer");
 	TG_HIP(hipStreamSynchronize(g_stream));
+	if (int rc = fused_check(s)) return rc;
 	const size_t bytes = sizeof(float) * (size_t)s->max_pos[(size_t)layer] * c.head_dim;
 	if (keys) TG_HIP(hipMemcpy(keys, s->kc[(size_t)layer], bytes, hipMemcpyDeviceToHost));
 	if (values) TG_HIP(hipMemcpy(values, s->vc[(size_t)layer], bytes, hipMemcpyDeviceToHost));

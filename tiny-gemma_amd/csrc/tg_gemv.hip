@@ -21,126 +21,11 @@
 // LUT-GeLU(gate) * up, or logits write-out plus the per-workgroup stage of the greedy argmax.
 
 #include "tg_internal.h"
+#include "tg_gemv_parts.h"
+
+using namespace tgp;
 
 namespace {
-
-constexpr int NT = 256;     // threads per workgroup (4 waves)
-constexpr int NWAVE = 4;
-constexpr int LUT_LDS = 1024;  // GeLU tables up to this size are staged in LDS (one 16-byte load per lane)
-constexpr uint32_t STEP_BYTES = NT * 16u;  // the workgroup reads 4 KiB of its slab per step
-
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-// Cache policy bits of a weight load.  TG_W_NT marks the data as non-temporal (read once): measured on the
-// 302 MB LM head, rotating over three copies so that nothing is left in the memory-side cache from the
-// previous launch, the stream runs at 6.4 TB/s with it and 5.6 TB/s without.
-constexpr int TG_W_DEFAULT = 0, TG_W_NT = 2;
-// 16-byte weight loads in flight per lane of the LM head, which streams 36 steps per tile.  The per-layer
-// projections cover 1 to 9 steps and are bound by latency, not by loads in flight: measured on whole decode steps, a
-// fixed 2 is 4 % faster than a fixed 8 (1B shape; 8 % on the 270m shape); tg_gemv_depth picks theirs per shape.
-constexpr int TG_DEPTH_STREAM = 8;
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
-	return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, bytes, 0x00020000);
-}
-template <int AUX>
-__device__ __forceinline__ i32x4 ldw(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
-	return __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, AUX);
-}
-__device__ __forceinline__ f32x4 ldx(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
-	i32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
-	return __builtin_bit_cast(f32x4, t);
-}
-
-__device__ __forceinline__ float wave_sum(float v) { return tg_wave_sum(v); }
-
-// Sum over the workgroup; every thread gets the same value (fixed order).
-__device__ __forceinline__ float block_sum(float v, float *sred) {
-	v = wave_sum(v);
-	__syncthreads();
-	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
-	__syncthreads();
-	return (sred[0] + sred[1]) + (sred[2] + sred[3]);
-}
-
-__device__ __forceinline__ float b2f(int d, int j) {  // signed byte j of d -> float (exact)
-	return (float)(int8_t)(d >> (8 * j));
-}
-
-// ops.hpp:41-51: truncating index, below the table -> 0, above -> identity
-__device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin, float geps, int size) {
-	int idx = (int)((x - gmin) / geps);
-	if (idx < 0) return 0.0f;
-	if (idx >= size) return x;
-	return lut[idx];
-}
-
-__device__ __forceinline__ void fma16(float acc[4], const i32x4 v, const f32x4 xv) {
-	const int d0 = v.x, d1 = v.y, d2 = v.z, d3 = v.w;
-	acc[0] = fmaf(xv.x, b2f(d0, 0), acc[0]); acc[0] = fmaf(xv.y, b2f(d0, 1), acc[0]);
-	acc[0] = fmaf(xv.z, b2f(d0, 2), acc[0]); acc[0] = fmaf(xv.w, b2f(d0, 3), acc[0]);
-	acc[1] = fmaf(xv.x, b2f(d1, 0), acc[1]); acc[1] = fmaf(xv.y, b2f(d1, 1), acc[1]);
-	acc[1] = fmaf(xv.z, b2f(d1, 2), acc[1]); acc[1] = fmaf(xv.w, b2f(d1, 3), acc[1]);
-	acc[2] = fmaf(xv.x, b2f(d2, 0), acc[2]); acc[2] = fmaf(xv.y, b2f(d2, 1), acc[2]);
-	acc[2] = fmaf(xv.z, b2f(d2, 2), acc[2]); acc[2] = fmaf(xv.w, b2f(d2, 3), acc[2]);
-	acc[3] = fmaf(xv.x, b2f(d3, 0), acc[3]); acc[3] = fmaf(xv.y, b2f(d3, 1), acc[3]);
-	acc[3] = fmaf(xv.z, b2f(d3, 2), acc[3]); acc[3] = fmaf(xv.w, b2f(d3, 3), acc[3]);
-}
-
-// Second stage of the greedy argmax over n per-workgroup (maximum, index) pairs: every thread of the workgroup gets
-// the winner (ops.hpp:749-757: strict '>' from index 0, so the lowest index wins ties; no comparison is true for a
-// row of NaN and the index stays at the reference's initial -1).  s_bv / s_bi: NWAVE entries of LDS.
-__device__ __forceinline__ int argmax_pairs(const float *blk_val, const int *blk_idx, int n, float *s_bv, int *s_bi) {
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-	float bv = -INFINITY;
-	int bi = 0x7fffffff;
-	// all loads first (clamped indices, no branches), then the comparisons: one memory round trip instead of one per pass
-	for (int i0 = 0; i0 < n; i0 += 8 * NT) {
-		float ovs[8];
-		int ois[8];
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			const int i = i0 + u * NT + tid, ic = i < n ? i : n - 1;
-			ovs[u] = blk_val[ic];
-			ois[u] = blk_idx[ic];
-		}
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			const bool in = i0 + u * NT + tid < n;
-			if (in && (ovs[u] > bv || (ovs[u] == bv && ois[u] < bi))) { bv = ovs[u]; bi = ois[u]; }
-		}
-	}
-#define TG_STEP(O)                                                      \
-	{                                                                   \
-		const float ov = tg_red_partner<O>(bv);                         \
-		const int oi = tg_red_partner<O>(bi);                           \
-		if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }     \
-	}
-	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
-#undef TG_STEP
-	if (lane == 0) { s_bv[w] = bv; s_bi[w] = bi; }
-	__syncthreads();
-	bv = s_bv[0];
-	bi = s_bi[0];
-	for (int i = 1; i < NWAVE; i++)
-		if (s_bv[i] > bv || (s_bv[i] == bv && s_bi[i] < bi)) { bv = s_bv[i]; bi = s_bi[i]; }
-	return bi == 0x7fffffff ? -1 : bi;
-}
-
-// Per-token bookkeeping once the pick is known: it becomes the next step's input token, is appended to the id log, and
-// KVCache::update_single's counters (decode.hpp:68-69) advance once per token.  One thread.
-__device__ __forceinline__ void record_pick(int tok, int *ctr, int *tok_log, int advance) {
-	ctr[4] = tok;
-	const int st = ctr[3];
-	tok_log[st] = tok;
-	ctr[3] = st + 1;
-	if (advance) {
-		ctr[0] += 1;
-		ctr[1] += 1;
-		ctr[2] += 1;
-	}
-}
 
 // DEPTH: 16-byte weight loads in flight per lane
 template <int PRO, int EPI, int AUX, int DEPTH>
@@ -206,55 +91,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	// Every global load of a prologue that does not depend on another one is issued up front, next
 	// to the weight loads above, so that the prologue costs one memory round trip, not several.
 	if (PRO == TG_PRO_ATTN_MERGE) {
-		// merge of the flash-decoding partials of the attention launch that precedes this projection:
-		//   out_h = sum_b acc_{b,h} * exp(m_{b,h} - M_h) / sum_b l_{b,h} * exp(m_{b,h} - M_h)
+		// merge of the flash-decoding partials of the attention launch that precedes this projection
 		const int pos = g.host_pos >= 0 ? g.host_pos : g.pos[0];
 		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
 		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
-		// wave w merges head w; a lane owns 4 consecutive dims: 16 loads of 16 bytes instead of 64 of 4
-		f32x4 a[TG_ATTN_MERGE_MAX];
-		float m = -INFINITY, l = 0.0f;
-		if (tid < 4 * TG_ATTN_MERGE_MAX && (tid % TG_ATTN_MERGE_MAX) < nb) {
-			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
-			m = g.part_ml[((size_t)b * 4 + h) * 2];
-			l = g.part_ml[((size_t)b * 4 + h) * 2 + 1];
-		}
-#pragma unroll
-		for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) {
-			// unconditional load from a clamped index, select afterwards: a load under a branch is waited for
-			// at the end of that branch, which would turn these loads into as many round trips
-			const int bb = b < nb ? b : 0;
-			const f32x4 val = *reinterpret_cast<const f32x4 *>(g.part_acc + ((size_t)bb * 4 + w) * 256 + 4 * lane);
-			a[b] = (b < nb) ? val : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-		}
-		issue_weights();
-		if (tid < 4 * TG_ATTN_MERGE_MAX) {
-			const int h = tid / TG_ATTN_MERGE_MAX, b = tid % TG_ATTN_MERGE_MAX;
-			const bool ok = b < nb;
-			static_assert(TG_ATTN_MERGE_MAX == 16, "one row of 16 lanes per head");
-			const float M = tg_row16_max(m);
-			const float e = ok ? expf(m - M) : 0.0f;
-			// __fmul_rn: the product must be rounded before the reduction; contracted into the first add
-			// (fma(l, e, partner)) the two lanes of a pair would no longer hold the same sum
-			const float L = tg_row16_sum(__fmul_rn(l, e));
-			wgt[h][b] = e / L;
-		}
-		__syncthreads();
-		{
-			f32x4 o = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-			for (int b = 0; b < TG_ATTN_MERGE_MAX; b++) {
-				const float wb = wgt[w][b];
-#pragma unroll
-				for (int e = 0; e < 4; e++) o[e] = fmaf(a[b][e], wb, o[e]);
-			}
-			*reinterpret_cast<f32x4 *>(&xs[w * 256 + 4 * lane]) = o;
-		}
-		__syncthreads();
+		attn_merge_prologue(xs, wgt, g.part_acc, g.part_ml, nb, issue_weights);
 	} else if (PRO != TG_PRO_PLAIN) {
 		const int h = g.hidden;
-		const float eps = 1e-06f;
-		constexpr int PER = (TG_MAX_HIDDEN + NT - 1) / NT;  // elements of the residual stream per lane
 		float t[PER], wpre[PER];
 #pragma unroll
 		for (int i = 0; i < PER; i++) {
@@ -277,7 +120,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
 				const int dd = d < h ? d : h - 1;
-				const float val = g.wte_scales[dd] * (g.emb_scale * (float)row[dd]);
+				const float val = embed_value(g.wte_scales[dd], g.emb_scale, row[dd]);
 				t[i] = (d < h) ? val : 0.0f;
 			}
 			issue_weights();
@@ -307,17 +150,13 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			// The LM head, which is bound by its stream, requests it at once.
 			constexpr bool late = (AUX == TG_W_DEFAULT);
 			if (!late) issue_weights();
-			float ss = 0.0f;
-#pragma unroll
-			for (int i = 0; i < PER; i++) ss = fmaf(p[i], p[i], ss);
+			float ss = sumsq(p);
 			if (late) {
 				asm volatile("" : "+v"(ss) : : "memory");
 				issue_weights();
 			}
 			ss = block_sum(ss, sred);
-			const float irms = 1.0f / sqrtf(ss / (float)h + eps);
-#pragma unroll
-			for (int i = 0; i < PER; i++) t[i] = (p[i] * irms) * (wpo[i] + 1.0f) + r[i];
+			post_norm_add(t, p, rms_inv(ss, h), wpo, r);
 		}
 		if (g.xr_out != nullptr && blockIdx.x == 0) {
 #pragma unroll
@@ -327,16 +166,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 			}
 		}
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
-		float ss = 0.0f;
-#pragma unroll
-		for (int i = 0; i < PER; i++) ss = fmaf(t[i], t[i], ss);  // lanes past h hold 0
-		ss = block_sum(ss, sred);
-		const float irms = 1.0f / sqrtf(ss / (float)h + eps);
-#pragma unroll
-		for (int i = 0; i < PER; i++) {
-			const int d = tid + i * NT;
-			if (d < h) xs[d] = (t[i] * irms) * (wpre[i] + 1.0f);
-		}
+		const float ss = block_sum(sumsq(t), sred);
+		pre_norm_store(xs, t, rms_inv(ss, h), wpre, h);
 		__syncthreads();
 	}
 
@@ -384,33 +215,14 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	}
 
 	// ---------------- reduction over the lanes along K (fixed order) ----------------
-	// lanes l and l' hold partial sums of the same columns iff l % LC == l' % LC
-#define TG_STEP(O)                                                   \
-	if (LC <= O) {                                                   \
-		_Pragma("unroll") for (int j = 0; j < 4; j++) acc[j] += tg_red_partner<O>(acc[j]); \
-	}
-	TG_STEP(32) TG_STEP(16) TG_STEP(8) TG_STEP(4) TG_STEP(2) TG_STEP(1)
-#undef TG_STEP
-	if (lane < LC) *reinterpret_cast<float4 *>(&red[w][lane * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+	lanes_reduce(acc, LC, red);
 	__syncthreads();
 
 	// ---------------- epilogue of tile `cur` ----------------
 	if (EPI == TG_EPI_STORE) {
-		if (tid < C) {
-			const int col = cur * C + tid;
-			const float sum = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
-			g.y[col] = sum * sc_cur_a;
-		}
+		epi_store<false>(red, C, cur, sc_cur_a, g.y);
 	} else if (EPI == TG_EPI_GEGLU) {
-		// modules.hpp:211-215: gelu(gate) * up; the tile holds C/2 up columns, then the same C/2 gate columns
-		const int C2 = C >> 1;
-		if (tid < C2) {
-			const float su = (red[0][tid] + red[1][tid]) + (red[2][tid] + red[3][tid]);
-			const float sg = (red[0][tid + C2] + red[1][tid + C2]) + (red[2][tid + C2] + red[3][tid + C2]);
-			const float up = su * sc_cur_a;
-			const float gate = sg * sc_cur_b;
-			g.y[cur * C2 + tid] = gelu_lut(gate, lut_in_lds ? lut_s : g.lut, g.gmin, g.geps, g.lut_size) * up;
-		}
+		epi_geglu<false>(red, C, cur, sc_cur_a, sc_cur_b, g.y, lut_in_lds ? lut_s : g.lut, g.gmin, g.geps, g.lut_size);
 	} else {
 		// TG_EPI_LOGITS: logits + first stage of the greedy argmax
 		// (ops.hpp:749-757: strict '>' scan from index 0, so the lowest index wins ties)

@@ -160,6 +160,63 @@ size_t tg_minp_segments(int n);
 void tg_launch_minp(const float *logits, int n, float minp, float temp, const float *randf, int rand_idx, int rand_base, float *probs,
                     float *seg, float *bsum, float *bmax, int *ctr, int *tok_log, int mode, int *out_tok, hipStream_t s);
 
+// ---- one-kernel decode step (tg_decode_fused.hip) --------------------------------------------------------------
+// All layers of a decode step in ONE launch of resident workgroups: `ng` GEMV workgroups that own fixed column tiles of
+// every projection (tiles g and g + ng) and TG_FUSED_ATTN_WGS attention workgroups.  Where the launch path has a launch
+// boundary, the workgroups hand over through device memory: producers store write-through, arrive on counters, consumers
+// poll the counters and then read the data with ordinary loads from a buffer that is written once per launch (a line
+// that was never read before cannot be stale in an L1 or in another XCD's L2).  The LM head stays a launch of its own.
+#define TG_FUSED_ATTN_WGS TG_ATTN_MERGE_MAX
+struct TgFusedMat {
+	int K, C, lc_shift, ntiles;
+};
+struct TgFusedLayer {
+	const int8_t *Wqkv, *Wo, *Wug, *Wd;      // GEMV tile layout
+	const float *sqkv, *so, *sug, *sd;       // column scales, tile order
+	const float *apre, *apost, *mpre, *mpost, *rms_q, *rms_k;
+	float *kc, *vc;
+	int max_pos, is_sw;
+};
+struct TgFused {
+	const TgFusedLayer *layers;  // device array [L]
+	int L, hidden, ng;
+	TgFusedMat mqkv, mo, mug, md;
+	// first layer: embedding of the device-side token, or of the previous step's pending greedy pick (see TgGemv)
+	const int8_t *wte;
+	const float *wte_scales;
+	const int *tok;
+	const float *am_val;
+	const int *am_idx;
+	int am_n;
+	int *am_ctr, *am_log;
+	int vocab;
+	float emb_scale;
+	// attention: tables [n_pos][128] of the global / local layers, counters of this step, keys per attention workgroup
+	const float *cos_g, *sin_g, *cos_l, *sin_l;
+	int pos, bp_local, bp_global, chunk_local, chunk_global;
+	const float *lut;
+	float gmin, geps;
+	int lut_size;
+	float *xr;            // [2L+1][hidden] residual stream after every block (written by GEMV workgroup 0)
+	// exchange buffer: per layer qkv | partial outputs | partial (max, sum) | o | h | d, every region 256-byte aligned
+	float *xch;
+	size_t layer_stride;  // floats
+	int off_qkv, off_pacc, off_pml, off_o, off_h, off_d;
+	// hand-over state: 8 arrival counters of the GEMV workgroups (one 128-byte line per XCD), 8 copies of the attention
+	// counter, one error word; all_base = sum of the GEMV counters at launch, attn_base = value of each attention counter
+	unsigned *sync;
+	unsigned all_base, attn_base;
+	int max_spins;
+	unsigned long long *ts;  // optional (debug): [L][24] timestamps of GEMV workgroup 0 (0..15) and attention workgroup 0 (16..18)
+};
+#define TG_FUSED_SYNC_WORDS (17 * 32)
+// Largest number of 4 KiB steps of one tile the kernel keeps in registers, per projection; the launcher picks the
+// instantiation: 0 = (2, 1, 9, 7) the 1B shape, 1 = (1, 1, 3, 2) the 270m shape; -1: no instantiation fits
+int tg_fused_variant(const TgFused &f);
+// returns false when the kernel cannot be co-resident on this device (the caller then uses the launch path)
+bool tg_fused_supported(int n_cu);
+void tg_launch_decode_fused(const TgFused &f, int variant, hipStream_t s);
+
 // ---- prefill kernels (rows = prompt positions) -----------------------------------------------
 void tg_launch_embed_rows(float *x, const int *ids, int S, const int8_t *wte, const float *scales, int hidden, int vocab,
                           hipStream_t s);

@@ -18,6 +18,7 @@
 #include "tg_internal.h"
 
 extern hipStream_t tg_probe_stream();  // the library's stream (tg_api.hip)
+extern int tg_probe_n_cu();             // compute units of the device the library runs on
 
 namespace {
 
@@ -70,6 +71,230 @@ __global__ __launch_bounds__(PNT) void grid_barrier_kernel(unsigned *counter, fl
 		}
 	}
 	if (tid < 16) sink[blockIdx.x * 16 + tid] = acc;
+}
+
+// ---- sharded hand-over between the workgroups of one resident kernel ----------------------------------------------
+// What the single-counter barrier above measures is mostly serialisation: every workgroup adds to one address and
+// then every workgroup polls that same address.  handover_kernel asks what the hand-over costs when arrivals and
+// polls are spread over the machine the way it is built: 8 XCDs with an L2 each, a memory side they all share.
+// Barrier (BAR):
+//   0  one counter, everyone polls it (the figure above, with the data volume and the check of this kernel)
+//   1  an arrival counter per XCD (its own 128-byte line), the last arriver of an XCD adds to one 8-way counter, the
+//      last of those writes a release flag per XCD; a workgroup polls its XCD's flag line with device-scope loads
+//   2  the same tree, but a workgroup polls its XCD's flag with a returning read-modify-write (which the L2 executes;
+//      a device-scope load is sent past the L2) and the XCD's last arriver polls the 8-way counter and sets the flag
+//   3  no tree: an arrival counter per XCD, added to without waiting for the old value; every workgroup polls all 8
+//      counters (8 lanes, one load instruction per poll)
+//   4  no atomics: every workgroup stores the round number into its own word of a flag array (8 lines for 256
+//      workgroups); one wave per workgroup polls the whole array, 16 bytes per lane
+// Data (DATA): workgroup b publishes words_per_wg floats per round with device-scope (write-through) stores; after the
+// hand-over every workgroup reads ALL nwg * words_per_wg of them
+//   0  with device-scope loads (sent past the L2), from one of two alternating slots
+//   1  with ordinary loads, from a slot that is used for this round only (a ring as long as the launch): a line that
+//      has never been read cannot be stale in any cache, so nothing is invalidated; the 32 workgroups of an XCD
+//      share one fetch through their L2
+//   2  with ordinary loads from two alternating slots: the XCD's last arriver invalidates the L2 (device-scope
+//      acquire) before it releases its XCD, every workgroup invalidates its L1 (BAR 2 only)
+//   3  no barrier at all: every datum is an 8-byte (value, round) pair written and polled with device-scope atomics
+//   4  no barrier and no tag: a slot is used for one round only and starts out filled with a NaN pattern no result
+//      can have; a consumer polls the floats themselves (16-byte device-scope loads) until none of them is the pattern
+// The reads of a round are all issued before the first is used (unrolled, clamped indices), as a real consumer would.
+// and checks their sum against the closed form, so a stale or early read is counted, not just timed.  Which XCD a
+// workgroup runs on is read from the hardware register; the number of workgroups per XCD is counted by a
+// registration round (single counter) at kernel start.
+constexpr int BL = 32;  // words per 128-byte line
+constexpr int HO_MAX_TOTAL = 7168;            // floats published per round, upper bound (28 per thread)
+constexpr unsigned HO_SENTINEL = 0xffffffffu;  // a NaN no arithmetic produces
+typedef float ho_f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned ho_u32x4 __attribute__((ext_vector_type(4)));
+enum { HS_TOP = 0, HS_SINGLE = 1, HS_MEMBERS = 2, HS_REG = 3, HS_ARRIVE = 4, HS_FLAG = 12, HS_LINES = 20 };
+
+#define TG_AG_ADD(p, v) __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define TG_AG_LD(p) __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+#define TG_AG_ST(p, v) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+
+__device__ __forceinline__ unsigned probe_xcc_id() {
+	unsigned v;
+	asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(v));
+	return v & 7u;
+}
+// the current value of *p through a returning atomic OR of 0 (written out: the compiler turns an atomic that cannot
+// change memory into a load, which an L1 may serve)
+__device__ __forceinline__ unsigned probe_rmw_read(unsigned *p) {
+	unsigned v;
+	const unsigned zero = 0u;
+	asm volatile("global_atomic_or %0, %1, %2, off sc0\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p), "v"(zero) : "memory");
+	return v;
+}
+__device__ __forceinline__ float handover_value(int r, int i) { return (float)((r * 131 + i * 7) & 255); }
+
+// Bounded wait of one thread: false (and *flag set, `dead` latched: later waits return at once) after max_spins polls.
+template <class F>
+__device__ __forceinline__ bool probe_wait(F ready, int max_spins, bool &dead, int *flag) {
+	if (dead) return false;
+	int spins = 0;
+	while (!ready()) {
+		if (++spins >= max_spins) {
+			dead = true;
+			TG_AG_ST(flag, 1);
+			return false;
+		}
+		__builtin_amdgcn_s_sleep(1);
+	}
+	return true;
+}
+
+template <int BAR, int DATA>
+__global__ __launch_bounds__(PNT) void handover_kernel(unsigned *st, float *xchg, unsigned long long *xchg2, int rounds, int wpw, int max_spins,
+                                                       int *flags /* [0] timed out, [1] wrong sums */, int *xcd_of_wg) {
+	__shared__ unsigned s_x, s_members, s_nx;
+	__shared__ unsigned s_target[8];
+	const int nwg = (int)gridDim.x, tid = threadIdx.x, b = blockIdx.x, total = nwg * wpw;
+	bool dead = false;
+	if (tid == 0) {
+		const unsigned x = probe_xcc_id();
+		TG_AG_ADD(&st[HS_MEMBERS * BL + x], 1u);
+		__builtin_amdgcn_s_waitcnt(0);
+		TG_AG_ADD(&st[HS_REG * BL], 1u);
+		probe_wait([&] { return TG_AG_LD(&st[HS_REG * BL]) >= (unsigned)nwg; }, max_spins, dead, &flags[0]);
+		unsigned nx = 0;
+		for (int k = 0; k < 8; k++) {
+			const unsigned mk = TG_AG_LD(&st[HS_MEMBERS * BL + k]);
+			s_target[k] = mk;
+			nx += mk != 0u;
+		}
+		s_x = x;
+		s_members = s_target[x];
+		s_nx = nx;
+		xcd_of_wg[b] = (int)x;
+	}
+	__syncthreads();
+	const unsigned x = s_x, members = s_members, nx = s_nx;
+	const unsigned my_target = s_target[tid & 7];
+	int wrong = 0;
+	for (int r = 0; r < rounds; r++) {
+		const unsigned e = (unsigned)r + 1u;
+		float *slot = xchg + (size_t)((DATA == 1 || DATA == 4) ? r : (r & 1)) * total;
+		unsigned long long *slot2 = xchg2 + (size_t)(r & 1) * total;
+		for (int j = tid; j < wpw; j += PNT) {
+			const int i = b * wpw + j;
+			const float v = handover_value(r, i);
+			if (DATA == 3) __hip_atomic_store(&slot2[i], ((unsigned long long)e << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			else TG_AG_ST(&slot[i], v);
+		}
+		if (DATA != 3 && DATA != 4) {
+			__builtin_amdgcn_s_waitcnt(0);  // the write-through stores have been acknowledged
+			__syncthreads();
+			if (BAR == 3) {
+				if (tid == 0) __hip_atomic_fetch_add(&st[(HS_ARRIVE + x) * BL], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				if (tid < 64) {  // lanes 0..7 poll one counter each; the wave leaves when all 8 are there
+					probe_wait([&] { return __all(tid >= 8 || TG_AG_LD(&st[(HS_ARRIVE + (tid & 7)) * BL]) >= e * my_target); }, max_spins, dead, &flags[0]);
+				}
+			} else if (BAR == 4) {
+				if (tid == 0) TG_AG_ST(&st[HS_LINES * BL + b], e);
+				if (tid < 64) {
+					const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(&st[HS_LINES * BL], 0, nwg * 4, 0x00020000);
+					probe_wait(
+					    [&] {
+						    bool ok = true;
+						    for (int i0 = 0; i0 < nwg; i0 += 256) {  // words past the array read as 0: counted as arrived below
+							    const ho_u32x4 f = __builtin_bit_cast(ho_u32x4, __builtin_amdgcn_raw_buffer_load_b128(rf, (unsigned)(i0 + 4 * tid) * 4u, 0, 16));
+#pragma unroll
+							    for (int c = 0; c < 4; c++) ok = ok && (i0 + 4 * tid + c >= nwg || f[c] >= e);
+						    }
+						    return (bool)__all(ok);
+					    },
+					    max_spins, dead, &flags[0]);
+				}
+			} else if (tid == 0) {
+				if (BAR == 0) {
+					TG_AG_ADD(&st[HS_SINGLE * BL], 1u);
+					probe_wait([&] { return TG_AG_LD(&st[HS_SINGLE * BL]) >= e * (unsigned)nwg; }, max_spins, dead, &flags[0]);
+				} else if (BAR == 1) {
+					if (TG_AG_ADD(&st[(HS_ARRIVE + x) * BL], 1u) + 1u == e * members) {
+						if (TG_AG_ADD(&st[HS_TOP * BL], 1u) + 1u == e * nx)
+							for (int k = 0; k < 8; k++) TG_AG_ST(&st[(HS_FLAG + k) * BL], e);
+					}
+					probe_wait([&] { return TG_AG_LD(&st[(HS_FLAG + x) * BL]) >= e; }, max_spins, dead, &flags[0]);
+				} else {
+					if (TG_AG_ADD(&st[(HS_ARRIVE + x) * BL], 1u) + 1u == e * members) {
+						TG_AG_ADD(&st[HS_TOP * BL], 1u);
+						probe_wait([&] { return TG_AG_LD(&st[HS_TOP * BL]) >= e * nx; }, max_spins, dead, &flags[0]);
+						if (DATA == 2) asm volatile("buffer_inv sc1\n\ts_waitcnt vmcnt(0)" ::: "memory");
+						__hip_atomic_fetch_max(&st[(HS_FLAG + x) * BL], e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					} else {
+						probe_wait([&] { return probe_rmw_read(&st[(HS_FLAG + x) * BL]) >= e; }, max_spins, dead, &flags[0]);
+					}
+				}
+			}
+			__syncthreads();
+		}
+		// read everything every workgroup published this round
+		float sum = 0.0f, want = 0.0f;
+		constexpr int MAXV = HO_MAX_TOTAL / PNT / 4;  // 16-byte pieces per thread
+		const int nvec = total >> 2;
+		if (DATA == 3) {
+			bool ok = false;
+			probe_wait(
+			    [&] {
+				    ok = true;
+				    sum = 0.0f;
+				    for (int i = tid; i < total; i += PNT) {
+					    const unsigned long long p = __hip_atomic_load(&slot2[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					    ok = ok && (unsigned)(p >> 32) == e;
+					    sum += __uint_as_float((unsigned)p);
+				    }
+				    return ok;
+			    },
+			    max_spins, dead, &flags[0]);
+		} else if (DATA == 0 || DATA == 4) {
+			// 16-byte loads with the device-scope bit (aux bit 4 = sc1) through a buffer descriptor
+			const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(slot, 0, (int)(total * 4), 0x00020000);
+			auto pass = [&] {
+				ho_f32x4 v[MAXV];
+#pragma unroll
+				for (int k = 0; k < MAXV; k++) {
+					const int i = tid + k * PNT;
+					v[k] = __builtin_bit_cast(ho_f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (unsigned)(i < nvec ? i : 0) * 16u, 0, 16));
+				}
+				bool ok = true;
+				sum = 0.0f;
+#pragma unroll
+				for (int k = 0; k < MAXV; k++) {
+					if (tid + k * PNT < nvec) {
+#pragma unroll
+						for (int c = 0; c < 4; c++) {
+							ok = ok && __float_as_uint(v[k][c]) != HO_SENTINEL;
+							sum += v[k][c];
+						}
+					}
+				}
+				return ok;
+			};
+			if (DATA == 0) (void)pass();
+			else probe_wait(pass, max_spins, dead, &flags[0]);
+		} else {
+			if (DATA == 2) asm volatile("buffer_inv sc0" ::: "memory");  // this compute unit's L1 may hold the slot's lines of two rounds ago
+			else asm volatile("" ::: "memory");
+			ho_f32x4 v[MAXV];
+#pragma unroll
+			for (int k = 0; k < MAXV; k++) {
+				const int i = tid + k * PNT;
+				v[k] = reinterpret_cast<const ho_f32x4 *>(slot)[i < nvec ? i : 0];
+			}
+#pragma unroll
+			for (int k = 0; k < MAXV; k++)
+				if (tid + k * PNT < nvec) sum += (v[k][0] + v[k][1]) + (v[k][2] + v[k][3]);
+		}
+		if (DATA == 3) {
+			for (int i = tid; i < total; i += PNT) want += handover_value(r, i);
+		} else {  // the 16-byte pieces tid, tid + PNT, ...
+			for (int i = tid; i < nvec; i += PNT)
+				for (int c = 0; c < 4; c++) want += handover_value(r, 4 * i + c);
+		}
+		if (sum != want) wrong++;
+	}
+	if (wrong) atomicAdd(&flags[1], wrong);
 }
 
 // Back-to-back matrix instructions on register operands: 12 independent accumulators (3 x 4, as in the GEMM's inner
@@ -216,6 +441,66 @@ int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins,
 	if (rc != TG_OK) return rc;
 	*timed_out = h_flag;
 	*us_per_barrier = (us_many - us_few) / rounds;
+	return TG_OK;
+}
+
+int tg_debug_handover(int rounds, int workgroups, int barrier, int data, int words_per_wg, int max_spins, double *us_per_round,
+                      int *timed_out, int *wrong_sums, int *xcd_of_wg) {
+	if (rounds < 1 || rounds > 4096 || workgroups < 2 || workgroups > 2 * tg_probe_n_cu() || barrier < 0 || barrier > 4 || data < 0 || data > 4 || (size_t)workgroups * words_per_wg > HO_MAX_TOTAL || ((workgroups * words_per_wg) & 3) ||
+	    (data == 2 && barrier != 2) || words_per_wg < 1 || words_per_wg > 64 || max_spins < 1 || max_spins > (1 << 22) || !us_per_round || !timed_out ||
+	    !wrong_sums)
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument (rounds <= 4096, workgroups <= 2 per compute unit, workgroups * words_per_wg <= 7168 and a multiple of 4, max_spins <= 2^22, data 2 needs barrier 2)");
+	hipStream_t s = tg_probe_stream();
+	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
+	const size_t total = (size_t)workgroups * words_per_wg, nslots = (data == 1 || data == 4) ? (size_t)rounds + 8 : 2;
+	const size_t head = sizeof(unsigned) * (HS_LINES * BL + 512) + 128, map_bytes = (sizeof(int) * (size_t)workgroups + 127) / 128 * 128;
+	const size_t bytes = head + map_bytes + sizeof(unsigned long long) * 2 * total + sizeof(float) * nslots * total;
+	unsigned char *buf = nullptr;
+	TG_HIP(hipMalloc((void **)&buf, bytes));
+	unsigned *st = (unsigned *)buf;
+	int *flags = (int *)(st + HS_LINES * BL + 512);
+	int *map = (int *)(buf + head);
+	unsigned long long *xchg2 = (unsigned long long *)(buf + head + map_bytes);
+	float *xchg = (float *)(xchg2 + 2 * total);
+	int rc = TG_OK;
+	auto run = [&](int n) {
+#define TG_HO(B, D) \
+	if (barrier == B && data == D) hipLaunchKernelGGL((handover_kernel<B, D>), dim3((unsigned)workgroups), dim3(PNT), 0, s, st, xchg, xchg2, n, words_per_wg, max_spins, flags, map)
+		TG_HO(0, 0); TG_HO(0, 1); TG_HO(0, 3);
+		TG_HO(1, 0); TG_HO(1, 1); TG_HO(1, 3);
+		TG_HO(2, 0); TG_HO(2, 1); TG_HO(2, 2); TG_HO(2, 3);
+		TG_HO(3, 0); TG_HO(3, 1); TG_HO(3, 3);
+		TG_HO(4, 0); TG_HO(4, 1); TG_HO(0, 4);
+#undef TG_HO
+	};
+	double us_few = 0.0, us_many = 0.0;
+	int h_flags[2] = {0, 0};
+	// two launches that differ only in the number of rounds: their difference is the cost of the rounds alone
+	for (int pass = 0; pass < 3 && rc == TG_OK; pass++) {  // pass 0: warm-up
+		const int n = pass == 2 ? rounds + 8 : 8;
+		// flags are kept across the passes; the counters and the exchange buffers start from zero each time
+		if (hipMemsetAsync(buf, 0, pass == 0 ? bytes : sizeof(unsigned) * (HS_LINES * BL + 512), s) != hipSuccess ||
+		    hipMemsetAsync(xchg2, 0, sizeof(unsigned long long) * 2 * total, s) != hipSuccess ||
+		    (data == 4 && hipMemsetAsync(xchg, 0xff, sizeof(float) * nslots * total, s) != hipSuccess)) {
+			rc = tg_fail(TG_ERR_HIP, "hipMemsetAsync failed");
+			break;
+		}
+		Timer t;
+		rc = t.begin(s);
+		if (rc != TG_OK) break;
+		run(n);
+		rc = t.end(s, pass == 2 ? &us_many : &us_few);
+		if (rc == TG_OK && hipMemcpy(h_flags, flags, sizeof(h_flags), hipMemcpyDeviceToHost) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+		if (h_flags[0]) break;  // a wait timed out: the workgroups may not be co-resident; do not start the long launch
+	}
+	if (rc == TG_OK && xcd_of_wg && hipMemcpy(xcd_of_wg, map, sizeof(int) * (size_t)workgroups, hipMemcpyDeviceToHost) != hipSuccess)
+		rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+	(void)hipStreamSynchronize(s);
+	(void)hipFree(buf);
+	if (rc != TG_OK) return rc;
+	*timed_out = h_flags[0];
+	*wrong_sums = h_flags[1];
+	*us_per_round = h_flags[0] ? 0.0 : (us_many - us_few) / rounds;
 	return TG_OK;
 }
 
