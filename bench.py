@@ -135,8 +135,11 @@ def _cpu_baseline_run(orc, image_path, cfg_name, prompt, n_decode):
         "unit": "tok/s",
         "cores": 1,
         "kind": kind,
-        "sample": f"{n_decode} greedy decode steps after the same {len(prompt)}-token prompt "
-                  f"(prefill on the same core: {len(prompt) / (t1 - t0):.2f} tok/s)",
+        "prefill_tok_s": len(prompt) / (t1 - t0),
+        "prefill_tokens": len(prompt),
+        "decode_steps": n_decode,
+        "sample": f"{n_decode} greedy decode steps after the same {len(prompt)}-token prompt; prefill_tok_s = that prompt through "
+                  f"forward_prefill alone on the same core (the reference's own figure also counts table and cache set-up, gemma.cpp:53-58)",
     }
 
 
@@ -417,6 +420,48 @@ def main():
                                 "resident kernel, per round 64 B published per workgroup + device-wide barrier + 64 B read from a workgroup on "
                                 "another XCD; fences = ordinary stores/loads + device-scope fences, atomic_data = the data moves through "
                                 "device-scope atomic accesses; null = a bounded wait gave up")
+        # the hand-over between resident workgroups, sharded over the 8 XCDs (tg_debug_handover): per round every workgroup
+        # publishes words_per_wg floats, all hand over, every workgroup reads and checks all of them
+        to, wrong = C.c_int32(), C.c_int32()
+        handover = {}
+        for label, bar, data in (("one_counter", 0, 0), ("tree_per_xcd", 1, 1), ("eight_counters_summed", 3, 1), ("flag_array", 4, 1),
+                                 ("pairs_value_round_in_data", 0, 3), ("sentinel_in_data", 0, 4)):
+            for wgs, wpw in ((64, 6), (256, 6), (256, 27)):
+                tg.check(L.tg_debug_handover(400, wgs, bar, data, wpw, 1 << 16, C.byref(us), C.byref(to), C.byref(wrong), None))
+                handover[f"{label}_us_{wgs}wg_{wgs * wpw}floats"] = None if (to.value or wrong.value) else us.value
+        launch_floor["handover"] = handover
+        launch_floor["handover_note"] = ("one resident kernel; a round = write-through stores of the data, hand-over, every workgroup reads all of it and "
+                                         "checks the sum; one_counter: every workgroup adds to and polls one word; tree_per_xcd: counter per XCD -> "
+                                         "8-way counter -> release flag per XCD; eight_counters_summed: counter per XCD, every workgroup polls all 8 "
+                                         "(what the one-kernel decode step uses); flag_array: a word per workgroup; *_in_data: no barrier, the consumer "
+                                         "polls the data itself; null = a wait gave up or a sum was wrong")
+        # the one-kernel decode step (all layers in one launch of resident workgroups) against one launch per projection:
+        # same bits, tested; 256 steps each on the same session
+        fused = {}
+        for mode in (1, 0):
+            L.tg_set_fused_decode(mode, 0, 0)
+            sess.decode_enqueue(8)
+            tg.synchronize()
+            ev.record(e0, stream)
+            sess.decode_enqueue(256)
+            ev.record(e1, stream)
+            tg.synchronize()
+            sess.read_ids(1)  # reports a wait that gave up
+            fused["one_kernel_step_tok_s" if mode else "launch_per_projection_tok_s"] = 256 / (1e-3 * ev.elapsed_ms(e0, e1))
+        if L.tg_set_fused_decode(1, 0, 0) == 0:
+            ts = np.zeros((cfg.n_layers, 24), np.uint64)
+            if L.tg_debug_fused_timestamps(sess.h, ts.ctypes.data_as(C.c_void_p), cfg.n_layers) == 0:
+                t = ts.astype(np.int64)[1:-1]
+                names = ("norms_qkv", "qkv_tiles", "arrive_qkv", "wait_attention", "merge", "o_tiles", "arrive_o", "wait_o", "norms_upgate",
+                         "upgate_tiles", "arrive_h", "wait_h", "down_tiles", "arrive_d", "wait_d")
+                fused["layer_timeline_us"] = {n: float((t[:, i + 1] - t[:, i]).mean() / 100.0) for i, n in enumerate(names)}
+                fused["layer_us"] = float((t[:, 15] - t[:, 0]).mean() / 100.0)
+                fused["attention_workgroup_us"] = {"sees_qkv_after_gemv_wg0_arrived": float((t[:, 16] - t[:, 3]).mean() / 100.0),
+                                                   "body": float((t[:, 17] - t[:, 16]).mean() / 100.0),
+                                                   "arrive": float((t[:, 18] - t[:, 17]).mean() / 100.0),
+                                                   "gemv_wg0_sees_it_after": float((t[:, 4] - t[:, 18]).mean() / 100.0)}
+            L.tg_set_fused_decode(0, 0, 0)
+        launch_floor["one_kernel_step"] = fused
         if not args.graphs and L.tg_set_graphs(1) == 0:
             rates = {}
             for mode in (1, 0):
@@ -453,12 +498,18 @@ def main():
         simg = tgw.random_weight_image(scfg, args.seed + 1)
         smodel = tg.Transformer(scfg)
         smodel.read_weights_mem(simg)
+        spath = None
+        if args.cpu_steps > 0:  # the CPU baseline of this shape reads the same weight file
+            spath = f"/tmp/tg_bench_270m_{args.seed + 1}.bin"
+            simg.tofile(spath)
         del simg
         ss = smodel.session()
         s_bytes = MODELS["270m"][1]
 
+        sprompt = rng.integers(0, scfg.n_vocab, 64).astype(np.int32)
+
         def run(n_prompt_s, n_steps):
-            ids = rng.integers(0, scfg.n_vocab, n_prompt_s).astype(np.int32)
+            ids = sprompt if n_prompt_s == sprompt.size else rng.integers(0, scfg.n_vocab, n_prompt_s).astype(np.int32)
             ss.reset()
             ss.prefill(ids, want_logits=False)  # allocates the workspace for this length
             ss.reset()
@@ -481,6 +532,12 @@ def main():
         small = {"shape": "gemma-3-270m", "weight_bytes_per_token": s_bytes, "prompt64_decode256": short,
                  "prompt16384_decode256": long_ctx}
         del ss, smodel
+        if spath is not None:
+            try:
+                small["cpu_baseline"] = cpu_baseline(spath, "270m", sprompt, 256)
+                small["cpu_baseline"]["host_cpus"] = os.cpu_count()
+            finally:
+                os.remove(spath)
 
     tok_s = args.steps / wall
     out = {

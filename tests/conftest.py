@@ -108,7 +108,14 @@ def golden_file():
 # differ where the reference's own two best logits are closer than a few times that: observed gaps at differing picks
 # 2.4e-4 .. 1.0e-2 (about 2 % of steps on a random-token stream).  A differing pick is accepted only if the
 # reference's top-2 gap at that step is below NEAR_TIE and the pick is the reference's runner-up.
+#
+# Calibration (tests/test_oracle_calibration.py, CPU): the strict-IEEE checker, teacher-forced over the random-token
+# streams, differs from the reference binary on CHECKER_STREAM_MISMATCHES of 321 picks, always on the reference's
+# runner-up, at reference gaps up to 6.4e-3, with logits 3.3e-3 .. 4.2e-3 away.  NEAR_TIE is a little over twice that
+# largest gap (the largest gap at which the GPU's pick ever differed is 1.0e-2); the GPU stream test allows twice the
+# checker's count on the same stream, plus two.
 NEAR_TIE = 1.5e-2
+CHECKER_STREAM_MISMATCHES = {"stream270m": 4, "stream1B": 7}
 
 
 def check_picks(picks, ref, gaps, pairs, what, near_tie=NEAR_TIE, max_mismatches=None):

@@ -23,7 +23,7 @@ import numpy as np
 import pytest
 
 import golden_inputs as gi
-from conftest import NEAR_TIE, check_picks, normrel
+from conftest import CHECKER_STREAM_MISMATCHES, NEAR_TIE, check_picks, normrel
 
 pytestmark = pytest.mark.gpu
 
@@ -163,7 +163,10 @@ def test_teacher_forced_random_token_stream(tg, oracle, blocks, weight_images, t
             rels.append(normrel(lg[:4096], heads[gi.STREAM_LOGIT_STEPS.index(i)]))
     print(f"{name}: logits head norm-relative at steps {gi.STREAM_LOGIT_STEPS}: " + ", ".join(f"{r:.2e}" for r in rels), flush=True)
     # near-continuous table: fp32 summation order is all that is left and no pick may differ
-    check_picks(picks, ref, gaps, pairs, name, near_tie=1e-3 if fine else NEAR_TIE, max_mismatches=0 if fine else 14)
+    # coarse table: runner-up picks are small-number draws (CPU checker 4 and 7 of 321, this library 6 and 6, earlier
+    # kernels 7 + 7 and 6 + 3): at most twice the strict-IEEE checker's count on the same stream, plus two
+    check_picks(picks, ref, gaps, pairs, name, near_tie=1e-3 if fine else NEAR_TIE,
+                max_mismatches=0 if fine else 2 * CHECKER_STREAM_MISMATCHES[name] + 2)
     assert max(rels) < (2e-5 if fine else 9e-3)
     sess.free()
     model.free()

@@ -125,6 +125,8 @@ def lib():
     L.tg_qgemm_dev_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
     L.tg_debug_launch_chain.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
     L.tg_debug_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p]
+    L.tg_set_fused_decode.argtypes = [C.c_int, C.c_int, C.c_int]
+    L.tg_debug_fused_timestamps.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
     L.tg_debug_handover.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p, c_i32p, c_i32p]
     L.tg_debug_gemm_launches.argtypes = [C.POINTER(C.c_longlong)] * 3
     L.tg_debug_mfma_clock.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
