@@ -20,18 +20,44 @@ def pkg():
     return tg
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "tinygemma_hip.h")).read()
+def declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tg_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_every_declared_symbol_is_exported(pkg):
+    """Both headers: the contract (tinygemma_hip.h) and the knobs, probes and planning helpers (tinygemma_hip_debug.h)."""
     lib = C.CDLL(pkg.LIB_PATH)
-    names = declared_symbols()
-    assert len(names) >= 30
-    missing = [n for n in names if not hasattr(lib, n)]
+    contract, debug = declared_symbols("tinygemma_hip.h"), declared_symbols("tinygemma_hip_debug.h")
+    assert len(contract) >= 30 and len(debug) >= 20
+    assert not set(contract) & set(debug)
+    missing = [n for n in contract + debug if not hasattr(lib, n)]
     assert not missing, missing
+
+
+def test_the_contract_header_holds_no_knobs_or_probes():
+    """What a maintainer of the reference binds to: entry points that stand for a reference interface, the lifetime of
+    models and sessions, taps, and the entry point that allocates nothing.  Process-wide knobs (other than the taps
+    switch), timing probes and planning helpers live in the debug header."""
+    contract = declared_symbols("tinygemma_hip.h")
+    stray = [n for n in contract if n.startswith(("tg_debug_", "tg_plan_")) or (n.startswith("tg_set_") and n != "tg_set_taps")
+             or n in ("tg_decode_profile", "tg_reset_knobs")]
+    assert not stray, stray
+    debug = declared_symbols("tinygemma_hip_debug.h")
+    for n in ("tg_reset_knobs", "tg_set_fused_decode", "tg_debug_handover", "tg_debug_grid_barrier", "tg_decode_profile",
+              "tg_plan_attention_prefill"):
+        assert n in debug, n
+
+
+def test_every_exported_symbol_is_declared(pkg):
+    """Nothing is exported behind the headers' backs."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", pkg.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted({ln.split()[-1] for ln in out.splitlines() if " T tg_" in ln})
+    declared = set(declared_symbols("tinygemma_hip.h")) | set(declared_symbols("tinygemma_hip_debug.h"))
+    undeclared = [n for n in exported if n not in declared]
+    assert not undeclared, undeclared
 
 
 def test_named_configs(pkg):

@@ -1517,7 +1517,7 @@ int tg_set_attn_prefill_mode(int mode) {
 }
 
 int tg_set_attn_prefill_format(int f16) {
-	if (f16 < 0 || f16 > 3) return tg_fail(TG_ERR_BAD_ARG, "format: 0, 1, 2 or 3");
+	if (f16 < 0 || f16 > 2) return tg_fail(TG_ERR_BAD_ARG, "format: 0, 1 or 2");
 	g_attn_prefill_f16 = f16;
 	return TG_OK;
 }

@@ -448,8 +448,16 @@ __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int
 		stage(st0 + 3, std::integral_constant<int, 3>{});
 	}
 	wait_copies_in_flight<0>();  // the surplus copies too: the table below reuses the ring
-	// the matrix pipeline finishes its last instruction (8 passes) before an accumulator is read by an ordinary instruction
-	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+	// The matrix pipeline finishes its last instruction (8 passes) before an accumulator is read by an ordinary
+	// instruction.  The compiler does not know the asm statements above as matrix instructions and inserts no wait of
+	// its own, so the wait names every accumulator as an operand: nothing that reads one can be scheduled above it.
+	// (Bit-equality of this kernel with the compiler-scheduled gemm_i8_kernel: tests/test_gpu_kernels.py,
+	// test_gemm_kernels_agree_bit_for_bit; the compiled code is walked by tests/test_isa_hazards.py.)
+	asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15"
+	             : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[1][2]),
+	               "+a"(acc[1][3]), "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3])
+	             :
+	             : "memory");
 	float *lut_lds = reinterpret_cast<float *>(ring);
 	if (GEGLU && LUTLDS) {
 		__syncthreads();  // every wave is done with the ring

@@ -1,5 +1,5 @@
 // Internal declarations shared by the HIP translation units of libtinygemma_hip.so.
-// Nothing here is part of the C ABI (that is include/tinygemma_hip.h).
+// Nothing here is part of the C ABI (that is include/tinygemma_hip.h and, for knobs and probes, include/tinygemma_hip_debug.h).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../include/tinygemma_hip.h"
+#include "../../include/tinygemma_hip_debug.h"
 
 // ---------------------------------------------------------------------------------------------
 // Packed int8 weight layout in HBM
@@ -237,7 +238,7 @@ struct TgAttnPrefillPlan {
 	int nitems, nsplit;
 	float *part_o, *part_ml;
 };
-extern int g_attn_prefill_split;  // prefill attention: 0 = fp32 matrix path, 1 = split-precision matrix path (two fp16 or three bf16 planes), 2 = the same with 32-query workgroups at any length
+extern int g_attn_prefill_split;  // prefill attention: 0 = fp32 matrix path, 1 = split-precision matrix path (two fp16 or three bf16 planes), 2 = the same with 32-query workgroups at any length, 3 = the same with 16-query workgroups at any length
 int tg_attn_prefill_query_tile(int S, int n_cu);  // query positions per workgroup of the kernel a launch will take
 // window < 0: causal layer; else a local layer whose queries see `window` keys before them and themselves
 bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4> &items, std::vector<int4> &split, int &nslots);

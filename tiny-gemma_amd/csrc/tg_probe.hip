@@ -57,7 +57,7 @@ __global__ __launch_bounds__(PNT) void grid_barrier_kernel(unsigned *counter, fl
 			int spins = 0;
 			while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
 				if (++spins >= max_spins) {  // bounded wait: give up, flag it, go on
-					*timed_out = 1;
+					__hip_atomic_store(timed_out, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 					break;
 				}
 				__builtin_amdgcn_s_sleep(1);
@@ -405,8 +405,11 @@ int tg_debug_launch_chain(int n_launches, int workgroups, double *us_per_launch)
 }
 
 int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins, double *us_per_barrier, int *timed_out) {
-	if (rounds < 1 || workgroups < 2 || workgroups > 1024 || max_spins < 1 || !us_per_barrier || !timed_out)
-		return tg_fail(TG_ERR_BAD_ARG, "bad argument");
+	// the workgroups must all be resident at once (they are small: several fit a compute unit) and the kernel must end
+	// in bounded time whatever happens
+	if (rounds < 1 || rounds > 100000 || workgroups < 2 || workgroups > 2 * tg_probe_n_cu() || max_spins < 1 || max_spins > (1 << 22) || !us_per_barrier ||
+	    !timed_out)
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument (workgroups <= 2 per compute unit, max_spins <= 2^22)");
 	hipStream_t s = tg_probe_stream();
 	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
 	const size_t xf = (size_t)2 * workgroups * 16, words = 2 + xf + (size_t)workgroups * 16;
