@@ -22,7 +22,12 @@ namespace {
 // The leading arguments repeat the descriptor's first-used fields so that the dispatcher preloads them into
 // scalar registers (kernarg preload): the q/k-path loads go out without waiting for an s_load of the descriptor.
 __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, const float *rms_q, const float *rms_k, const float *cos_t,
-                                                          const float *sin_t, int host_pos, int host_bp, const TgAttnDecode a_in) {
+                                                          const float *sin_t, int host_pos, int host_bp, int nblocks, int chunk,
+                                                          const TgAttnDecode a_in) {
+	if ((int)blockIdx.x >= nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
+		tg_prefetch_dispatch(a_in.pf, a_in.pf2, nblocks);
+		return;
+	}
 	TgAttnDecode a = a_in;
 	a.qkv = qkv;
 	a.rms_q = rms_q;
@@ -31,10 +36,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, cons
 	a.sin_t = sin_t;
 	a.host_pos = host_pos;
 	a.host_bp = host_bp;
-	if ((int)blockIdx.x >= a.nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
-		tg_prefetch_dispatch(a.pf, a.pf2, a.nblocks);
-		return;
-	}
+	a.chunk = chunk;
 	attn_decode_body<false>(a, (int)blockIdx.x, [] {});
 }
 
@@ -127,7 +129,7 @@ void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t
 	if (a.pf.ptr == nullptr) a.pf.nblocks = 0;
 	if (a.pf2.ptr == nullptr) a.pf2.nblocks = 0;
 	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(max_blocks + a.pf.nblocks + a.pf2.nblocks)), dim3(ANT), 0, s, a.qkv, a.rms_q,
-	                   a.rms_k, a.cos_t, a.sin_t, a.host_pos, a.host_bp, a);
+	                   a.rms_k, a.cos_t, a.sin_t, a.host_pos, a.host_bp, a.nblocks, a.chunk, a);
 }
 
 // nblk: workgroups of the attention launch whose partials are folded

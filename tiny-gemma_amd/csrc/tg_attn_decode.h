@@ -54,9 +54,7 @@ __device__ __forceinline__ void norm_rope_head(const float *src, const float *w,
 	head_finish(in, mul, out);
 }
 
-// Keys of a chunk whose K rows / V elements are fetched before anything else in the kernel (the rest, for
-// chunks longer than this, is fetched inside the loops).
-constexpr int PRE = 32;
+typedef float af4 __attribute__((ext_vector_type(4)));
 
 // WT: the partials are stored write-through at device scope (for a consumer inside the same kernel on another XCD)
 template <bool WT>
@@ -65,19 +63,95 @@ __device__ __forceinline__ void attn_store(float *p, float v) {
 	else *p = v;
 }
 
-// One workgroup's chunk b of the keys: q/k norm + RoPE, cache write (chunk 0), scores, softmax partial, P.V.
+template <int CTRL>
+__device__ __forceinline__ float attn_dpp(float v) { return __uint_as_float(tg_dpp_u32<CTRL>(__float_as_uint(v))); }
+
+// 32 partial sums per lane, index 8 * head + key, are summed over the 64 lanes AND dealt out in the same pass: each
+// step adds the partner lane's half of the values this lane keeps and hands the other half over, so the value count
+// halves while the lane count doubles (70 instructions instead of 32 butterflies of 6).  Afterwards lane l holds the
+// complete sum of head l / 16, key (l % 16) / 2 (two neighbouring lanes hold each sum).  Partner lanes: the other
+// half-wave and the neighbouring row through the swap instructions; inside a row of 16 lanes l ^ 8 (rotation by 8),
+// l ^ 7 (mirror of the 8-lane half), l ^ 3 (quad reversed), l ^ 1.
+__device__ __forceinline__ float attn_transpose_reduce(float (&d)[32]) {
+	const int lane = (int)__lane_id();
+#pragma unroll
+	for (int v = 0; v < 16; v++) {  // lanes 32..63 keep heads 2, 3
+		const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(d[v]), __float_as_uint(d[v + 16]), false, false);
+		d[v] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+	}
+#pragma unroll
+	for (int v = 0; v < 8; v++) {   // odd rows keep heads 1, 3
+		const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(d[v]), __float_as_uint(d[v + 8]), false, false);
+		d[v] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+	}
+	const bool b3 = (lane & 8) != 0, b2 = (lane & 4) != 0, b1 = (lane & 2) != 0;
+#pragma unroll
+	for (int v = 0; v < 4; v++) {   // lanes with bit 3 keep keys 4..7
+		const float keep = b3 ? d[v + 4] : d[v], send = b3 ? d[v] : d[v + 4];
+		d[v] = keep + attn_dpp<0x128>(send);  // row_ror:8
+	}
+#pragma unroll
+	for (int v = 0; v < 2; v++) {   // lanes with bit 2 keep keys 2, 3 (6, 7)
+		const float keep = b2 ? d[v + 2] : d[v], send = b2 ? d[v] : d[v + 2];
+		d[v] = keep + attn_dpp<0x141>(send);  // row_half_mirror
+	}
+	const float keep = b1 ? d[1] : d[0], send = b1 ? d[0] : d[1];
+	const float s = keep + attn_dpp<0x1B>(send);  // quad_perm:[3,2,1,0]
+	return s + attn_dpp<0xB1>(s);                 // quad_perm:[1,0,3,2]
+}
+
+// RMSNorm + half-rotation RoPE of one 256-wide head vector spread over a wave, lane l owning dims 4l .. 4l+3
+// (ops.hpp:126-180, decode.hpp:136-211); the rotation partner of dim d, d +- 128, sits in lane l ^ 32.
+// cs4 / sn4: the table entries of dims (4l .. 4l+3) % 128.
+__device__ __forceinline__ af4 attn_head_finish(af4 x, af4 w, af4 cs4, af4 sn4, float mul) {
+	float ss = 0.0f;
+#pragma unroll
+	for (int e = 0; e < 4; e++) ss = fmaf(x[e], x[e], ss);
+	ss = wsum(ss);
+	const float irms = 1.0f / sqrtf(ss / (float)HD + 1e-06f);
+	const bool upper = (__lane_id() & 32) != 0;
+	af4 out;
+#pragma unroll
+	for (int e = 0; e < 4; e++) {
+		const float xn = (x[e] * irms) * (w[e] + 1.0f);
+		const float xp = tg_red_partner<32>(xn);
+		out[e] = fmaf(cs4[e], xn, (upper ? xp : -xp) * sn4[e]) * mul;
+	}
+	return out;
+}
+
+// Keys per wave and pass: a wave walks the blocks w, w + 4, ... of 8 keys of the workgroup's chunk.  The first block of
+// every wave (32 keys per workgroup) is requested before anything else in the kernel.
+constexpr int KB = 8;
+
+// One workgroup's chunk b of the keys: q/k norm + RoPE, cache write (chunk 0), and an exact softmax partial (maximum, sum,
+// unnormalised output) of the chunk for the four heads.  Every wave does the whole chain for its own keys and all four
+// heads without talking to the others - scores (the K rows are read once per workgroup), softmax over its keys, P.V -
+// and the four per-wave partials meet in LDS at the end: one workgroup barrier in all.
 // after_loads() is called once the body has issued its up-front loads.
 template <bool WT, class F>
 __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F after_loads) {
-	__shared__ __attribute__((aligned(16))) float qs[NH][HD];
-	__shared__ __attribute__((aligned(16))) float knew[HD];
-	__shared__ __attribute__((aligned(16))) float vnew[HD];
-	__shared__ __attribute__((aligned(16))) float sc[NH][MAXCHUNK];
-	__shared__ __attribute__((aligned(16))) float pv[ANT / 64][NH][HD];  // per-wave partial outputs of the first PRE keys
-	__shared__ float s_m[NH], s_l[NH];
+	__shared__ __attribute__((aligned(16))) float pacc[ANT / 64][NH][HD];  // per-wave unnormalised outputs
+	__shared__ float pm[ANT / 64][NH], pl[ANT / 64][NH];
 
-	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, sub = lane >> 4, sl = lane & 15;
+	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];          // position_ptr before this token (decode.hpp:154)
+
+	// Everything is requested up front.  The few values the q/k path needs go first (the previous launch's
+	// q|k|v vector, norm weights, RoPE row): a wait for them must not include the cache rows behind them.  Their
+	// addresses come from the launch arguments that the dispatcher preloads into scalar registers, so they go out
+	// before anything has to be fetched from the argument block.
+	const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
+	af4 xq[NH];
+#pragma unroll
+	for (int h = 0; h < NH; h++) xq[h] = *reinterpret_cast<const af4 *>(a.qkv + h * HD + 4 * lane);
+	const af4 xk = *reinterpret_cast<const af4 *>(a.qkv + NH * HD + 4 * lane);
+	const af4 vnew = *reinterpret_cast<const af4 *>(a.qkv + NH * HD + HD + 4 * lane);
+	const af4 wq = *reinterpret_cast<const af4 *>(a.rms_q + 4 * lane), wk = *reinterpret_cast<const af4 *>(a.rms_k + 4 * lane);
+	const af4 cs4 = *reinterpret_cast<const af4 *>(cs + 4 * (lane & 31)), sn4 = *reinterpret_cast<const af4 *>(sn + 4 * (lane & 31));
+	// The rest of the descriptor is fetched now, in one batch, behind the loads above (a scalar fetch per use, each under
+	// its own branch, was three dependent round trips in front of the first vector load).
+	asm volatile("" ::"s"(a.max_pos), "s"(a.kc), "s"(a.vc), "s"(a.part_acc), "s"(a.part_ml) : "memory");
 	const int bp = a.host_bp >= 0 ? a.host_bp : a.pos[a.bp_index];    // buffer_ptr before this token (decode.hpp:59)
 	const int cur = bp % a.max_pos;
 	const int valid = (pos + 1 < a.max_pos) ? pos + 1 : a.max_pos;  // decode.hpp:45-47 after update_single
@@ -85,180 +159,125 @@ __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F
 	if (b >= nb) return;
 	const int k0 = b * a.chunk;
 	const int n = (valid - k0 < a.chunk) ? valid - k0 : a.chunk;
-
-	// Everything is requested up front.  The few values the q/k path needs go first (the previous launch's
-	// q|k|v vector, norm weights, RoPE row): a wait for them must not include the cache rows behind them.
-	HeadIn qin, kin;
-	const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
-	head_load(qin, a.qkv + w * HD, a.rms_q, cs, sn, lane);
-	if (w == 0) head_load(kin, a.qkv + NH * HD, a.rms_k, cs, sn, lane);
-	const float vnew_r = a.qkv[NH * HD + HD + tid];
-	// Cache rows of the first PRE keys of this chunk: they depend on nothing computed here.
-	// K: 16 lanes per key row (pass p covers keys 16p + 4w + sub); V: wave w takes keys 8w .. 8w+7, a lane 4 dims.
-	float4 kpre[PRE / 16][4];
-	float4 vpre[PRE / 4];
-	// Rows are addressed as base + constant * row so that the 40 loads cost no per-load address arithmetic; rows
-	// past the chunk (and slot `cur`, which workgroup 0 rewrites below) are fetched and ignored: every row index is
-	// clamped into the cache, whose max_pos rows are all allocated.
-	{
-		const int lim = a.max_pos - 1 - k0;  // >= 0: last row of the cache, relative to the chunk
-		const float *kbase = a.kc + (size_t)k0 * HD + sl * 4;
-		const float *vbase = a.vc + (size_t)k0 * HD + 4 * lane;
+	const int nblk = (n + KB - 1) / KB;
+	// Cache rows of the wave's first block: they depend on nothing computed here.  Rows are addressed as base + constant
+	// * row; rows past the chunk (and slot `cur`, which workgroup 0 rewrites below) are fetched and ignored: every row
+	// index is clamped into the cache, whose max_pos rows are all allocated.
+	const int lim = a.max_pos - 1 - k0;  // >= 0: last row of the cache, relative to the chunk
+	const float *kbase = a.kc + (size_t)k0 * HD + 4 * lane, *vbase = a.vc + (size_t)k0 * HD + 4 * lane;
+	af4 kr[KB], vr[KB];
+	auto load_block = [&](int t) {
 #pragma unroll
-		for (int p = 0; p < PRE / 16; p++) {
-			int jj = 16 * p + w * 4 + sub;
-			jj = jj < lim ? jj : lim;
-			const float *kr = kbase + (size_t)jj * HD;
-#pragma unroll
-			for (int i = 0; i < 4; i++) kpre[p][i] = *reinterpret_cast<const float4 *>(kr + i * 64);
+		for (int jj = 0; jj < KB; jj++) {
+			int r = KB * t + jj;
+			r = r < lim ? r : lim;
+			kr[jj] = *reinterpret_cast<const af4 *>(kbase + (size_t)r * HD);
 		}
 #pragma unroll
-		for (int u = 0; u < PRE / 4; u++) {
-			const int jj = (PRE / 4) * w + u;
-			vpre[u] = *reinterpret_cast<const float4 *>(vbase + (size_t)(jj < lim ? jj : lim) * HD);
+		for (int jj = 0; jj < KB; jj++) {
+			int r = KB * t + jj;
+			r = r < lim ? r : lim;
+			vr[jj] = *reinterpret_cast<const af4 *>(vbase + (size_t)r * HD);
 		}
-	}
-
+	};
+	load_block(w);
 	after_loads();  // the caller's own loads go out behind this body's: a wait for a load covers every load issued before it
+	__builtin_amdgcn_sched_barrier(0);  // the requests stay in front of the arithmetic below
 
-	// q heads: one wave each; k: wave 0 again
-	{
-		float o[4];
-		head_finish(qin, 0.0625f, o);  // ops.hpp:257: q *= 1/sqrt(256)
+	// q heads and the new key: every wave normalises and rotates all five vectors for itself (five independent chains that
+	// overlap), which costs less than handing them round through LDS
+	af4 q[NH];
 #pragma unroll
-		for (int i = 0; i < 4; i++) qs[w][lane + 64 * i] = o[i];
-		if (w == 0) {
-			head_finish(kin, 1.0f, o);
-#pragma unroll
-			for (int i = 0; i < 4; i++) knew[lane + 64 * i] = o[i];
-		}
-		vnew[tid] = vnew_r;
-	}
-	__syncthreads();
-	if (b == 0) {  // KVCache::update_single, decode.hpp:49-70
-		a.kc[(size_t)cur * HD + tid] = knew[tid];
-		a.vc[(size_t)cur * HD + tid] = vnew[tid];
+	for (int h = 0; h < NH; h++) q[h] = attn_head_finish(xq[h], wq, cs4, sn4, 0.0625f);  // ops.hpp:257: q *= 1/sqrt(256)
+	const af4 knew = attn_head_finish(xk, wk, cs4, sn4, 1.0f);
+	if (b == 0 && w == 0) {  // KVCache::update_single, decode.hpp:49-70
+		*reinterpret_cast<af4 *>(a.kc + (size_t)cur * HD + 4 * lane) = knew;
+		*reinterpret_cast<af4 *>(a.vc + (size_t)cur * HD + 4 * lane) = vnew;
 	}
 
-	// scores: q_h . k_j for the 4 heads; the token being decoded (slot cur) comes from knew
-	{
-		float4 q[NH][4];
+	// the wave's blocks: scores, online softmax, P.V; m_run / l_run are those of the head of this lane's row
+	float m_run = -INFINITY, l_run = 0.0f;
+	af4 acc[NH];
 #pragma unroll
-		for (int h = 0; h < NH; h++)
+	for (int h = 0; h < NH; h++) acc[h] = af4{0.0f, 0.0f, 0.0f, 0.0f};
+	const int jl = (lane & 15) >> 1;  // the key (within a block) whose score this lane ends up with
+	for (int t = w; t < nblk; t += ANT / 64) {
+		if (t != w) load_block(t);
+		float d[32];
 #pragma unroll
-			for (int i = 0; i < 4; i++) q[h][i] = *reinterpret_cast<const float4 *>(&qs[h][i * 64 + sl * 4]);
-		auto pass = [&](int base, const float4 *kin) {
-			const int jj = base + w * 4 + sub;
-			const bool ok = jj < n;
-			const int j = k0 + (ok ? jj : 0);
-			float4 kv[4];
-#pragma unroll
-			for (int i = 0; i < 4; i++) kv[i] = (j == cur) ? *reinterpret_cast<const float4 *>(&knew[i * 64 + sl * 4]) : kin[i];
+		for (int jj = 0; jj < KB; jj++) {
+			const af4 kv = (k0 + KB * t + jj == cur) ? knew : kr[jj];  // the token being decoded comes from registers
 #pragma unroll
 			for (int h = 0; h < NH; h++) {
-				float d = 0.0f;
-#pragma unroll
-				for (int i = 0; i < 4; i++) {
-					d = fmaf(q[h][i].x, kv[i].x, d);
-					d = fmaf(q[h][i].y, kv[i].y, d);
-					d = fmaf(q[h][i].z, kv[i].z, d);
-					d = fmaf(q[h][i].w, kv[i].w, d);
-				}
-				d = sum16(d);
-				if (ok && sl == 0) sc[h][jj] = d;
+				float x = q[h][0] * kv[0];
+				x = fmaf(q[h][1], kv[1], x);
+				x = fmaf(q[h][2], kv[2], x);
+				x = fmaf(q[h][3], kv[3], x);
+				d[h * KB + jj] = x;
 			}
-		};
-#pragma unroll
-		for (int p = 0; p < PRE / 16; p++)
-			if (16 * p < n) pass(16 * p, kpre[p]);
-		for (int base = PRE; base < n; base += 16) {
-			const int jj = base + w * 4 + sub;
-			const int j = k0 + (jj < n ? jj : 0);
-			const float *kr = a.kc + (size_t)(j == cur ? k0 : j) * HD;
-			float4 kv[4];
-#pragma unroll
-			for (int i = 0; i < 4; i++) kv[i] = *reinterpret_cast<const float4 *>(kr + i * 64 + sl * 4);
-			pass(base, kv);
 		}
+		float s = attn_transpose_reduce(d);
+		const bool ok = KB * t + jl < n;
+		s = ok ? s : -INFINITY;
+		const float m_new = fmaxf(m_run, tg_row16_max(s));  // finite: the first key of a block is always valid
+		const float p = ok ? expf(s - m_new) : 0.0f;
+		const float scale = expf(m_run - m_new);            // 0 for the first block
+		l_run = fmaf(l_run, scale, 0.5f * tg_row16_sum(p));  // every sum sits in two lanes
+		m_run = m_new;
+#pragma unroll
+		for (int h = 0; h < NH; h++) {
+			const float sh = __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(scale), 16 * h));
+#pragma unroll
+			for (int e = 0; e < 4; e++) acc[h][e] *= sh;
+		}
+#pragma unroll
+		for (int jj = 0; jj < KB; jj++) {
+			const af4 vv = (k0 + KB * t + jj == cur) ? vnew : vr[jj];
+#pragma unroll
+			for (int h = 0; h < NH; h++) {
+				const float ph = __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(p), 16 * h + 2 * jj));
+#pragma unroll
+				for (int e = 0; e < 4; e++) acc[h][e] = fmaf(ph, vv[e], acc[h][e]);
+			}
+		}
+	}
+#pragma unroll
+	for (int h = 0; h < NH; h++) *reinterpret_cast<af4 *>(&pacc[w][h][4 * lane]) = acc[h];
+	if ((lane & 15) == 0) {
+		pm[w][lane >> 4] = m_run;
+		pl[w][lane >> 4] = l_run;
 	}
 	__syncthreads();
 
-	// softmax statistics of this chunk: wave h owns head h
+	// the four per-wave partials of head w -> the chunk's partial (max, sum, unnormalised output); merged by the consumer
 	{
-		float m = -INFINITY;
-		for (int j = lane; j < n; j += 64) m = fmaxf(m, sc[w][j]);
-		m = wmax(m);
+		float mw[ANT / 64], M = -INFINITY;
+#pragma unroll
+		for (int i = 0; i < ANT / 64; i++) {
+			mw[i] = pm[i][w];
+			M = fmaxf(M, mw[i]);
+		}
+		af4 o = af4{0.0f, 0.0f, 0.0f, 0.0f};
 		float l = 0.0f;
-		for (int j = lane; j < n; j += 64) {
-			const float p = expf(sc[w][j] - m);
-			sc[w][j] = p;
-			l += p;
+#pragma unroll
+		for (int i = 0; i < ANT / 64; i++) {
+			const float e = expf(mw[i] - M);  // a wave without keys: exp(-inf) = 0
+			const af4 pa = *reinterpret_cast<const af4 *>(&pacc[i][w][4 * lane]);
+#pragma unroll
+			for (int c = 0; c < 4; c++) o[c] = fmaf(pa[c], e, o[c]);
+			l = fmaf(pl[i][w], e, l);
 		}
-		l = wsum(l);
-		if (lane == 0) { s_m[w] = m; s_l[w] = l; }
-	}
-	__syncthreads();
-
-	// P.V of the first PRE keys: wave w owns keys 8w..8w+7, lane = 4 consecutive dims; summed over the waves via LDS
-	{
-		float4 part[NH];
+		float *dst = a.part_acc + ((size_t)b * NH + w) * HD + 4 * lane;
+		if (WT) {
 #pragma unroll
-		for (int h = 0; h < NH; h++) part[h] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-		const int ub = (PRE / 4) * w;
-		if (ub < n) {  // entries of sc past n are read with the group but not used
-			float4 p[NH][2];
-#pragma unroll
-			for (int h = 0; h < NH; h++) {
-				p[h][0] = *reinterpret_cast<const float4 *>(&sc[h][ub]);
-				p[h][1] = *reinterpret_cast<const float4 *>(&sc[h][ub + 4]);
-			}
-			const float4 vn = *reinterpret_cast<const float4 *>(&vnew[4 * lane]);
-#pragma unroll
-			for (int u = 0; u < PRE / 4; u++) {
-				if (ub + u < n) {
-					const float4 vv = (k0 + ub + u == cur) ? vn : vpre[u];
-#pragma unroll
-					for (int h = 0; h < NH; h++) {
-						const float ph = reinterpret_cast<const float *>(&p[h][u >> 2])[u & 3];
-						part[h].x = fmaf(ph, vv.x, part[h].x);
-						part[h].y = fmaf(ph, vv.y, part[h].y);
-						part[h].z = fmaf(ph, vv.z, part[h].z);
-						part[h].w = fmaf(ph, vv.w, part[h].w);
-					}
-				}
-			}
+			for (int c = 0; c < 4; c++) attn_store<true>(dst + c, o[c]);
+		} else {
+			*reinterpret_cast<af4 *>(dst) = o;
 		}
-#pragma unroll
-		for (int h = 0; h < NH; h++) *reinterpret_cast<float4 *>(&pv[w][h][4 * lane]) = part[h];
-	}
-	__syncthreads();
-	// from here on: thread = output dim, 4 heads
-	float acc[NH];
-#pragma unroll
-	for (int h = 0; h < NH; h++) acc[h] = (pv[0][h][tid] + pv[1][h][tid]) + (pv[2][h][tid] + pv[3][h][tid]);
-	for (int j0 = PRE; j0 < n; j0 += 8) {
-		float vv[8];
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			const int jj = j0 + u;
-			const int j = k0 + (jj < n ? jj : 0);
-			vv[u] = (j == cur) ? vnew[tid] : a.vc[(size_t)j * HD + tid];
+		if (lane == 0) {
+			attn_store<WT>(&a.part_ml[((size_t)b * NH + w) * 2 + 0], M);
+			attn_store<WT>(&a.part_ml[((size_t)b * NH + w) * 2 + 1], l);
 		}
-#pragma unroll
-		for (int u = 0; u < 8; u++) {
-			if (j0 + u < n) {
-#pragma unroll
-				for (int h = 0; h < NH; h++) acc[h] = fmaf(sc[h][j0 + u], vv[u], acc[h]);
-			}
-		}
-	}
-
-	// partial (max, sum, unnormalised output) of this chunk; merged by the consumer
-#pragma unroll
-	for (int h = 0; h < NH; h++) attn_store<WT>(&a.part_acc[((size_t)b * NH + h) * HD + tid], acc[h]);
-	if (tid < NH) {
-		attn_store<WT>(&a.part_ml[((size_t)b * NH + tid) * 2 + 0], s_m[tid]);
-		attn_store<WT>(&a.part_ml[((size_t)b * NH + tid) * 2 + 1], s_l[tid]);
 	}
 }
 

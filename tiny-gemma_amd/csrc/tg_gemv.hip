@@ -27,9 +27,15 @@ using namespace tgp;
 
 namespace {
 
+// Where the descriptor sits in the argument block of every GEMV kernel: behind the leading arguments of TG_GEMV_ARGS
+// (4 pointers, the weight pointer, 4 ints = 56 bytes, which is a multiple of the descriptor's alignment).
+constexpr int TG_GEMV_DESC_OFFSET = 4 * 8 + 8 + 4 * 4;
+static_assert(TG_GEMV_DESC_OFFSET % alignof(TgGemv) == 0, "the descriptor follows the leading arguments without padding");
+
 // DEPTH: 16-byte weight loads in flight per lane
 template <int PRO, int EPI, int AUX, int DEPTH>
-__device__ __forceinline__ void gemv_body(const TgGemv &g) {
+__device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
+	TgGemv g = g_in;  // the fields fetch_rest() names are not known to the code before it (see there)
 	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
 	__shared__ __attribute__((aligned(16))) float lut_s[(EPI == TG_EPI_GEGLU) ? LUT_LDS : 4];  // GeLU table of the GeGLU epilogue
 	__shared__ __attribute__((aligned(16))) float red2[2][NWAVE][TG_CT];  // double buffered across the tile loop
@@ -38,10 +44,6 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	__shared__ float s_bv[2][NWAVE];
 	__shared__ int s_bi[2][NWAVE];
 
-	if ((int)blockIdx.x >= g.nmain) {  // extra workgroups: prefetch the next launch's weights and leave
-		tg_prefetch_dispatch(g.pf, g.pf2, g.nmain);
-		return;
-	}
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	int tile = blockIdx.x;
 	const int C = g.C, LC = C >> 2, lcs = g.lc_shift;  // LC = 1 << lcs lanes across the tile's columns
@@ -74,16 +76,40 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		if (EPI == TG_EPI_GEGLU) sc_b = g.scales[t * C + (C >> 1) + c];
 	};
 	f32x4 lutv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-	const bool lut_in_lds = (EPI == TG_EPI_GEGLU) && g.lut_size <= LUT_LDS && (g.lut_size & 3) == 0;
+	auto lut_in_lds_f = [&]() { return (EPI == TG_EPI_GEGLU) && g.lut_size <= LUT_LDS && (g.lut_size & 3) == 0; };
+	// Everything the first vector loads need (pointers, K, C, the number of computing workgroups) arrives in scalar
+	// registers with the launch (leading arguments, preloaded by the dispatcher).  The rest of the descriptor is fetched
+	// from the argument block in ONE batch, by fetch_rest(), which every prologue calls right behind its first vector
+	// loads: fetched field by field at first use, each under its own branch, it was two dependent scalar round trips
+	// (0.3 us each) in front of the first vector load of every launch.
+	auto fetch_rest = [&]() {
+		// The fields are read through the address of the argument block, which is made opaque here: the compiler can
+		// neither start these fetches earlier (hoisted to the top of the kernel they end up with a wait in front of the
+		// vector loads as soon as one of their registers is reused) nor use a field before this point.
+		typedef const TgGemv __attribute__((address_space(4))) *KernargDesc;
+		KernargDesc gp = (KernargDesc)((const char __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr() + TG_GEMV_DESC_OFFSET);
+		asm volatile("" : "+s"(gp) : : "memory");
+		g.scales = gp->scales;
+		g.y = gp->y;
+		g.xr_out = gp->xr_out;
+		g.lut = gp->lut;
+		g.lut_size = gp->lut_size;
+		g.gmin = gp->gmin;
+		g.geps = gp->geps;
+		g.ntiles = gp->ntiles;
+		g.blk_val = gp->blk_val;
+		g.blk_idx = gp->blk_idx;
+	};
 	auto issue_weights = [&]() {
-		load_scales(tile);
-		if (lut_in_lds) lutv = *reinterpret_cast<const f32x4 *>(g.lut + (4 * tid < g.lut_size ? 4 * tid : 0));
 #pragma unroll
 		for (int u = 0; u < DEPTH; u++) {
 			xq[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 			v[u] = ldw<AUX>(rw, voff, min((uint32_t)u * STEP_BYTES, slab));  // past the end of the slab: reads as 0
 			if (PRO == TG_PRO_PLAIN) xq[u] = ldx(rx, xoff, min((uint32_t)u * xstep, xbytes));
 		}
+		if (PRO == TG_PRO_PLAIN) fetch_rest();
+		load_scales(tile);
+		if (lut_in_lds_f()) lutv = *reinterpret_cast<const f32x4 *>(g.lut + (4 * tid < g.lut_size ? 4 * tid : 0));
 	};
 	if (PRO == TG_PRO_PLAIN) issue_weights();
 
@@ -92,10 +118,16 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 	// to the weight loads above, so that the prologue costs one memory round trip, not several.
 	if (PRO == TG_PRO_ATTN_MERGE) {
 		// merge of the flash-decoding partials of the attention launch that precedes this projection
-		const int pos = g.host_pos >= 0 ? g.host_pos : g.pos[0];
-		const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
-		const int nb = (valid + g.attn_chunk - 1) / g.attn_chunk;  // <= TG_ATTN_MERGE_MAX, checked on the host
-		attn_merge_prologue(xs, wgt, g.part_acc, g.part_ml, nb, issue_weights);
+		int nb = g.merge_nb;  // <= TG_ATTN_MERGE_MAX, checked on the host
+		if (nb < 0) {         // a captured step is replayed at other positions: the count follows the device-side counter
+			const int pos = g.pos[0];
+			const int valid = (pos + 1 < g.attn_max_pos) ? pos + 1 : g.attn_max_pos;
+			nb = (valid + g.attn_chunk - 1) / g.attn_chunk;
+		}
+		attn_merge_prologue(xs, wgt, g.part_acc, g.part_ml, nb, [&] {
+			fetch_rest();
+			issue_weights();
+		});
 	} else if (PRO != TG_PRO_PLAIN) {
 		const int h = g.hidden;
 		float t[PER], wpre[PER];
@@ -123,6 +155,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				const float val = embed_value(g.wte_scales[dd], g.emb_scale, row[dd]);
 				t[i] = (d < h) ? val : 0.0f;
 			}
+			fetch_rest();
 			issue_weights();
 		} else if (PRO == TG_PRO_NORM) {
 #pragma unroll
@@ -131,6 +164,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				const float val = g.x[d < h ? d : h - 1];
 				t[i] = (d < h) ? val : 0.0f;
 			}
+			fetch_rest();
 			issue_weights();
 		} else {
 			// modules.hpp:166-168 / 218-219: x = rmsnorm(block_out, post) + residual
@@ -145,6 +179,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 				r[i] = ok ? rv : 0.0f;
 				wpo[i] = ok ? wv : 0.0f;
 			}
+			fetch_rest();
 			// The weight stream of a per-layer projection starts once the prologue's inputs are here (the empty asm
 			// keeps the scheduler from hoisting it): requested together with them it made a decode step 0.7 % slower.
 			// The LM head, which is bound by its stream, requests it at once.
@@ -171,6 +206,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 		__syncthreads();
 	}
 
+	const bool lut_in_lds = lut_in_lds_f();
 	if (lut_in_lds && 4 * tid < g.lut_size) *reinterpret_cast<f32x4 *>(&lut_s[4 * tid]) = lutv;  // visible after the barrier that precedes the epilogue
 	// A workgroup walks tiles blockIdx.x, blockIdx.x + nmain, ...: the prologue above is paid once.
 	const int xlast = g.K - 4;
@@ -263,11 +299,14 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g) {
 // s_load of the argument block (0.35 us on the critical path of every launch).
 template <int PRO>
 __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *a0, const void *a1, const void *a2, const void *a3,
-                                                const int8_t *W, int hidden, int K) {
+                                                const int8_t *W, int hidden, int K, int nmain, int aux) {
 	TgGemv g = g_in;
 	g.W = W;
 	g.hidden = hidden;
 	g.K = K;
+	g.nmain = nmain;
+	g.C = aux;  // tile width: what the addresses of the weight stream need first
+	g.lc_shift = 29 - __builtin_clz((unsigned)aux);  // log2(C / 4)
 	if (PRO == TG_PRO_RESNORM || PRO == TG_PRO_NORM) {
 		g.pend = (const float *)a0;
 		g.x = (const float *)a1;
@@ -276,6 +315,7 @@ __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *
 	} else if (PRO == TG_PRO_ATTN_MERGE) {
 		g.part_acc = (const float *)a0;
 		g.part_ml = (const float *)a1;
+		g.merge_nb = hidden;  // partials to merge, or -1: from the device-side position
 	} else if (PRO == TG_PRO_EMBED) {
 		g.wte = (const int8_t *)a0;
 		g.wte_scales = (const float *)a1;
@@ -288,15 +328,22 @@ __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *
 }
 // The per-layer roles are templates over DEPTH (the launcher picks it from the number of steps); the LM head has
 // one depth.
-#define TG_GEMV_ARGS const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, int hidden, int K, const TgGemv g
+#define TG_GEMV_ARGS \
+	const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, int hidden, int K, int nmain, int aux, const TgGemv g
+#define TG_GEMV_BODY(PRO, EPI, AUX, DEPTH)                                                            \
+	if ((int)blockIdx.x >= nmain) { /* extra workgroups: prefetch the next launch's weights and leave */ \
+		tg_prefetch_dispatch(g.pf, g.pf2, nmain);                                                     \
+		return;                                                                                       \
+	}                                                                                                 \
+	gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K, nmain, aux));
 #define TG_GEMV_KERNEL_T(NAME, PRO, EPI, AUX)                                                         \
 	template <int DEPTH>                                                                              \
 	__global__ __launch_bounds__(NT) void NAME(TG_GEMV_ARGS) {                                        \
-		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));         \
+		TG_GEMV_BODY(PRO, EPI, AUX, DEPTH)                                                            \
 	}
 #define TG_GEMV_KERNEL(NAME, PRO, EPI, AUX, DEPTH)                                                    \
 	__global__ __launch_bounds__(NT) void NAME(TG_GEMV_ARGS) {                                        \
-		gemv_body<PRO, EPI, AUX, DEPTH>(with_hot_args<PRO>(g, a0, a1, a2, a3, W, hidden, K));         \
+		TG_GEMV_BODY(PRO, EPI, AUX, DEPTH)                                                            \
 	}
 TG_GEMV_KERNEL_T(tg_gemv_qkv_embed, TG_PRO_EMBED, TG_EPI_STORE, TG_W_DEFAULT)        // layer 0: embedding + pre-norm + Q|K|V
 TG_GEMV_KERNEL_T(tg_gemv_qkv, TG_PRO_RESNORM, TG_EPI_STORE, TG_W_DEFAULT)            // post-norm + residual + pre-norm + Q|K|V
@@ -351,7 +398,15 @@ void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
 	const void *a0 = g.pend, *a1 = g.x, *a2 = g.w_post, *a3 = g.w_pre;
 	if (role == TG_ROLE_OPROJ) { a0 = g.part_acc; a1 = g.part_ml; a2 = a3 = nullptr; }
 	if (role == TG_ROLE_QKV_EMBED) { a0 = g.wte; a1 = g.wte_scales; a2 = g.tok; a3 = g.w_pre; }
-#define TG_LAUNCH(KERNEL) hipLaunchKernelGGL(KERNEL, grid, block, 0, s, a0, a1, a2, a3, g.W, g.hidden, g.K, g)
+	int hot_hidden = g.hidden;
+	if (role == TG_ROLE_OPROJ) {  // the number of attention partials to merge rides in the slot of `hidden`
+		hot_hidden = -1;
+		if (g.host_pos >= 0) {
+			const int valid = (g.host_pos + 1 < g.attn_max_pos) ? g.host_pos + 1 : g.attn_max_pos;
+			hot_hidden = (valid + g.attn_chunk - 1) / g.attn_chunk;
+		}
+	}
+#define TG_LAUNCH(KERNEL) hipLaunchKernelGGL(KERNEL, grid, block, 0, s, a0, a1, a2, a3, g.W, hot_hidden, g.K, g.nmain, g.C, g)
 #define TG_LAUNCH_D(KERNEL)                          \
 	switch (depth) {                                 \
 		case 2: TG_LAUNCH(KERNEL<2>); break;         \

@@ -118,6 +118,7 @@ struct TgGemv {
 	int host_pos;          // ATTN_MERGE: the same position as a launch argument, or -1 to read the device counter
 	int attn_max_pos;      // ATTN_MERGE: cache slots of this layer
 	int attn_chunk;        // ATTN_MERGE: keys per attention workgroup
+	int merge_nb;          // ATTN_MERGE, set by the kernel from its leading arguments: partials to merge, or -1 (derive from pos)
 	const float *part_acc; // ATTN_MERGE: [nb][4][256]
 	const float *part_ml;  // ATTN_MERGE: [nb][4][2]
 	// epilogue (the TG_EPI_* mode is fixed by the kernel role)
