@@ -127,12 +127,13 @@ constexpr int KB = 8;
 // One workgroup's chunk b of the keys: q/k norm + RoPE, cache write (chunk 0), and an exact softmax partial (maximum, sum,
 // unnormalised output) of the chunk for the four heads.  Every wave does the whole chain for its own keys and all four
 // heads without talking to the others - scores (the K rows are read once per workgroup), softmax over its keys, P.V -
-// and the four per-wave partials meet in LDS at the end: one workgroup barrier in all.
+// and the four per-wave partials meet in LDS at the end: two workgroup barriers in all (the q heads, the partials).
 // after_loads() is called once the body has issued its up-front loads.
 template <bool WT, class F>
 __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F after_loads) {
 	__shared__ __attribute__((aligned(16))) float pacc[ANT / 64][NH][HD];  // per-wave unnormalised outputs
 	__shared__ float pm[ANT / 64][NH], pl[ANT / 64][NH];
+	__shared__ __attribute__((aligned(16))) float qs[NH][HD];  // normalised, rotated, scaled q heads
 
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 	const int pos = a.host_pos >= 0 ? a.host_pos : a.pos[0];          // position_ptr before this token (decode.hpp:154)
@@ -142,9 +143,7 @@ __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F
 	// addresses come from the launch arguments that the dispatcher preloads into scalar registers, so they go out
 	// before anything has to be fetched from the argument block.
 	const float *cs = a.cos_t + (size_t)pos * (HD / 2), *sn = a.sin_t + (size_t)pos * (HD / 2);
-	af4 xq[NH];
-#pragma unroll
-	for (int h = 0; h < NH; h++) xq[h] = *reinterpret_cast<const af4 *>(a.qkv + h * HD + 4 * lane);
+	const af4 xw = *reinterpret_cast<const af4 *>(a.qkv + w * HD + 4 * lane);  // q head w
 	const af4 xk = *reinterpret_cast<const af4 *>(a.qkv + NH * HD + 4 * lane);
 	const af4 vnew = *reinterpret_cast<const af4 *>(a.qkv + NH * HD + HD + 4 * lane);
 	const af4 wq = *reinterpret_cast<const af4 *>(a.rms_q + 4 * lane), wk = *reinterpret_cast<const af4 *>(a.rms_k + 4 * lane);
@@ -184,12 +183,15 @@ __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F
 	after_loads();  // the caller's own loads go out behind this body's: a wait for a load covers every load issued before it
 	__builtin_amdgcn_sched_barrier(0);  // the requests stay in front of the arithmetic below
 
-	// q heads and the new key: every wave normalises and rotates all five vectors for itself (five independent chains that
-	// overlap), which costs less than handing them round through LDS
+	// q heads and the new key.  Wave w normalises and rotates q head w; the new key, which every wave needs, is done by
+	// every wave for itself (two independent chains that overlap); the q heads are handed round through LDS.  (Every
+	// wave doing all five vectors saved the barrier but took 0.86 us: the chains are 100 instructions each.)
+	*reinterpret_cast<af4 *>(&qs[w][4 * lane]) = attn_head_finish(xw, wq, cs4, sn4, 0.0625f);  // ops.hpp:257: q *= 1/sqrt(256)
+	const af4 knew = attn_head_finish(xk, wk, cs4, sn4, 1.0f);
+	__syncthreads();
 	af4 q[NH];
 #pragma unroll
-	for (int h = 0; h < NH; h++) q[h] = attn_head_finish(xq[h], wq, cs4, sn4, 0.0625f);  // ops.hpp:257: q *= 1/sqrt(256)
-	const af4 knew = attn_head_finish(xk, wk, cs4, sn4, 1.0f);
+	for (int h = 0; h < NH; h++) q[h] = *reinterpret_cast<const af4 *>(&qs[h][4 * lane]);
 	if (b == 0 && w == 0) {  // KVCache::update_single, decode.hpp:49-70
 		*reinterpret_cast<af4 *>(a.kc + (size_t)cur * HD + 4 * lane) = knew;
 		*reinterpret_cast<af4 *>(a.vc + (size_t)cur * HD + 4 * lane) = vnew;
