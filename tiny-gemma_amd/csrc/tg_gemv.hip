@@ -39,7 +39,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 	__shared__ __attribute__((aligned(16))) float xs[TG_MAX_HIDDEN];  // input vector (all prologues but PLAIN)
 	__shared__ __attribute__((aligned(16))) float lut_s[(EPI == TG_EPI_GEGLU) ? LUT_LDS : 4];  // GeLU table of the GeGLU epilogue
 	__shared__ __attribute__((aligned(16))) float red2[2][NWAVE][TG_CT];  // double buffered across the tile loop
-	__shared__ float sred[NWAVE];
+	__shared__ float sred[NWAVE], sred2[NWAVE];  // one per norm of a prologue: neither needs a barrier in front of it
 	__shared__ float wgt[4][TG_ATTN_MERGE_MAX];
 	__shared__ float s_bv[2][NWAVE];
 	__shared__ int s_bi[2][NWAVE];
@@ -190,7 +190,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 				asm volatile("" : "+v"(ss) : : "memory");
 				issue_weights();
 			}
-			ss = block_sum(ss, sred);
+			ss = block_sum_fresh(ss, sred);
 			post_norm_add(t, p, rms_inv(ss, h), wpo, r);
 		}
 		if (g.xr_out != nullptr && blockIdx.x == 0) {
@@ -201,7 +201,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 			}
 		}
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
-		const float ss = block_sum(sumsq(t), sred);
+		const float ss = block_sum_fresh(sumsq(t), sred2);
 		pre_norm_store(xs, t, rms_inv(ss, h), wpre, h);
 		__syncthreads();
 	}

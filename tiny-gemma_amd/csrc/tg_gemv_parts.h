@@ -46,6 +46,16 @@ __device__ __forceinline__ float block_sum(float v, float *sred) {
 	return (sred[0] + sred[1]) + (sred[2] + sred[3]);
 }
 
+// The same sum for an `sred` that no thread of the workgroup can still be reading (its first use in a kernel, or one
+// separated from the last by another barrier): the leading barrier of block_sum, which only protects such a reader, is
+// dropped.  Same order of additions, same bits.
+__device__ __forceinline__ float block_sum_fresh(float v, float *sred) {
+	v = wave_sum(v);
+	if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = v;
+	__syncthreads();
+	return (sred[0] + sred[1]) + (sred[2] + sred[3]);
+}
+
 __device__ __forceinline__ float b2f(int d, int j) {  // signed byte j of d -> float (exact)
 	return (float)(int8_t)(d >> (8 * j));
 }
