@@ -381,8 +381,26 @@ def main():
             "note": "tg_qgemm_dev, 20 back-to-back launches incl. the quantising pre-pass; algorithmic 2*M*K*N flops against the dense int8 "
                     "rate; the matrix cores execute 3x that (three int8 digit planes of the activations)",
         }
+        # the shader clock the part held inside the matrix kernel itself (every workgroup reports its own clocks): random
+        # operands as above, and all-zero activations, for which the power limit leaves the clock higher
+        gz = tg.DeviceBuffer.from_numpy(np.zeros((gm, gk), np.float32))
+        clocks = {}
+        for label, abuf in (("random_operands", ga), ("zero_activations", gz)):
+            for _ in range(3):
+                gw.gemm(gc, abuf, gm)
+            mhz, wg_us, nwg = gw.gemm_clock(gc, abuf, gm)
+            tg.synchronize()
+            ev.record(e0, stream)
+            for _ in range(10):
+                gw.gemm(gc, abuf, gm)
+            ev.record(e1, stream)
+            tg.synchronize()
+            clocks[label] = {"shader_clock_mhz": mhz, "workgroup_lifetime_us": wg_us, "workgroups": nwg,
+                             "entry_point_us": ev.elapsed_ms(e0, e1) * 1e3 / 10}
+        extra_rooflines["prefill_gemm"]["clock_inside_the_kernel"] = clocks
+        gz.free()
         gw.free()
-        del ga, gc
+        del ga, gc, gz
         # what the integer matrix cores sustain when every compute unit issues nothing else (register operands, no
         # memory traffic): 32 clocks per instruction always, but the clock the part holds depends on the operand values
         cpm, mhz = C.c_double(), C.c_double()

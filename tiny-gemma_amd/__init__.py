@@ -126,6 +126,7 @@ def lib():
     L.tg_debug_launch_chain.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
     L.tg_debug_grid_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p]
     L.tg_set_fused_decode.argtypes = [C.c_int, C.c_int, C.c_int]
+    L.tg_debug_gemm_clock.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double), c_i32p]
     L.tg_debug_fused_timestamps.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
     L.tg_debug_handover.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p, c_i32p, c_i32p]
     L.tg_debug_gemm_launches.argtypes = [C.POINTER(C.c_longlong)] * 3
@@ -238,6 +239,12 @@ class QWeight:
 
     def gemm(self, C_dev, A_dev, m):
         check(lib().tg_qgemm_dev(C_dev.p, A_dev.p, self.h, m))
+
+    def gemm_clock(self, C_dev, A_dev, m):
+        """tg_qgemm_dev with the matrix kernel reporting the shader clock it ran at: (MHz, average workgroup lifetime in us, workgroups)."""
+        mhz, us, n = C.c_double(), C.c_double(), C.c_int32()
+        check(lib().tg_debug_gemm_clock(C_dev.p, A_dev.p, self.h, m, C.byref(mhz), C.byref(us), C.byref(n)))
+        return mhz.value, us.value, n.value
 
     def gemm_static(self, C_dev, A_dev, m):
         """tg_qgemm_dev on the library's fixed scratch: allocates nothing."""

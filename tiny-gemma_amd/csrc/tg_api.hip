@@ -538,6 +538,20 @@ int tg_qgemm_dev(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 // tg_qgemm_dev on the fixed scratch above: no hipMalloc/hipFree, nothing set up on the way.  Calls share the one
 // array (the planes of the previous call are overwritten; nothing in it needs to start at zero), so calls that
 // overlap on one GPU would race: the library's single stream orders them.
+// tg_qgemm_dev with every workgroup of the matrix kernel reporting the clocks it lived for (see tg_gemm_clk)
+int tg_debug_gemm_clock(float *C_dev, const float *A_dev, const tg_qweight *w, int m, double *clock_mhz, double *workgroup_us, int *workgroups) {
+	if (!clock_mhz || !workgroup_us || !workgroups) return tg_fail(TG_ERR_BAD_ARG, "null argument");
+	if (int rc = ensure_init()) return rc;
+	constexpr int MAX_WGS = 1 << 16;
+	if (!w || m < 1 || (long long)((m + 127) / 128) * w->p.ntiles_g * 2 > MAX_WGS) return tg_fail(TG_ERR_BAD_ARG, "bad argument (at most 32768 output tiles)");
+	unsigned long long *buf = nullptr;
+	if (int rc = tg_gemm_clk_begin(&buf, MAX_WGS, g_stream)) return rc;
+	int rc = tg_qgemm_dev(C_dev, A_dev, w, m);
+	if (rc == TG_OK && hipStreamSynchronize(g_stream) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipStreamSynchronize failed");
+	const int rc2 = tg_gemm_clk_end(buf, MAX_WGS, clock_mhz, workgroup_us, workgroups);
+	return rc != TG_OK ? rc : rc2;
+}
+
 int tg_qgemm_dev_static(float *C_dev, const float *A_dev, const tg_qweight *w, int m) {
 	if (!g_inited || !g_static_scratch) return tg_fail(TG_ERR_STATE, "tg_init has not run: this entry point sets nothing up itself");
 	if (!C_dev || !A_dev || !w || m < 1) return tg_fail(TG_ERR_BAD_ARG, "bad argument");

@@ -24,7 +24,7 @@ namespace {
 __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, const float *rms_q, const float *rms_k, const float *cos_t,
                                                           const float *sin_t, int host_pos, int host_bp, int nblocks, int chunk,
                                                           const TgAttnDecode a_in) {
-	if ((int)blockIdx.x >= nblocks) {  // extra workgroups: prefetch the next launch's weights and leave
+	if (__builtin_expect((int)blockIdx.x >= nblocks, 0)) {  // extra workgroups: prefetch the next launch's weights and leave
 		tg_prefetch_dispatch(a_in.pf, a_in.pf2, nblocks);
 		return;
 	}

@@ -357,6 +357,11 @@ __device__ __forceinline__ void gemm_static_for(F &&f) {
 	gemm_static_for_impl(std::make_integer_sequence<int, N>{}, f);
 }
 
+// Debug (tg_debug_gemm_clock): when this points at a buffer, thread 0 of every workgroup of gemm_i8_lds_kernel leaves
+// the shader clocks and the ticks of the constant 100 MHz counter it lived for: their ratio is the clock the part held
+// while the kernel ran (it lowers the clock under the power limit, by an amount that depends on the operand values).
+__device__ unsigned long long *tg_gemm_clk = nullptr;
+
 template <bool GEGLU, bool LUTLDS>
 __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int8_t *Apack, const float *rowinv, const int8_t *Wg,
                                                              const float *scales, int M, int K, int ldc, const float *lut, float gmin,
@@ -365,6 +370,12 @@ __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int
 	extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];  // LDS_NSLOT slots; the GeLU table afterwards
 	const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, hb = lane >> 5;
 	const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+	unsigned long long *const clkp = tg_gemm_clk;
+	unsigned long long clk_c0 = 0, clk_r0 = 0;
+	if (clkp != nullptr) {
+		clk_c0 = __builtin_readcyclecounter();
+		clk_r0 = __builtin_amdgcn_s_memrealtime();
+	}
 	// (row block, column tile) of this workgroup: every XCD a contiguous share, row blocks fastest (as gemm_i8_kernel)
 	int tile, mblock;
 	{
@@ -503,6 +514,10 @@ __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int
 	if (GEGLU && rowmax_part != nullptr) {
 		omax = fmaxf(omax, tg_red_partner<32>(omax));
 		if (hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(omax));
+	}
+	if (clkp != nullptr && tid == 0) {
+		clkp[2 * (size_t)blockIdx.x] = __builtin_readcyclecounter() - clk_c0;
+		clkp[2 * (size_t)blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - clk_r0;
 	}
 }
 
@@ -778,3 +793,34 @@ int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu) {
 	return (eff(wgs) < 0.6 && eff(2 * wgs) > eff(wgs) + 0.1) ? 2 : 1;
 }
 
+
+// tg_debug_gemm_clock: the buffer gemm_i8_lds_kernel leaves its clock readings in (n workgroups at most), and their
+// evaluation: sum of shader clocks / sum of 100 MHz ticks over the workgroups that ran.
+int tg_gemm_clk_begin(unsigned long long **buf, int n, hipStream_t s) {
+	TG_HIP(hipMalloc((void **)buf, sizeof(unsigned long long) * 2 * (size_t)n));
+	TG_HIP(hipMemsetAsync(*buf, 0, sizeof(unsigned long long) * 2 * (size_t)n, s));
+	TG_HIP(hipStreamSynchronize(s));
+	TG_HIP(hipMemcpyToSymbol(HIP_SYMBOL(tg_gemm_clk), buf, sizeof(*buf)));
+	return TG_OK;
+}
+int tg_gemm_clk_end(unsigned long long *buf, int n, double *clock_mhz, double *workgroup_us, int *workgroups) {
+	unsigned long long *null_ptr = nullptr;
+	const hipError_t e0 = hipMemcpyToSymbol(HIP_SYMBOL(tg_gemm_clk), &null_ptr, sizeof(null_ptr));
+	std::vector<unsigned long long> h(2 * (size_t)n);
+	const hipError_t e1 = hipMemcpy(h.data(), buf, sizeof(unsigned long long) * h.size(), hipMemcpyDeviceToHost);
+	(void)hipFree(buf);
+	if (e0 != hipSuccess || e1 != hipSuccess) return tg_fail(TG_ERR_HIP, "reading the clock samples failed");
+	double c = 0.0, r = 0.0;
+	int k = 0;
+	for (int i = 0; i < n; i++)
+		if (h[2 * (size_t)i + 1] != 0) {
+			c += (double)h[2 * (size_t)i];
+			r += (double)h[2 * (size_t)i + 1];
+			k++;
+		}
+	if (k == 0) return tg_fail(TG_ERR_STATE, "the product did not run on the kernel with two workgroups per compute unit (too few rows or tiles)");
+	*clock_mhz = 100.0 * c / r;
+	*workgroup_us = r / k / 100.0;
+	*workgroups = k;
+	return TG_OK;
+}

@@ -331,7 +331,7 @@ __device__ __forceinline__ TgGemv with_hot_args(const TgGemv &g_in, const void *
 #define TG_GEMV_ARGS \
 	const void *a0, const void *a1, const void *a2, const void *a3, const int8_t *W, int hidden, int K, int nmain, int aux, const TgGemv g
 #define TG_GEMV_BODY(PRO, EPI, AUX, DEPTH)                                                            \
-	if ((int)blockIdx.x >= nmain) { /* extra workgroups: prefetch the next launch's weights and leave */ \
+	if (__builtin_expect((int)blockIdx.x >= nmain, 0)) { /* extra workgroups: prefetch the next launch's weights and leave */ \
 		tg_prefetch_dispatch(g.pf, g.pf2, nmain);                                                     \
 		return;                                                                                       \
 	}                                                                                                 \

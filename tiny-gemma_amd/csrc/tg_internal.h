@@ -287,6 +287,8 @@ void tg_launch_gemm_mfma(float *C, const int8_t *apack, const float *rowfac, con
                          int ntiles, int epi, const float *lut, float gmin, float geps, int lut_size, float *rowmax_part,
                          int kparts, size_t part_stride, hipStream_t s);
 extern int g_gemm_lds, g_gemm_lds_cus, g_gemm_lds_ksplit;
+int tg_gemm_clk_begin(unsigned long long **buf, int n, hipStream_t s);
+int tg_gemm_clk_end(unsigned long long *buf, int n, double *clock_mhz, double *workgroup_us, int *workgroups);
 extern long g_gemm_launches[3];
 // parts of K (1, 2, 4) a plain-epilogue product should run in; part p writes C + p * part_stride, the consumer adds them
 int tg_gemm_mfma_k_parts(int M, int K, int ntiles, int n_cu);
