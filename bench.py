@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0   # dense int8 matrix rate
 # HBM bytes of one tg_gemv_lmhead_argmax launch from two `rocprofv3 --pmc` runs (FETCH_SIZE x 1.9999 +
 # WRITE_SIZE x 1.0000, both in KiB, scaled on a 256 MiB copy kernel): profiles/decode_1B_hbm_traffic.md
-LMHEAD_TRAFFIC_BYTES = {"1B": 304_493_961}
+LMHEAD_TRAFFIC_BYTES = {"1B": 304_496_732}
 
 MODELS = {
     # name: (prompt tokens, decode bytes of weights+scales per token, LM-head GEMV algorithmic bytes)

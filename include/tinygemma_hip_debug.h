@@ -125,7 +125,8 @@ int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins,
  * per instruction (32 when nothing stalls) and the average shader clock in MHz during the loop, which the part
  * lowers under load depending on the operand values.  workgroups <= 4096, iters <= 2^20. */
 int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_per_mfma, double *clock_mhz);
-/* tg_qgemm_dev (same arguments) with the matrix kernel that runs two workgroups per compute unit reporting its own clocks:
+/* tg_qgemm_dev (same arguments), five times back to back, with the matrix kernel that runs two workgroups per compute unit
+ * reporting its own clocks (the figures are those of the last launch):
  * *clock_mhz = shader clocks / ticks of the constant 100 MHz counter, summed over the workgroups (the clock the part held
  * while the product ran: it lowers it under the power limit, more so the more operand bits toggle), *workgroup_us = the
  * average lifetime of a workgroup, *workgroups = how many reported.  TG_ERR_STATE when the product is too small for that
