@@ -528,7 +528,7 @@ __global__ __launch_bounds__(GNT, 2) void gemm_i8_lds_kernel(float *C, const int
 // four waves take the K stages round-robin (stage w, w + 4, ...), each with a private register pipeline: no LDS and
 // no barrier in the main loop, weights fetched straight from global memory in operand order (32 lanes x 16 bytes =
 // 512 contiguous bytes per fragment).  The integer partial sums are added through LDS at the end (exact, so the
-// result equals the unsplit one bit for bit) and wave j finishes column block j.
+// result equals the unsplit one bit for bit) and every wave finishes a quarter of each column block.
 // gridDim.z > 1 (plain epilogue only): K is also cut into gridDim.z equal parts over workgroups; part z writes its own
 // partial result C + z * part_stride and the consumer adds them (a long K with few rows and few column tiles would
 // otherwise run on a few dozen compute units, each pulling megabytes of weights through its own L1).
@@ -539,7 +539,8 @@ __global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int
                                                              size_t part_stride) {
 	__shared__ __attribute__((aligned(16))) i32x4 red[4][3][4][64];  // [wave][plane][quarter of the 16 registers][lane]
 	__shared__ float lut_lds[(GEGLU && LUTLDS) ? LUT_LDS_MAX : 1];
-	__shared__ float pmax[2][32];
+	__shared__ float pmax[4][32];
+	typedef i32x4 fin_t;
 	const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c = lane & 31, hb = lane >> 5;
 	const int tile = blockIdx.x, mtile = blockIdx.y, z = blockIdx.z;
 	const int nstage = K / KSTAGE / (int)gridDim.z, last = nstage - 1;  // stages of this workgroup's part of K
@@ -601,9 +602,10 @@ __global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int
 	if (i0 < n_it) stage(i0, std::integral_constant<int, 0>{});
 	if (i0 + 1 < n_it) stage(i0 + 1, std::integral_constant<int, 1>{});
 
-	// reduction over the waves, one column block per round; STORE: wave j keeps block j; GEGLU: waves 0 and 1 keep
-	// the up block j and the gate block j + 2
-	i32x16 fin[2][3];
+	// reduction over the waves, one column block per round: every wave leaves its partial sums of the block in LDS and
+	// adds up one quarter of it (registers 4 w .. 4 w + 3 of each plane, from all four waves).  After the four
+	// rounds wave w holds, of every column block j, the four consecutive output columns 32 j + 8 w + 4 (lane / 32) ..
+	fin_t fin[4][3];
 #pragma unroll
 	for (int j = 0; j < 4; j++) {
 #pragma unroll
@@ -612,61 +614,48 @@ __global__ __launch_bounds__(GNT) void gemm_i8_skinny_kernel(float *C, const int
 			for (int qq = 0; qq < 4; qq++)
 				red[w][p][qq][lane] = i32x4{acc[p][j][4 * qq], acc[p][j][4 * qq + 1], acc[p][j][4 * qq + 2], acc[p][j][4 * qq + 3]};
 		__syncthreads();
-		const int owner = GEGLU ? (j & 1) : j;
-		if (w == owner) {
 #pragma unroll
-			for (int p = 0; p < 3; p++)
-#pragma unroll
-				for (int qq = 0; qq < 4; qq++) {
-					const i32x4 t = (red[0][p][qq][lane] + red[1][p][qq][lane]) + (red[2][p][qq][lane] + red[3][p][qq][lane]);
-#pragma unroll
-					for (int e = 0; e < 4; e++) fin[(GEGLU && j >= 2) ? 1 : 0][p][4 * qq + e] = t[e];
-				}
-		}
-		__syncthreads();
+		for (int p = 0; p < 3; p++) fin[j][p] = (red[0][p][w][lane] + red[1][p][w][lane]) + (red[2][p][w][lane] + red[3][p][w][lane]);
+		if (j < 3) __syncthreads();
 	}
 
 	const int m = mtile * 32 + c;
 	const float rs = rowinv[m];
-	const int jb = w;  // column block this wave finishes (GEGLU: waves 0 and 1 only)
-	auto value = [&](const i32x16 *f, int i, float scale) {
-		const float v = fmaf((float)f[2][i], 65536.0f, fmaf((float)f[1][i], 256.0f, (float)f[0][i]));
+	auto value = [&](const fin_t *f, int e, float scale) {
+		const float v = fmaf((float)f[2][e], 65536.0f, fmaf((float)f[1][e], 256.0f, (float)f[0][e]));
 		return (v * rs) * scale;
 	};
 	float omax = 0.0f;
-	if (!GEGLU || w < 2) {
-		f32x4 sc_u[4], sc_g[4];
+	const int col = 8 * w + 4 * hb;  // of a column block
+	f32x4 sc[4];
 #pragma unroll
-		for (int q = 0; q < 4; q++) {
-			sc_u[q] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * jb + 8 * q + 4 * hb);
-			if (GEGLU) sc_g[q] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * (jb + 2) + 8 * q + 4 * hb);
-		}
-		if (m < M) {
-			float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + 32 * jb + 4 * hb;
+	for (int j = 0; j < 4; j++) sc[j] = *reinterpret_cast<const f32x4 *>(scales + tile * TG_CT + 32 * j + col);
+	if (m < M) {
+		float *crow = C + (size_t)m * ldc + (size_t)tile * (GEGLU ? TG_CT / 2 : TG_CT) + col;
 #pragma unroll
-			for (int q = 0; q < 4; q++) {
-				f32x4 o;
+		for (int j = 0; j < (GEGLU ? 2 : 4); j++) {  // GEGLU: blocks 0 and 1 are up, 2 and 3 their gates
+			f32x4 o;
 #pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int i = 4 * q + e;
-					if (GEGLU) {
-						const float gate = value(fin[1], i, sc_g[q][e]);
-						o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
-						       value(fin[0], i, sc_u[q][e]);
-						omax = fmaxf(omax, fabsf(o[e]));
-					} else {
-						o[e] = value(fin[0], i, sc_u[q][e]);
-					}
+			for (int e = 0; e < 4; e++) {
+				if (GEGLU) {
+					const float gate = value(fin[j + 2], e, sc[j + 2][e]);
+					o[e] = (LUTLDS ? gelu_lut(gate, lut_lds, gmin, geps, ginv, lut_size) : gelu_lut(gate, lut, gmin, geps, ginv, lut_size)) *
+					       value(fin[j], e, sc[j][e]);
+					omax = fmaxf(omax, fabsf(o[e]));
+				} else {
+					o[e] = value(fin[j], e, sc[j][e]);
 				}
-				*reinterpret_cast<f32x4 *>(crow + 8 * q) = o;
 			}
+			*reinterpret_cast<f32x4 *>(crow + 32 * j) = o;
 		}
 	}
 	if (GEGLU && rowmax_part != nullptr) {
 		omax = fmaxf(omax, tg_red_partner<32>(omax));
-		if (w < 2 && hb == 0) pmax[w][c] = omax;
+		if (hb == 0) pmax[w][c] = omax;
 		__syncthreads();
-		if (w == 0 && hb == 0 && m < M) atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m, __float_as_uint(fmaxf(pmax[0][c], pmax[1][c])));
+		if (w == 0 && hb == 0 && m < M)
+			atomicMax(reinterpret_cast<unsigned *>(rowmax_part) + m,
+			          __float_as_uint(fmaxf(fmaxf(pmax[0][c], pmax[1][c]), fmaxf(pmax[2][c], pmax[3][c]))));
 	}
 }
 
