@@ -421,6 +421,18 @@ def main():
                                    "which it only holds for all-zero operands or a mostly idle chip.  frac_of_sustained_int8_rate = executed "
                                    "(3 x algorithmic) rate / the uniform_int8 figure")
 
+        # what a compute unit pulls through its vector L1 (one workgroup of 4 waves per unit): from its XCD's L2, and
+        # from memory with every unit streaming a share of its own
+        a, b, c3 = C.c_double(), C.c_double(), C.c_double()
+        fill = {}
+        for label, wgs, kib, disjoint, steps in (("l2_256wg", 256, 1024, 0, 256), ("l2_512wg", 512, 1024, 0, 256), ("l2_1024wg", 1024, 1024, 0, 256),
+                                                  ("memory_256wg", 256, 1 << 20, 1, 126), ("memory_1024wg", 1024, 1 << 20, 1, 30)):
+            tg.check(L.tg_debug_l1_fill(wgs, 8, steps, kib, disjoint, C.byref(a), C.byref(b), C.byref(c3)))
+            fill[label] = {"GBps_per_workgroup": a.value, "TBps_all": b.value / 1e3, "clock_mhz": c3.value}
+        pg["l1_fill"] = fill
+        pg["l1_fill_note"] = ("tg_debug_l1_fill: workgroups of 256 threads stream 16-byte loads, 8 x 4 KiB per step, two steps in flight; l2 = all walk "
+                              "one megabyte (L2 hits, never L1 hits), memory = every workgroup streams its own share of a gigabyte")
+
     # ---- what a dependent launch and a device-wide barrier cost here; the same steps replayed from captured graphs ----
     launch_floor = None
     if not args.headline_only:

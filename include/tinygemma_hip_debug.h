@@ -125,6 +125,15 @@ int tg_debug_grid_barrier(int rounds, int workgroups, int fenced, int max_spins,
  * per instruction (32 when nothing stalls) and the average shader clock in MHz during the loop, which the part
  * lowers under load depending on the operand values.  workgroups <= 4096, iters <= 2^20. */
 int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_per_mfma, double *clock_mhz);
+/* What a compute unit can pull through its vector L1 (no counterpart in the reference: measurement aid).  `workgroups`
+ * x 256 threads walk a buffer of buf_kib KiB (a power of two, 64 .. 2^20) cyclically with 16-byte loads,
+ * loads_per_step (4, 8 or 16) x 4 KiB per step and workgroup, the next step requested before this one is consumed,
+ * `steps` (even, <= 2^16) steps.  disjoint = 0: all walk the same buffer from different starts (1 MiB stays in every
+ * XCD's L2 and never in an L1); 1: every workgroup starts in a share of its own (a large buffer: streamed from
+ * memory).  Returns GB/s of the median workgroup, GB/s of the whole launch (first start to last end) and the shader
+ * clock.  workgroups <= 4096. */
+int tg_debug_l1_fill(int workgroups, int loads_per_step, int steps, int buf_kib, int disjoint, double *gbps_per_workgroup, double *gbps_total,
+                     double *clock_mhz);
 /* tg_qgemm_dev (same arguments), five times back to back, with the matrix kernel that runs two workgroups per compute unit
  * reporting its own clocks (the figures are those of the last launch):
  * *clock_mhz = shader clocks / ticks of the constant 100 MHz counter, summed over the workgroups (the clock the part held

@@ -366,3 +366,12 @@ def test_machine_probes_return_sane_figures(tg):
         assert 31.9 < cpm.value < 36.0 and 1000.0 < mhz.value < 2600.0
     assert L.tg_debug_mfma_clock(0, 10, 0, C.byref(cpm), C.byref(mhz)) == -4
     assert L.tg_debug_mfma_clock(8, 10, 3, C.byref(cpm), C.byref(mhz)) == -4
+    # what a compute unit pulls through its L1: from its XCD's L2 (a shared megabyte) far more than from memory
+    per_wg, total, per_wg_mem, total_mem = C.c_double(), C.c_double(), C.c_double(), C.c_double()
+    tg.check(L.tg_debug_l1_fill(256, 8, 256, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)))
+    tg.check(L.tg_debug_l1_fill(256, 8, 126, 1 << 20, 1, C.byref(per_wg_mem), C.byref(total_mem), C.byref(mhz)))
+    print(f"l1 fill: {per_wg.value:.0f} GB/s per workgroup from L2 ({total.value / 1e3:.1f} TB/s), {per_wg_mem.value:.0f} from memory ({total_mem.value / 1e3:.1f} TB/s)")
+    assert 30.0 < per_wg.value < 400.0 and 5.0 < per_wg_mem.value < per_wg.value and total_mem.value < 8000.0
+    assert L.tg_debug_l1_fill(256, 5, 256, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
+    assert L.tg_debug_l1_fill(256, 8, 255, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
+    assert L.tg_debug_l1_fill(256, 8, 256, 1000, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4

@@ -12,10 +12,15 @@
 // registers (no memory traffic at all) and reports clocks per instruction and the clock itself, for operands that
 // are all zero, small, or uniformly random int8: the ceiling the prefill GEMM can be measured against.
 //
+// tg_debug_l1_fill: the rate at which a compute unit takes data that its L1 does not hold (from its XCD's L2, or from
+// memory): the bound of the prefill products on short prompts, whose workgroups pull their operands straight through
+// the L1 with one wave per SIMD.
+//
 // Every wait in here is bounded: a workgroup that does not see the others arrive within max_spins polls gives up,
 // sets a flag and goes on, so the kernel always drains.
 
 #include "tg_internal.h"
+#include <algorithm>
 
 extern hipStream_t tg_probe_stream();  // the library's stream (tg_api.hip)
 extern int tg_probe_n_cu();             // compute units of the device the library runs on
@@ -348,6 +353,43 @@ __global__ __launch_bounds__(PNT) void mfma_clock_kernel(long long *out, int *si
 	}
 }
 
+// What one compute unit can pull through its vector L1: every workgroup walks `buf` (a power of two of 16-byte
+// pieces, cyclically, from a start of its own) with 16-byte loads, N x 4 KiB per step, the next step's loads issued
+// before this step's are consumed.  A buffer of a megabyte stays in every XCD's L2 and never in a 32 KB L1.
+template <int N>
+__global__ __launch_bounds__(PNT) void l1_fill_kernel(const int4 *buf, unsigned mask, unsigned start_stride, int steps, long long *out, int *sink) {
+	const unsigned tid = threadIdx.x;
+	unsigned pos = blockIdx.x * start_stride + tid;
+	int4 a[N], b[N];
+	int x = 0;
+	auto load = [&](int4 *r) {
+#pragma unroll
+		for (int i = 0; i < N; i++) r[i] = buf[(pos + i * PNT) & mask];
+		pos += N * PNT;
+	};
+	auto eat = [&](const int4 *r) {
+#pragma unroll
+		for (int i = 0; i < N; i++) x ^= r[i].x ^ r[i].y ^ r[i].z ^ r[i].w;
+	};
+	__syncthreads();
+	const long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+	load(a);
+	for (int st = 0; st < steps; st += 2) {
+		load(b);
+		eat(a);
+		load(a);
+		eat(b);
+	}
+	eat(a);
+	const long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+	if (x == 0x5a5a5a5a && steps < 0) sink[tid] = x;  // keeps the loads alive; never taken
+	if (tid == 0) {
+		out[3 * blockIdx.x] = c1 - c0;
+		out[3 * blockIdx.x + 1] = r0;
+		out[3 * blockIdx.x + 2] = r1;
+	}
+}
+
 struct Timer {
 	hipEvent_t e0 = nullptr, e1 = nullptr;
 	int begin(hipStream_t s) {
@@ -534,6 +576,59 @@ int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_
 		}
 	}
 	(void)hipFree(buf);
+	return rc;
+}
+
+int tg_debug_l1_fill(int workgroups, int loads_per_step, int steps, int buf_kib, int disjoint, double *gbps_per_workgroup, double *gbps_total,
+                     double *clock_mhz) {
+	if (workgroups < 1 || workgroups > 4096 || (loads_per_step != 4 && loads_per_step != 8 && loads_per_step != 16) || steps < 2 || steps > (1 << 16) ||
+	    (steps & 1) || buf_kib < 64 || buf_kib > (1 << 20) || (buf_kib & (buf_kib - 1)) || !gbps_per_workgroup || !gbps_total || !clock_mhz)
+		return tg_fail(TG_ERR_BAD_ARG, "bad argument (loads_per_step 4, 8 or 16; steps even; buf_kib a power of two from 64 to 2^20)");
+	hipStream_t s = tg_probe_stream();
+	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
+	const size_t bytes = (size_t)buf_kib << 10, pieces = bytes / 16;
+	char *mem = nullptr;
+	TG_HIP(hipMalloc((void **)&mem, bytes + sizeof(long long) * 3 * (size_t)workgroups + sizeof(int) * PNT));
+	long long *out = (long long *)(mem + bytes);
+	int *sink = (int *)(out + 3 * (size_t)workgroups);
+	int rc = TG_OK;
+	if (hipMemsetAsync(mem, 1, bytes, s) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemsetAsync failed");
+	// disjoint: every workgroup starts in a share of its own (a large buffer streamed once from memory); otherwise the
+	// starts are 4 KiB x an odd number apart, so that workgroups of one compute unit never walk in step
+	const unsigned stride = disjoint ? (unsigned)(pieces / (size_t)workgroups) : 37u * PNT;
+	for (int pass = 0; pass < 2 && rc == TG_OK; pass++) {
+		const dim3 grid((unsigned)workgroups), block(PNT);
+		if (loads_per_step == 4) hipLaunchKernelGGL(l1_fill_kernel<4>, grid, block, 0, s, (const int4 *)mem, (unsigned)(pieces - 1), stride, steps, out, sink);
+		if (loads_per_step == 8) hipLaunchKernelGGL(l1_fill_kernel<8>, grid, block, 0, s, (const int4 *)mem, (unsigned)(pieces - 1), stride, steps, out, sink);
+		if (loads_per_step == 16) hipLaunchKernelGGL(l1_fill_kernel<16>, grid, block, 0, s, (const int4 *)mem, (unsigned)(pieces - 1), stride, steps, out, sink);
+	}
+	if (rc == TG_OK && (hipStreamSynchronize(s) != hipSuccess || hipGetLastError() != hipSuccess)) rc = tg_fail(TG_ERR_HIP, "launch failed");
+	if (rc == TG_OK) {
+		std::vector<long long> h(3 * (size_t)workgroups);
+		if (hipMemcpy(h.data(), out, sizeof(long long) * h.size(), hipMemcpyDeviceToHost) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+		if (rc == TG_OK) {
+			const double wg_bytes = (double)(steps + 1) * loads_per_step * PNT * 16.0;
+			std::vector<double> ticks((size_t)workgroups);
+			long long first = h[1], last = h[2];
+			double c = 0.0, r = 0.0;
+			for (int i = 0; i < workgroups; i++) {
+				ticks[(size_t)i] = (double)(h[3 * (size_t)i + 2] - h[3 * (size_t)i + 1]);
+				first = std::min(first, h[3 * (size_t)i + 1]);
+				last = std::max(last, h[3 * (size_t)i + 2]);
+				c += (double)h[3 * (size_t)i];
+				r += ticks[(size_t)i];
+			}
+			std::sort(ticks.begin(), ticks.end());
+			const double med = ticks[(size_t)workgroups / 2];
+			if (med <= 0.0 || last <= first) rc = tg_fail(TG_ERR_STATE, "the constant-rate counter did not advance");
+			else {
+				*gbps_per_workgroup = wg_bytes / (med * 10.0);  // a tick is 10 ns
+				*gbps_total = wg_bytes * workgroups / ((double)(last - first) * 10.0);
+				*clock_mhz = 100.0 * c / r;
+			}
+		}
+	}
+	(void)hipFree(mem);
 	return rc;
 }
 
