@@ -132,6 +132,10 @@ int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_
  * XCD's L2 and never in an L1); 1: every workgroup starts in a share of its own (a large buffer: streamed from
  * memory).  Returns GB/s of the median workgroup, GB/s of the whole launch (first start to last end) and the shader
  * clock.  workgroups <= 4096. */
+/* How the dispatcher deals workgroups to the 8 XCDs (measurement aid, no counterpart in the reference): n_launches
+ * (<= 64) launches of workgroups[i] x 256 threads back to back on tg_stream().  first_xcd[i] = the XCD workgroup 0 of
+ * launch i ran on, out_of_order[i] = how many of its workgroups b did not run on XCD (first_xcd[i] + b) mod 8. */
+int tg_debug_xcd_deal(int n_launches, const int *workgroups, int *first_xcd, int *out_of_order);
 int tg_debug_l1_fill(int workgroups, int loads_per_step, int steps, int buf_kib, int disjoint, double *gbps_per_workgroup, double *gbps_total,
                      double *clock_mhz);
 /* tg_qgemm_dev (same arguments), five times back to back, with the matrix kernel that runs two workgroups per compute unit

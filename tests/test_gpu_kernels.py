@@ -373,5 +373,14 @@ def test_machine_probes_return_sane_figures(tg):
     print(f"l1 fill: {per_wg.value:.0f} GB/s per workgroup from L2 ({total.value / 1e3:.1f} TB/s), {per_wg_mem.value:.0f} from memory ({total_mem.value / 1e3:.1f} TB/s)")
     assert 30.0 < per_wg.value < 400.0 and 5.0 < per_wg_mem.value < per_wg.value and total_mem.value < 8000.0
     assert L.tg_debug_l1_fill(256, 5, 256, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
+    # the deal of workgroups to the XCDs that the few-row GEMM, the prefetch workgroups and the tile mappings rely on:
+    # round-robin inside a launch, and launches that follow each other on the stream start on the same XCD
+    wgs = [288, 416, 16, 3, 1000, 257]
+    n = len(wgs)
+    first, bad = (C.c_int * n)(), (C.c_int * n)()
+    tg.check(L.tg_debug_xcd_deal(n, (C.c_int * n)(*wgs), first, bad))
+    print("xcd deal: first", list(first), "out of order", list(bad))
+    assert list(bad) == [0] * n and len(set(first)) == 1 and 0 <= first[0] < 8
+    assert L.tg_debug_xcd_deal(0, (C.c_int * n)(*wgs), first, bad) == -4
     assert L.tg_debug_l1_fill(256, 8, 255, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
     assert L.tg_debug_l1_fill(256, 8, 256, 1000, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4

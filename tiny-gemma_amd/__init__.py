@@ -131,6 +131,7 @@ def lib():
     L.tg_debug_handover.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), c_i32p, c_i32p, c_i32p]
     L.tg_debug_gemm_launches.argtypes = [C.POINTER(C.c_longlong)] * 3
     L.tg_debug_mfma_clock.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    L.tg_debug_xcd_deal.argtypes = [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]
     L.tg_debug_l1_fill.argtypes = [C.c_int] * 5 + [C.POINTER(C.c_double)] * 3
     L.tg_decode_profile.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_double), c_i32p]
     L.tg_debug_repeat_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]

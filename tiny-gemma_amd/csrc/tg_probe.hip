@@ -390,6 +390,11 @@ __global__ __launch_bounds__(PNT) void l1_fill_kernel(const int4 *buf, unsigned 
 	}
 }
 
+// Which XCD every workgroup of a launch ran on (for tg_debug_xcd_deal).
+__global__ __launch_bounds__(PNT) void xcd_deal_kernel(int *out) {
+	if (threadIdx.x == 0) out[blockIdx.x] = (int)probe_xcc_id();
+}
+
 struct Timer {
 	hipEvent_t e0 = nullptr, e1 = nullptr;
 	int begin(hipStream_t s) {
@@ -630,6 +635,39 @@ int tg_debug_l1_fill(int workgroups, int loads_per_step, int steps, int buf_kib,
 	}
 	(void)hipFree(mem);
 	return rc;
+}
+
+int tg_debug_xcd_deal(int n_launches, const int *workgroups, int *first_xcd, int *out_of_order) {
+	if (n_launches < 1 || n_launches > 64 || !workgroups || !first_xcd || !out_of_order) return tg_fail(TG_ERR_BAD_ARG, "bad argument (1 to 64 launches)");
+	size_t total = 0;
+	for (int i = 0; i < n_launches; i++) {
+		if (workgroups[i] < 1 || workgroups[i] > 65536) return tg_fail(TG_ERR_BAD_ARG, "1 to 65536 workgroups per launch");
+		total += (size_t)workgroups[i];
+	}
+	hipStream_t s = tg_probe_stream();
+	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
+	int *buf = nullptr;
+	TG_HIP(hipMalloc((void **)&buf, sizeof(int) * total));
+	size_t at = 0;
+	for (int i = 0; i < n_launches; i++) {  // back to back, nothing else on the stream in between
+		hipLaunchKernelGGL(xcd_deal_kernel, dim3((unsigned)workgroups[i]), dim3(PNT), 0, s, buf + at);
+		at += (size_t)workgroups[i];
+	}
+	int rc = TG_OK;
+	if (hipStreamSynchronize(s) != hipSuccess || hipGetLastError() != hipSuccess) rc = tg_fail(TG_ERR_HIP, "launch failed");
+	std::vector<int> h(total);
+	if (rc == TG_OK && hipMemcpy(h.data(), buf, sizeof(int) * total, hipMemcpyDeviceToHost) != hipSuccess) rc = tg_fail(TG_ERR_HIP, "hipMemcpy failed");
+	(void)hipFree(buf);
+	if (rc != TG_OK) return rc;
+	at = 0;
+	for (int i = 0; i < n_launches; i++) {
+		first_xcd[i] = h[at];
+		int bad = 0;
+		for (int b = 0; b < workgroups[i]; b++) bad += h[at + (size_t)b] != ((h[at] + b) & 7);
+		out_of_order[i] = bad;
+		at += (size_t)workgroups[i];
+	}
+	return TG_OK;
 }
 
 }  // extern "C"
