@@ -37,7 +37,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, cons
 	a.host_pos = host_pos;
 	a.host_bp = host_bp;
 	a.chunk = chunk;
-	attn_decode_body<false>(a, (int)blockIdx.x, [] {});
+	attn_decode_body<true>(a, (int)blockIdx.x, [] {});
 }
 
 // Long contexts only: folds every TG_ATTN_FOLD consecutive partials into one partial of the same form (maximum, sum,

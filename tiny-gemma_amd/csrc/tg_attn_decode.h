@@ -193,8 +193,16 @@ __device__ __forceinline__ void attn_decode_body(const TgAttnDecode &a, int b, F
 #pragma unroll
 	for (int h = 0; h < NH; h++) q[h] = *reinterpret_cast<const af4 *>(&qs[h][4 * lane]);
 	if (b == 0 && w == 0) {  // KVCache::update_single, decode.hpp:49-70
-		*reinterpret_cast<af4 *>(a.kc + (size_t)cur * HD + 4 * lane) = knew;
-		*reinterpret_cast<af4 *>(a.vc + (size_t)cur * HD + 4 * lane) = vnew;
+		if (WT) {
+#pragma unroll
+			for (int c = 0; c < 4; c++) {
+				attn_store<true>(a.kc + (size_t)cur * HD + 4 * lane + c, knew[c]);
+				attn_store<true>(a.vc + (size_t)cur * HD + 4 * lane + c, vnew[c]);
+			}
+		} else {
+			*reinterpret_cast<af4 *>(a.kc + (size_t)cur * HD + 4 * lane) = knew;
+			*reinterpret_cast<af4 *>(a.vc + (size_t)cur * HD + 4 * lane) = vnew;
+		}
 	}
 
 	// the wave's blocks: scores, online softmax, P.V; m_run / l_run are those of the head of this lane's row

@@ -197,7 +197,7 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 #pragma unroll
 			for (int i = 0; i < PER; i++) {
 				const int d = tid + i * NT;
-				if (d < h) g.xr_out[d] = t[i];
+				if (d < h) st_f32<true>(&g.xr_out[d], t[i]);
 			}
 		}
 		// ops.hpp:126-180: x * rsqrt(mean(x^2) + eps) * (1 + w)
@@ -256,9 +256,9 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 
 	// ---------------- epilogue of tile `cur` ----------------
 	if (EPI == TG_EPI_STORE) {
-		epi_store<false>(red, C, cur, sc_cur_a, g.y);
+		epi_store<true>(red, C, cur, sc_cur_a, g.y);
 	} else if (EPI == TG_EPI_GEGLU) {
-		epi_geglu<false>(red, C, cur, sc_cur_a, sc_cur_b, g.y, lut_in_lds ? lut_s : g.lut, g.gmin, g.geps, g.lut_size);
+		epi_geglu<true>(red, C, cur, sc_cur_a, sc_cur_b, g.y, lut_in_lds ? lut_s : g.lut, g.gmin, g.geps, g.lut_size);
 	} else {
 		// TG_EPI_LOGITS: logits + first stage of the greedy argmax
 		// (ops.hpp:749-757: strict '>' scan from index 0, so the lowest index wins ties)
@@ -284,8 +284,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 		if (tid == 0) {
 			for (int i = 1; i < NWAVE; i++)
 				if (s_bv[it & 1][i] > bv || (s_bv[it & 1][i] == bv && s_bi[it & 1][i] < bi)) { bv = s_bv[it & 1][i]; bi = s_bi[it & 1][i]; }
-			g.blk_val[cur] = bv;
-			g.blk_idx[cur] = bi;
+			st_f32<true>(&g.blk_val[cur], bv);
+			__hip_atomic_store(&g.blk_idx[cur], bi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		}
 	}
 	if (!more) break;
