@@ -589,6 +589,9 @@ int tg_debug_l1_fill(int workgroups, int loads_per_step, int steps, int buf_kib,
 	if (workgroups < 1 || workgroups > 4096 || (loads_per_step != 4 && loads_per_step != 8 && loads_per_step != 16) || steps < 2 || steps > (1 << 16) ||
 	    (steps & 1) || buf_kib < 64 || buf_kib > (1 << 20) || (buf_kib & (buf_kib - 1)) || !gbps_per_workgroup || !gbps_total || !clock_mhz)
 		return tg_fail(TG_ERR_BAD_ARG, "bad argument (loads_per_step 4, 8 or 16; steps even; buf_kib a power of two from 64 to 2^20)");
+	// a launch that ends in seconds at any rate the machine reaches: at most 16 GiB read in all
+	if ((unsigned long long)workgroups * (unsigned long long)(steps + 1) * (unsigned long long)loads_per_step * 4096ull > (16ull << 30))
+		return tg_fail(TG_ERR_BAD_ARG, "workgroups x steps x loads_per_step x 4 KiB exceeds 16 GiB");
 	hipStream_t s = tg_probe_stream();
 	if (!s) return tg_fail(TG_ERR_STATE, "tg_init has not run");
 	const size_t bytes = (size_t)buf_kib << 10, pieces = bytes / 16;
