@@ -131,7 +131,7 @@ int tg_debug_mfma_clock(int workgroups, int iters, int operands, double *clocks_
  * `steps` (even, <= 2^16) steps.  disjoint = 0: all walk the same buffer from different starts (1 MiB stays in every
  * XCD's L2 and never in an L1); 1: every workgroup starts in a share of its own (a large buffer: streamed from
  * memory).  Returns GB/s of the median workgroup, GB/s of the whole launch (first start to last end) and the shader
- * clock.  workgroups <= 4096. */
+ * clock.  workgroups <= 4096, and workgroups x (steps + 1) x loads_per_step x 4 KiB <= 16 GiB (the launch ends in seconds). */
 /* How the dispatcher deals workgroups to the 8 XCDs (measurement aid, no counterpart in the reference): n_launches
  * (<= 64) launches of workgroups[i] x 256 threads back to back on tg_stream().  first_xcd[i] = the XCD workgroup 0 of
  * launch i ran on, out_of_order[i] = how many of its workgroups b did not run on XCD (first_xcd[i] + b) mod 8. */

@@ -384,3 +384,4 @@ def test_machine_probes_return_sane_figures(tg):
     assert L.tg_debug_xcd_deal(0, (C.c_int * n)(*wgs), first, bad) == -4
     assert L.tg_debug_l1_fill(256, 8, 255, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
     assert L.tg_debug_l1_fill(256, 8, 256, 1000, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4
+    assert L.tg_debug_l1_fill(4096, 16, 65536, 1024, 0, C.byref(per_wg), C.byref(total), C.byref(mhz)) == -4  # hours of reads
