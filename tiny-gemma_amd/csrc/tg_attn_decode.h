@@ -39,7 +39,7 @@ __device__ __forceinline__ void head_finish(const HeadIn &in, float mul, float o
 #pragma unroll
 	for (int i = 0; i < 4; i++) ss = fmaf(in.x[i], in.x[i], ss);
 	ss = wsum(ss);
-	const float irms = 1.0f / sqrtf(ss / (float)HD + 1e-06f);
+	const float irms = __builtin_amdgcn_rsqf(ss * (1.0f / (float)HD) + 1e-06f);
 #pragma unroll
 	for (int i = 0; i < 4; i++) x[i] = (in.x[i] * irms) * (in.w[i] + 1.0f);
 	out[0] = fmaf(in.c0, x[0], (-x[2]) * in.s0) * mul;
@@ -108,7 +108,7 @@ __device__ __forceinline__ af4 attn_head_finish(af4 x, af4 w, af4 cs4, af4 sn4, 
 #pragma unroll
 	for (int e = 0; e < 4; e++) ss = fmaf(x[e], x[e], ss);
 	ss = wsum(ss);
-	const float irms = 1.0f / sqrtf(ss / (float)HD + 1e-06f);
+	const float irms = __builtin_amdgcn_rsqf(ss * (1.0f / (float)HD) + 1e-06f);
 	const bool upper = (__lane_id() & 32) != 0;
 	af4 out;
 #pragma unroll
