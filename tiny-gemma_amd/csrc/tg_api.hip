@@ -1245,6 +1245,7 @@ static AttnGeom attn_geometry(tg_session *s, int l, bool full_grid) {
 	// a captured step is replayed at other positions: only then are the counters read from device memory
 	a.host_pos = full_grid ? -1 : s->pos;
 	a.host_bp = full_grid ? -1 : (Ld.is_sw ? s->bp_local : s->bp_global);
+	a.host_cur = full_grid ? -1 : a.host_bp % a.max_pos;
 	const int valid = std::min(s->pos + 1, a.max_pos);
 	ag.needs_merge = false;
 	a.chunk = attn_chunk_for(valid, &ag.needs_merge);

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(ANT) void attn_decode_kernel(const float *qkv, cons
 	a.host_pos = host_pos;
 	a.host_bp = host_bp;
 	a.chunk = chunk;
+	a.nblocks = nblocks;
 	attn_decode_body<true>(a, (int)blockIdx.x, [] {});
 }
 

@@ -202,16 +202,16 @@ __global__ __launch_bounds__(PNT) void attn_prefill_mfma_kernel(float *o, const 
 		}
 		return;
 	}
-	float lr[4];
+	float lr[4];  // 1 / l of the lane's four query rows: one division per row, then multiplications
 #pragma unroll
-	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+	for (int i = 0; i < 4; i++) lr[i] = 1.0f / __shfl(l_run, 4 * g + i, 64);
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0 + 4 * g + i;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] * lr[i];
 		}
 	}
 }
@@ -519,16 +519,16 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_split_kernel(float *o, 
 		}
 		return;
 	}
-	float lr[4];
+	float lr[4];  // 1 / l of the lane's four query rows: one division per row, then multiplications
 #pragma unroll
-	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+	for (int i = 0; i < 4; i++) lr[i] = 1.0f / __shfl(l_run, 4 * g + i, 64);
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0w + 4 * g + i;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] * lr[i];
 		}
 	}
 }
@@ -870,16 +870,16 @@ __global__ __launch_bounds__(256 * QG) void attn_prefill_planes_kernel(float *o,
 		}
 		return;
 	}
-	float lr[4];
+	float lr[4];  // 1 / l of the lane's four query rows: one division per row, then multiplications
 #pragma unroll
-	for (int i = 0; i < 4; i++) lr[i] = __shfl(l_run, 4 * g + i, 64);
+	for (int i = 0; i < 4; i++) lr[i] = 1.0f / __shfl(l_run, 4 * g + i, 64);
 #pragma unroll
 	for (int i = 0; i < 4; i++) {
 		const int qo = q0w + 4 * g + i;
 		if (qo < S) {
 			float *op = o + (size_t)qo * ldo + head * HD + c;
 #pragma unroll
-			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] / lr[i];
+			for (int dt = 0; dt < HD / 16; dt++) op[16 * dt] = oacc[dt][i] * lr[i];
 		}
 	}
 }
@@ -1234,12 +1234,13 @@ __global__ __launch_bounds__(512) void attn_prefill_wide_kernel(float *o, const 
 		return;
 	}
 	if (qpos < S) {
+		const float l_inv = 1.0f / l_run;  // one division per query row, then multiplications
 		float *op = o + (size_t)qpos * ldo + head * HD + 128 * dh + 4 * h;
 #pragma unroll
 		for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
 			for (int j = 0; j < 4; j++)
-				*reinterpret_cast<f32x4 *>(op + 32 * dt + 8 * j) = f32x4{oacc[dt][4 * j] / l_run, oacc[dt][4 * j + 1] / l_run, oacc[dt][4 * j + 2] / l_run, oacc[dt][4 * j + 3] / l_run};
+				*reinterpret_cast<f32x4 *>(op + 32 * dt + 8 * j) = f32x4{oacc[dt][4 * j] * l_inv, oacc[dt][4 * j + 1] * l_inv, oacc[dt][4 * j + 2] * l_inv, oacc[dt][4 * j + 3] * l_inv};
 	}
 }
 
@@ -1262,7 +1263,7 @@ __global__ __launch_bounds__(PNT) void attn_prefill_merge_kernel(float *o, int S
 		const f32x4 x = *reinterpret_cast<const f32x4 *>(part_o + row * HD + 4 * lane);
 		acc += x * wgt;
 	}
-	const f32x4 res = acc / L;
+	const f32x4 res = acc * (1.0f / L);
 	*reinterpret_cast<f32x4 *>(o + (size_t)qpos * ldo + head * HD + 4 * lane) = res;
 }
 
@@ -1300,8 +1301,9 @@ __global__ __launch_bounds__(PNT) void attn_prefill_finish_kernel(const float *o
 			a += *reinterpret_cast<const f32x4 *>(part_o + r * HD + d0) * wgt;
 			b += *reinterpret_cast<const f32x4 *>(part_o + r * HD + d0 + 4) * wgt;
 		}
-		a = a / L;
-		b = b / L;
+		const float Linv = 1.0f / L;
+		a = a * Linv;
+		b = b * Linv;
 #pragma unroll
 		for (int e = 0; e < 4; e++) {
 			v[e] = a[e];

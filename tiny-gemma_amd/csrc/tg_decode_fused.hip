@@ -189,6 +189,7 @@ __global__ __launch_bounds__(NT) void decode_fused_kernel(const TgFused f) {
 			ad.part_ml = xl + f.off_pml;
 			ad.n_head = 4;
 			ad.nblocks = 0;
+			ad.host_cur = -1;
 			const int nb = layer_nb(Ld.max_pos, Ld.is_sw);
 			if (!fused_wait(f.sync, 0, f.all_base + (unsigned)(4 * l + 1) * (unsigned)ng, xcd, f.max_spins, &s_dead)) return;
 			stamp(l, 16);

@@ -61,8 +61,12 @@ __device__ __forceinline__ float b2f(int d, int j) {  // signed byte j of d -> f
 }
 
 // ops.hpp:41-51: truncating index, below the table -> 0, above -> identity
+// A step that is a power of two (the table of the command line: 8 / 1024) has an exact reciprocal: the product equals the
+// quotient bit for bit and saves the IEEE division.
 __device__ __forceinline__ float gelu_lut(float x, const float *lut, float gmin, float geps, int size) {
-	int idx = (int)((x - gmin) / geps);
+	const bool pow2 = (__float_as_uint(geps) & 0x007fffffu) == 0u && geps > 1e-30f && geps < 1e30f;
+	const float ginv = __uint_as_float((254u << 23) - __float_as_uint(geps));  // 2^-e for geps = 2^e
+	int idx = pow2 ? (int)((x - gmin) * ginv) : (int)((x - gmin) / geps);
 	if (idx < 0) return 0.0f;
 	if (idx >= size) return x;
 	return lut[idx];
@@ -201,11 +205,11 @@ __device__ __forceinline__ void attn_merge_prologue(float *xs, float (*wgt)[TG_A
 		const bool ok = b < nb;
 		static_assert(TG_ATTN_MERGE_MAX == 16, "one row of 16 lanes per head");
 		const float M = tg_row16_max(m);
-		const float e = ok ? expf(m - M) : 0.0f;
+		const float e = ok ? __builtin_amdgcn_exp2f((m - M) * 1.44269504088896341f) : 0.0f;  // as the attention kernel's weights
 		// __fmul_rn: the product must be rounded before the reduction; contracted into the first add
 		// (fma(l, e, partner)) the two lanes of a pair would no longer hold the same sum
 		const float L = tg_row16_sum(__fmul_rn(l, e));
-		wgt[h][b] = e / L;
+		wgt[h][b] = e * __builtin_amdgcn_rcpf(L);  // v_rcp_f32 (1 ulp) instead of an IEEE division in front of the product
 	}
 	__syncthreads();
 	{

@@ -140,6 +140,7 @@ struct TgAttnDecode {
 	const int *pos;          // device counters: pos[0] = position_ptr, pos[1]/pos[2] = buffer_ptr of local/global layers
 	int bp_index;            // 1 (local layer) or 2 (global layer)
 	int host_pos, host_bp;   // the same counters as launch arguments (saves a dependent load), or -1 to read the device ones
+	int host_cur;            // host_bp % max_pos when the host knows it (then nblocks is exactly the workgroups the keys need), else -1
 	int chunk;               // keys per workgroup
 	float *part_acc;         // [nblocks][n_head][hd]
 	float *part_ml;          // [nblocks][n_head][2]

@@ -111,7 +111,7 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 		}
 	ss = tg_wave_sum(ss);
 	if (resid != nullptr) {
-		const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
+		const float irms = __builtin_amdgcn_rsqf(ss * (1.0f / (float)dim) + eps);  // v_rsq_f32, as the decode kernels
 		float s2 = 0.0f;
 #pragma unroll
 		for (int r = 0; r < ROUNDS; r++)
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(RNT) void norm_rows_kernel(float *out, const float 
 		ss = tg_wave_sum(s2);
 	}
 	if (out == nullptr && apack == nullptr) return;
-	const float irms = 1.0f / sqrtf(ss / (float)dim + eps);
+	const float irms = __builtin_amdgcn_rsqf(ss * (1.0f / (float)dim) + eps);
 	float amax = 0.0f;
 #pragma unroll
 	for (int r = 0; r < ROUNDS; r++)
