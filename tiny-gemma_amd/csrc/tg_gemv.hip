@@ -50,7 +50,8 @@ __device__ __forceinline__ void gemv_body(const TgGemv &g_in) {
 	const int KL = NT >> lcs;                          // lanes along K
 	const int kpos = tid >> lcs;
 	const int kgs = g.K >> 2;
-	const int nit = (kgs + KL - 1) / KL;  // steps; one step = the 256 lanes reading 4 KiB of the slab
+	static_assert(NT == 256, "KL = 2^(8 - lcs)");
+	const int nit = (kgs + KL - 1) >> (8 - lcs);  // steps (KL is a power of two: a shift, not a division in front of the first loads); one step = the 256 lanes reading 4 KiB of the slab
 
 	// The tile slab and (for the PLAIN prologue) the input vector are read through buffer
 	// descriptors: the per-step address is a scalar offset, so addressing costs no vector
