@@ -68,7 +68,7 @@ __global__ __launch_bounds__(ANT) void attn_merge_kernel(const TgAttnDecode a, f
 		const float m = ok ? a.part_ml[((size_t)(b_lo + lane) * NH + h) * 2] : -INFINITY;
 		const float l = ok ? a.part_ml[((size_t)(b_lo + lane) * NH + h) * 2 + 1] : 0.0f;
 		const float M = wmax(m);
-		const float e = ok ? expf(m - M) : 0.0f;
+		const float e = ok ? attn_exp(m - M) : 0.0f;  // as the attention kernel's own weights
 		const float L = wsum(l * e);
 		wg[lane] = e;
 		if (lane == 0) {
