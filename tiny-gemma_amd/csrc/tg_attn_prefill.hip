@@ -28,6 +28,8 @@
 #include "tg_internal.h"
 
 #include <algorithm>
+#include <functional>
+#include <queue>
 #include <type_traits>
 #include <utility>
 #include <vector>
@@ -1373,32 +1375,82 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 	// SIMD, nothing overlaps), so the chains are cut as short as the number of compute units allows: the smallest
 	// chunk that still gives at most one item per unit.  Local layers of long prompts are balanced as they are.
 	int chunk = window < 0 ? (int)std::max<long>(16, total / ((long)n_cu * 8)) : longest;
+	bool one_round = false;
 	for (int c = 1; c < chunk; c++) {
 		long n = 0;
 		for (int qt = 0; qt < nq; qt++) n += (end_tile(qt) - first_tile(qt) + c - 1) / c;
 		if (n <= n_cu) {
 			chunk = c;
+			one_round = true;
 			break;
 		}
+	}
+	// Causal layers whose items take several rounds: the chunk length decides how the rounds end.  With 16 key tiles a
+	// layer of 4096 tokens has 527 items for 256 compute units, and the 15 that start last, when the first units have
+	// done their two, add 20 % (148-154 us measured, 151 by the model below; 17 key tiles give 492 items and 124).
+	// The lists of the candidate lengths are played through on the host: an item costs its key tiles plus 4 (start-up
+	// until the first image is in LDS, 7 us, and storing its partial result, 5 us, against 2.95 us per key tile, all
+	// measured inside the kernel), the units take the items in list order.  Built once per prompt length.
+	if (window < 0 && !one_round) {
+		auto lengths = [&](int c, std::vector<int> &len) {
+			len.clear();
+			for (int qt = 0; qt < nq; qt++) {
+				const int nt = end_tile(qt) - first_tile(qt);
+				int nc = (nt + c - 1) / c;
+				if (nc > 1 && nt - (nc - 1) * c < (c + 1) / 2) nc--;
+				for (int ch = 0; ch < nc; ch++) len.push_back(ch + 1 == nc ? nt - ch * c : c);
+			}
+			std::sort(len.begin(), len.end(), std::greater<int>());
+		};
+		auto span = [&](const std::vector<int> &len) {
+			std::priority_queue<long, std::vector<long>, std::greater<long>> free_at;
+			for (int i = 0; i < n_cu; i++) free_at.push(0);
+			long end = 0;
+			for (int l : len) {
+				const long t = free_at.top() + 4 + l;
+				free_at.pop();
+				free_at.push(t);
+				end = std::max(end, t);
+			}
+			return end + (long)len.size() / 100;  // the finishing launch reads every partial result
+		};
+		std::vector<int> len;
+		long best = -1;
+		int best_c = chunk;
+		const int lo = std::max(6, chunk / 2), hi = std::min(longest, 3 * chunk), step = std::max(1, chunk / 16);
+		for (int c = lo; c <= hi; c += step) {
+			lengths(c, len);
+			const long sp = span(len);
+			if (best < 0 || sp < best) {
+				best = sp;
+				best_c = c;
+			}
+		}
+		chunk = best_c;
 	}
 	items.clear();
 	split.clear();
 	nslots = 0;
 	// Chunk boundaries are the same for every query tile (multiples of `chunk` key tiles, counted from the query tile's
 	// first key tile for local layers, whose windows all start differently): the workgroups that run next to each
-	// other then walk the same keys at the same time and find each other's K/V tiles in their XCD's L2.  A last chunk
-	// of less than half a chunk is merged into the one before it.
+	// other then walk the same keys at the same time and find each other's K/V tiles in their XCD's L2.  Causal layers: a
+	// last chunk of less than half a chunk is merged into the one before it.
 	for (int qt = 0; qt < nq; qt++) {
 		const int t0 = first_tile(qt), nt = end_tile(qt) - t0;
 		int nc = (nt + chunk - 1) / chunk;
-		if (nc > 1 && nt - (nc - 1) * chunk < (chunk + 1) / 2) nc--;
+		// Local layers have at most one item per compute unit, so the longest item is the launch: a short last chunk is
+		// evened out with the others instead (9 + 4 key tiles -> 7 + 6; merged into 13, such items took 45 us next to
+		// 36 us for the 9-tile items of all the later query tiles).
+		const bool even = window >= 0;
+		if (!even && nc > 1 && nt - (nc - 1) * chunk < (chunk + 1) / 2) nc--;
+		const int each = even ? (nt + nc - 1) / nc : chunk;
 		if (nc == 1) {
 			items.push_back(int4{qt, t0, t0 + nt, -1});
 			continue;
 		}
 		split.push_back(int4{qt, nslots, nc, 0});
 		for (int ch = 0; ch < nc; ch++) {
-			const int tb = t0 + ch * chunk, te = ch + 1 == nc ? t0 + nt : tb + chunk;
+			const int tb = t0 + ch * each, te = ch + 1 == nc ? t0 + nt : tb + each;
 			items.push_back(int4{qt, tb, te, nslots++});
 		}
 	}
