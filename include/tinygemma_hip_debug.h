@@ -69,7 +69,7 @@ int tg_set_prefetch_blocks(int n);
  * the up|gate matrix, o the down matrix, up|gate the next layer's q|k|v.  1: an alternative kept for measurement
  * (q|k|v touches o and up|gate, attention touches down). */
 int tg_set_prefetch_plan(int plan);
-/* tuning knob: decode attention gives a workgroup at most this many keys (multiple of 16 in 32..256, default 48) while 16
+/* tuning knob: decode attention gives a workgroup at most this many keys (multiple of 16 in 32..256, default 64) while 16
  * workgroups cover the context; longer contexts use up to 1024 workgroups of 32 keys and one extra merge launch. */
 int tg_set_attn_merge_chunk(int keys);
 /* Kernel classes of one decode step, in launch order per layer; the head runs once per step. */

@@ -303,10 +303,10 @@ def test_chained_picks_equal_a_finishing_launch_per_step(tg, oracle, weight_imag
     assert np.array_equal(taps_a, taps_b) and pos_a == pos_b == prompt.size + 33 and ptr_a == ptr_b
 
 
-@pytest.mark.parametrize("n_prompt", [1000, 4100])
+@pytest.mark.parametrize("n_prompt", [1100, 4100])
 def test_long_context_merge_path(tg, oracle, weight_images, tables, n_prompt):
-    """More than 768 keys on a global layer: 32-key workgroups plus the merge launch, which folds groups of 64
-    partials (1000 keys: one partly filled group; 4100 keys: two full groups and a group of one)."""
+    """More than 1024 keys on a global layer: 32-key workgroups plus the merge launch, which folds groups of 64
+    partials (1100 keys: one partly filled group; 4100 keys: two full groups and a group of one)."""
     cfg_o = gi.oracle_config("270m", 2)
     cfg_o.pattern = 2  # layer 0 local, layer 1 global
     image = oracle.generate_weights(cfg_o, 21)

@@ -39,7 +39,7 @@ hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
 int g_n_cu = 256;
 bool g_gemm_split = true;       // prefill: products that would leave most compute units idle run in 2 or 4 parts of K
-int g_attn_merge_chunk = 48;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
+int g_attn_merge_chunk = 64;  // decode attention: past this many keys per workgroup, use more workgroups and a merge launch
 bool g_chain_picks = true;  // inside a batch of greedy decode steps the next step's first launch finishes the previous pick
 bool g_keep_taps = false;  // prefill keeps a copy of the residual stream after every block (parity checks)
 // Decode: all layers of a step in one launch of resident workgroups (tg_decode_fused.hip) instead of 5 launches per layer.
@@ -1662,7 +1662,7 @@ int tg_reset_knobs() {
 	g_gemm_split = true;
 	g_gemm_lds = 2;
 	g_gemm_lds_ksplit = 1;
-	g_attn_merge_chunk = 48;
+	g_attn_merge_chunk = 64;
 	g_attn_prefill_split = 1;
 	g_attn_prefill_planes = 1;
 	g_attn_prefill_f16 = 1;
