@@ -29,7 +29,9 @@
 
 #include <algorithm>
 #include <functional>
+#include <map>
 #include <queue>
+#include <tuple>
 #include <type_traits>
 #include <utility>
 #include <vector>
@@ -1385,48 +1387,72 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 			break;
 		}
 	}
-	// Causal layers whose items take several rounds: the chunk length decides how the rounds end.  With 16 key tiles a
-	// layer of 4096 tokens has 527 items for 256 compute units, and the 15 that start last, when the first units have
-	// done their two, add 20 % (148-154 us measured, 151 by the model below; 17 key tiles give 492 items and 124).
-	// The lists of the candidate lengths are played through on the host: an item costs its key tiles plus 4 (start-up
-	// until the first image is in LDS, 7 us, and storing its partial result, 5 us, against 2.95 us per key tile, all
-	// measured inside the kernel), the units take the items in list order.  Built once per prompt length.
+	// Causal layers whose items take several rounds: the chunk length decides how many items there are and how the
+	// rounds end.  With 16 key tiles a layer of 4096 tokens has 527 items for 256 compute units, and the 15 that start
+	// last, when the first units have done their two, add 20 % (148-154 us measured, 151 by the model below; 17 key
+	// tiles give 492 items and 124 us); at 8192 tokens and more, 8 items per unit pay the start-up of an item more
+	// often than the balance needs.  Candidates: the rule above, and the shortest chunks that give at most 2, 3 and 4
+	// items per unit.  Their lists are played through on the host: an item costs its key tiles plus 4 (start-up until
+	// the first image is in LDS, 7 us, and storing its partial result, 5 us, against 2.95 us per key tile, all measured
+	// inside the kernel), the units take the items in list order.  0.05-0.6 ms on the host for 4096-32768 tokens, once
+	// per prompt length and process.
 	if (window < 0 && !one_round) {
-		auto lengths = [&](int c, std::vector<int> &len) {
-			len.clear();
-			for (int qt = 0; qt < nq; qt++) {
-				const int nt = end_tile(qt) - first_tile(qt);
-				int nc = (nt + c - 1) / c;
-				if (nc > 1 && nt - (nc - 1) * c < (c + 1) / 2) nc--;
-				for (int ch = 0; ch < nc; ch++) len.push_back(ch + 1 == nc ? nt - ch * c : c);
+		static std::map<std::tuple<int, int, int>, int> chosen;
+		const auto key = std::make_tuple(S, n_cu, tq);
+		const auto hit = chosen.find(key);
+		if (hit != chosen.end()) {
+			chunk = hit->second;
+		} else {
+			auto chunks_of = [&](int nt, int c) {
+				const int nc = (nt + c - 1) / c;
+				return (nc > 1 && nt - (nc - 1) * c < (c + 1) / 2) ? nc - 1 : nc;
+			};
+			auto n_items = [&](int c) {
+				long n = 0;
+				for (int qt = 0; qt < nq; qt++) n += chunks_of(end_tile(qt) - first_tile(qt), c);
+				return n;
+			};
+			std::vector<int> count((size_t)longest + 1);  // items by length
+			auto span = [&](int c) {
+				std::fill(count.begin(), count.end(), 0);
+				long n = 0;
+				for (int qt = 0; qt < nq; qt++) {
+					const int nt = end_tile(qt) - first_tile(qt), nc = chunks_of(nt, c);
+					count[(size_t)c] += nc - 1;
+					count[(size_t)(nt - (nc - 1) * c)]++;
+					n += nc;
+				}
+				std::priority_queue<long, std::vector<long>, std::greater<long>> free_at;
+				for (int i = 0; i < n_cu; i++) free_at.push(0);
+				long end = 0;
+				for (int l = longest; l >= 1; l--)
+					for (int k = 0; k < count[(size_t)l]; k++) {
+						const long t = free_at.top() + 4 + l;
+						free_at.pop();
+						free_at.push(t);
+						end = std::max(end, t);
+					}
+				return end + n / 100;  // the finishing launch reads every partial result
+			};
+			long best = span(chunk);
+			int best_c = chunk;
+			for (int per_unit = 2; per_unit <= 4; per_unit++) {
+				int lo = 6, hi = longest;  // the shortest chunk with at most per_unit items per unit (the count falls with the length)
+				while (lo < hi) {
+					const int mid = (lo + hi) / 2;
+					if (n_items(mid) <= (long)per_unit * n_cu) hi = mid;
+					else lo = mid + 1;
+				}
+				if (lo == best_c) continue;
+				const long sp = span(lo);
+				if (sp < best) {
+					best = sp;
+					best_c = lo;
+				}
 			}
-			std::sort(len.begin(), len.end(), std::greater<int>());
-		};
-		auto span = [&](const std::vector<int> &len) {
-			std::priority_queue<long, std::vector<long>, std::greater<long>> free_at;
-			for (int i = 0; i < n_cu; i++) free_at.push(0);
-			long end = 0;
-			for (int l : len) {
-				const long t = free_at.top() + 4 + l;
-				free_at.pop();
-				free_at.push(t);
-				end = std::max(end, t);
-			}
-			return end + (long)len.size() / 100;  // the finishing launch reads every partial result
-		};
-		std::vector<int> len;
-		long best = -1;
-		int best_c = chunk;
-		const int lo = std::max(6, chunk / 2), hi = std::min(longest, 3 * chunk), step = std::max(1, chunk / 16);
-		for (int c = lo; c <= hi; c += step) {
-			lengths(c, len);
-			const long sp = span(len);
-			if (best < 0 || sp < best) {
-				best = sp;
-				best_c = c;
-			}
+			chunk = best_c;
+			chosen[key] = chunk;
 		}
-		chunk = best_c;
 	}
 	items.clear();
 	split.clear();
