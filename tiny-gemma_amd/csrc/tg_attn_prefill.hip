@@ -1372,7 +1372,8 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 		total += end_tile(qt) - first_tile(qt);
 		longest = std::max(longest, end_tile(qt) - first_tile(qt));
 	}
-	// Long prompts (causal): about 8 items per compute unit, and never chunks below 16 key tiles (512 keys).
+	// Long prompts (causal): to begin with about 8 items per compute unit, and never chunks below 16 key tiles (512 keys);
+	// the play-through below may choose another length.
 	// Prompts with fewer query tiles than compute units: a workgroup's time is its chain of key tiles (one wave per
 	// SIMD, nothing overlaps), so the chains are cut as short as the number of compute units allows: the smallest
 	// chunk that still gives at most one item per unit.  Local layers of long prompts are balanced as they are.
