@@ -174,7 +174,9 @@ def main():
     from tiny_gemma_amd import weights as tgw
 
     dev = tg.init(0)
-    if tg.lib().tg_set_graphs(1 if args.graphs else 0) != 0:
+    # the headline model's steps: stream launches unless --graphs; the library's own choice (-1) would be the same for the
+    # 1B shape and updated-graph replay for the 270m shape (its section below runs both)
+    if tg.lib().tg_set_graphs(1 if args.graphs else (0 if args.model == "1B" else -1)) != 0:
         print("bench.py: " + tg.lib().tg_last_error().decode(), file=sys.stderr)
         sys.exit(2)
     if args.prefetch_blocks is not None:
@@ -255,6 +257,7 @@ def main():
     for b in range(n_blocks):
         sess.decode_enqueue(sizes[b])
         ev.record(marks[b + 1], stream)
+    host_enqueue = time.perf_counter() - t0  # the host has issued every launch: below `wall` the device sets the pace
     tg.synchronize()
     wall = time.perf_counter() - t0
     gpu_ms = ev.elapsed_ms(marks[0], marks[-1])
@@ -557,14 +560,27 @@ def main():
             tp = time.perf_counter() - t0
             ss.decode_enqueue(16)
             tg.synchronize()
+            time.sleep(settle_ms * 1e-3)
             t0 = time.perf_counter()
             ss.decode_enqueue(n_steps)
+            te = time.perf_counter() - t0
             tg.synchronize()
             td = time.perf_counter() - t0
+            # host_enqueue_ms_per_step next to ms_per_step tells which side set the pace: this shape's step is 91 launches
+            # of 3.6 us on the device, and the host issues a launch in 2.5 us or in 4.2 us depending on the core the
+            # thread happens to run on and on what else that core is doing (2,600 or 3,070 tok/s)
             return {"prompt_tokens": n_prompt_s, "prefill_ms": 1e3 * tp, "prefill_tok_s": n_prompt_s / tp, "decode_steps": n_steps,
-                    "decode_tok_s": n_steps / td, "ms_per_step": 1e3 * td / n_steps}
+                    "decode_tok_s": n_steps / td, "ms_per_step": 1e3 * td / n_steps, "host_enqueue_ms_per_step": 1e3 * te / n_steps}
 
+        # The library's own choice for this shape (tg_set_graphs(-1)): replay of a captured step whose position-dependent
+        # nodes are updated before every replay, one graph launch and 36 node updates per step on the host instead of 91
+        # kernel launches.  Beside it the same 256 steps as stream launches, which follow the host wherever the launching
+        # thread sits on a slow core (`host_enqueue_ms_per_step` = `ms_per_step`).
+        L.tg_set_graphs(-1)
         short, long_ctx = run(64, 256), run(16384, 256)
+        short["launch"] = long_ctx["launch"] = "updated hipGraph replay (library default for this shape)"
+        L.tg_set_graphs(0)
+        short["stream_launches"] = {k: v for k, v in run(64, 256).items() if k in ("decode_tok_s", "ms_per_step", "host_enqueue_ms_per_step")}
         short["weight_stream_GBps"] = s_bytes * short["decode_tok_s"] / 1e9
         short["frac_of_hbm_roofline"] = short["weight_stream_GBps"] / HBM_PEAK_GBS
         small = {"shape": "gemma-3-270m", "weight_bytes_per_token": s_bytes, "prompt64_decode256": short,
@@ -586,6 +602,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "settle_ms": settle_ms,
+        "host_enqueue_ms_per_step": 1e3 * host_enqueue / args.steps,
         "ms_per_step": 1e3 * wall / args.steps,
         "higher_is_better": True,
         "scaling": "weak",

@@ -16,7 +16,11 @@ extern "C" {
 /* device-to-device streaming copy kernel (bytes % 16 == 0), asynchronous: the known-size kernel
  * that hardware byte counters are calibrated against */
 int tg_dev_copy(void *dst_dev, const void *src_dev, size_t bytes);
-/* 1: tg_decode_enqueue replays captured HIP graphs of a decode step; 0 (default): plain stream launches.
+/* How tg_decode_enqueue issues greedy decode steps.  0 (default): plain stream launches.  1: replay of a captured step
+ * whose kernels read the position from device memory and launch the largest grids their geometry can need.  2: replay
+ * of a captured step of the stream path's own launches; the nodes that depend on the position (attention, its merge
+ * launch, the output projection) get new parameters before every replay: one graph launch and 2-3 node updates per
+ * layer on the host instead of 5-6 kernel launches.  Other values: TG_ERR_BAD_ARG.
  * Refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
  * replayed graphs ended the process.  Captured graphs are dropped whenever a tuning knob changes. */
 int tg_set_graphs(int enable);

@@ -256,10 +256,12 @@ def test_full_1b_greedy_ids(tg, oracle, golden, weight_images, tables):
 
 
 def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
-    """HIP-graph replay must give the same bits as plain launches, on every replay."""
+    """HIP-graph replay must give the same bits as plain launches, on every replay: mode 1 (a captured step that reads
+    its position from device memory) and mode 2 (a captured step of the stream path's own launches whose attention,
+    merge and output-projection nodes get the position's parameters before every replay)."""
     model, sess, osess, prompt = build(tg, oracle, weight_images, tables, "small6")
     results = []
-    for graphs in (0, 1, 1):
+    for graphs in (0, 1, 1, 2, 2):
         tg.lib().tg_set_graphs(graphs)
         sess.reset()
         sess.prefill(prompt, want_logits=False)
@@ -269,11 +271,44 @@ def test_graph_replay_equals_stream_launches(tg, oracle, weight_images, tables):
             tg.synchronize()
             chunks.append(sess.taps(rows=1).copy())
         results.append((sess.read_ids(16).copy(), chunks))
-    tg.lib().tg_set_graphs(0)
+    tg.lib().tg_set_graphs(-1)
     for ids, chunks in results[1:]:
         assert np.array_equal(ids, results[0][0])
         for a, b in zip(chunks, results[0][1]):
             assert np.array_equal(a, b)
+
+
+def test_updated_graph_replay_across_attention_geometries(tg, oracle):
+    """Graph replay with node updates over 80 steps that start at 990 keys: the global layer's chunk grows with the
+    context (a parameter of its nodes, not another graph) and at 1025 keys its attention gets a merge launch (another
+    graph).  Ids, residual stream and cache rows as with plain launches, bit for bit; sampled steps (always plain
+    launches) and a stepwise call in between."""
+    cfg = tg.named_config("270m", 6)   # layer 5 is a global one
+    model = tg.Transformer(cfg)
+    model.read_weights_mem(oracle.generate_weights(gi.oracle_config("270m", 6), 43))
+    sess = model.session()
+    prompt = gi.prompt_ids(53, 990)
+    L = tg.lib()
+    out = []
+    try:
+        for graphs in (0, 2):
+            tg.check(L.tg_set_graphs(graphs))
+            sess.reset()
+            sess.prefill(prompt, want_logits=False)
+            for n in (1, 30, 7):
+                sess.decode_enqueue(n)
+            sess.decode_enqueue_sampled(3, 0.05, 1.0, np.array([0.3, 0.6, 0.9], np.float32))
+            tok, _ = sess.decode(int(sess.read_ids(64)[-1]), want_logits=False)
+            sess.decode_enqueue(38)
+            tg.synchronize()
+            out.append((sess.read_ids(128).copy(), sess.taps(rows=1).copy(), sess.position, [sess.kv(l) for l in (0, 5)]))
+    finally:
+        tg.check(L.tg_set_graphs(-1))
+    (ids_a, taps_a, pos_a, kv_a), (ids_b, taps_b, pos_b, kv_b) = out
+    assert pos_a == pos_b == 990 + 80 and ids_a.size == ids_b.size and np.array_equal(ids_a, ids_b)
+    assert np.array_equal(taps_a, taps_b)
+    for (k0, v0, p0, b0), (k1, v1, p1, b1) in zip(kv_a, kv_b):
+        assert (p0, b0) == (p1, b1) and np.array_equal(k0, k1) and np.array_equal(v0, v1)
 
 
 def test_chained_picks_equal_a_finishing_launch_per_step(tg, oracle, weight_images, tables):

@@ -33,7 +33,10 @@ int g_prefetch_blocks = 128;   // extra workgroups per launch that prefetch the 
 // once: the LM head's 2048 tiles each get their own (47 us per launch streamed from HBM, 50-54 us with 1024 that
 // walk two tiles each).
 int g_gemv_max_blocks = 2048;
-bool g_use_graphs = false;  // measured: no gain (the decode step is bound by GPU-side dispatch, not by host launches)
+// How greedy decode steps are issued.  0: stream launches; 1: replay of a captured step that reads its position from device
+// memory; 2: replay with the position-dependent nodes re-described before every replay (the kernels and grids of the
+// stream launches); -1 (default): 2 for models whose step is bound by the host's launch rate, else 0 (decode_graph_mode).
+int g_use_graphs = -1;
 int g_device = -1;
 hipStream_t g_stream = nullptr;
 char g_devname[256] = "";
@@ -312,6 +315,14 @@ struct tg_session {
 	float *taps = nullptr;    // prefill taps [(2L+1)][rows][hidden] (kept only for short prompts)
 	int tap_rows = 0;
 	std::map<uint64_t, hipGraphExec_t> graphs;  // captured decode steps, keyed by the attention launch geometry
+	// graphs of mode 2, keyed by which layer kinds have a merge launch: the template graph stays alive (its nodes name
+	// what is updated in the executable graph); attn / merge / oproj: the nodes by layer (merge: null where there is none)
+	struct PatchedGraph {
+		hipGraph_t graph = nullptr;
+		hipGraphExec_t exec = nullptr;
+		std::vector<hipGraphNode_t> attn, merge, oproj;
+	};
+	std::map<uint64_t, PatchedGraph> pgraphs;
 	// min-p sampling (allocated on first use): scratch of the three sampler launches and the caller's uniform draws
 	float *probs = nullptr, *seg = nullptr, *bsum = nullptr, *bmax = nullptr, *randf = nullptr;
 	int randf_cap = 0;
@@ -860,6 +871,11 @@ void tg_session_destroy(tg_session *s) {
 	(void)hipStreamSynchronize(g_stream);
 	for (auto &kv : s->graphs) (void)hipGraphExecDestroy(kv.second);
 	s->graphs.clear();
+	for (auto &kv : s->pgraphs) {
+		if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+		if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);
+	}
+	s->pgraphs.clear();
 	void *ps[] = {s->cos_g, s->sin_g, s->cos_l, s->sin_l, s->lut, s->xr, s->qkv, s->attn_out, s->o_out, s->hbuf, s->d_out,
 	              s->logits, s->part_acc, s->part_ml, s->merged_acc, s->merged_ml, s->blk_val, s->blk_idx, s->ctr,
 	              s->tok_log, s->pf_ws, s->probs, s->seg, s->bsum, s->bmax, s->randf, s->zeros, s->blk_x, s->blk_y, s->fused_layers,
@@ -1265,7 +1281,7 @@ static void launch_attn(tg_session *s, const AttnGeom &ag) {
 	if (ag.needs_merge) tg_launch_attn_merge(ag.a, ag.nblk, s->merged_acc, s->merged_ml, g_stream);
 }
 // merge of the attention partials + O projection (modules.hpp:161-164)
-static void launch_oproj(tg_session *s, int l, const AttnGeom &ag) {
+static TgGemv oproj_gemv(tg_session *s, int l, const AttnGeom &ag) {
 	const LayerDev &Ld = s->m->L[(size_t)l];
 	TgGemv g = gemv_base(Ld.o);
 	g.pos = s->ctr;
@@ -1276,8 +1292,9 @@ static void launch_oproj(tg_session *s, int l, const AttnGeom &ag) {
 	g.part_ml = ag.needs_merge ? s->merged_ml : s->part_ml;
 	g.y = s->o_out;
 	if (g_prefetch_plan == 0) g.pf = prefetch_of(Ld.d);
-	tg_launch_gemv(g, TG_ROLE_OPROJ, g_stream);
+	return g;
 }
+static void launch_oproj(tg_session *s, int l, const AttnGeom &ag) { tg_launch_gemv(oproj_gemv(s, l, ag), TG_ROLE_OPROJ, g_stream); }
 // post-norm + residual of the attention block, pre-norm, up|gate, gelu(gate)*up (modules.hpp:166-168, 205-215)
 static void launch_upgate(tg_session *s, int l, const float *pend, const float *x, float *xr_out) {
 	tg_model *m = s->m;
@@ -1428,21 +1445,175 @@ static uint64_t decode_graph_key(const tg_session *s) {
 static void session_drop_graphs(tg_session *s) {
 	for (auto &kv : s->graphs) (void)hipGraphExecDestroy(kv.second);
 	s->graphs.clear();
+	for (auto &kv : s->pgraphs) {
+		if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+		if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);
+	}
+	s->pgraphs.clear();
+}
+
+// ---- graph replay, mode 2 ----------------------------------------------------------------------------------------
+// A decode step captured with the launches of the stream path (position known on the host: exact grids, nothing read
+// from the device-side counters in front of a kernel's loads).  Three launches per layer depend on the position: the
+// attention (grid, chunk, ring slot, RoPE row), its merge launch where there is one, and the output projection (number
+// of partials).  Their nodes are looked up once in the captured graph and given new parameters before every replay;
+// everything else in a step is position independent.  The host then issues one graph launch and 2-3 node updates per
+// layer instead of 5-6 kernel launches: a decode step of the 270m shape, 91 launches of 3.6 us on the device, is bound
+// by the host's launch rate whenever the launching thread sits on a slow core (2.5 or 4.2 us per launch: 3,070 or
+// 2,500-2,600 tok/s from process to process).
+static uint64_t patched_graph_key(const tg_session *s, bool chained) {
+	const tg_config &c = s->m->cfg;
+	bool ml = false, mg = false;
+	(void)attn_chunk_for(std::min(s->pos + 1, c.n_pos_local), &ml);
+	(void)attn_chunk_for(std::min(s->pos + 1, c.n_pos), &mg);
+	return (uint64_t)ml | ((uint64_t)mg << 1) | ((uint64_t)chained << 2);
+}
+
+// chained: the step's first launch finishes the previous step's greedy pick and its own pick stays pending (the caller
+// has a pick pending on entry and flushes after its last step); else the step ends with the finishing launch.
+static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bool chained) {
+	const int L = s->m->cfg.n_layers;
+	TG_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
+	const int rc = enqueue_decode_step(s, nullptr, false, nullptr, chained);  // advances the host mirrors once
+	const hipError_t e = hipStreamEndCapture(g_stream, &pg->graph);
+	if (rc != TG_OK) return rc;
+	if (e != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
+	size_t n = 0;
+	TG_HIP(hipGraphGetNodes(pg->graph, nullptr, &n));
+	std::vector<hipGraphNode_t> nodes(n);
+	TG_HIP(hipGraphGetNodes(pg->graph, nodes.data(), &n));
+	pg->attn.assign((size_t)L, nullptr);
+	pg->merge.assign((size_t)L, nullptr);
+	pg->oproj.assign((size_t)L, nullptr);
+	for (hipGraphNode_t node : nodes) {
+		hipGraphNodeType type;
+		TG_HIP(hipGraphNodeGetType(node, &type));
+		if (type != hipGraphNodeTypeKernel) continue;
+		hipKernelNodeParams kp;
+		TG_HIP(hipGraphKernelNodeGetParams(node, &kp));
+		const int kind = tg_decode_node_kind(kp.func);
+		if (kind == 0 || kp.kernelParams == nullptr) continue;
+		// which layer: by the cache (attention, merge) or the weights (projection) the node's descriptor names
+		int layer = -1;
+		if (kind == 3) {
+			const TgGemv *g = static_cast<const TgGemv *>(kp.kernelParams[9]);
+			for (int l = 0; l < L; l++)
+				if (g->W == s->m->L[(size_t)l].o.W) layer = l;
+		} else {
+			const TgAttnDecode *a = static_cast<const TgAttnDecode *>(kp.kernelParams[kind == 1 ? 9 : 0]);
+			for (int l = 0; l < L; l++)
+				if (a->kc == s->kc[(size_t)l]) layer = l;
+		}
+		if (layer < 0) return tg_fail(TG_ERR_STATE, "graph replay: a captured node names no layer of this session");
+		std::vector<hipGraphNode_t> &slot = kind == 1 ? pg->attn : (kind == 2 ? pg->merge : pg->oproj);
+		if (slot[(size_t)layer] != nullptr) return tg_fail(TG_ERR_STATE, "graph replay: two captured nodes for one launch");
+		slot[(size_t)layer] = node;
+	}
+	for (int l = 0; l < L; l++)
+		if (pg->attn[(size_t)l] == nullptr || pg->oproj[(size_t)l] == nullptr)
+			return tg_fail(TG_ERR_STATE, "graph replay: the captured step lacks a layer's attention or projection node");
+	const hipError_t e2 = hipGraphInstantiate(&pg->exec, pg->graph, nullptr, nullptr, 0);
+	if (e2 != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e2));
+	return TG_OK;
+}
+
+static int patched_graph_update(tg_session *s, const tg_session::PatchedGraph &pg) {
+	const int L = s->m->cfg.n_layers;
+	TgLaunchDesc d;
+	auto set = [&](hipGraphNode_t node) -> hipError_t {
+		hipKernelNodeParams kp;
+		memset(&kp, 0, sizeof(kp));
+		kp.func = const_cast<void *>(d.func);
+		kp.gridDim = d.grid;
+		kp.blockDim = d.block;
+		kp.sharedMemBytes = 0;
+		kp.kernelParams = d.args;
+		kp.extra = nullptr;
+		return hipGraphExecKernelNodeSetParams(pg.exec, node, &kp);
+	};
+	for (int l = 0; l < L; l++) {
+		const AttnGeom ag = attn_geometry(s, l, false);
+		tg_desc_attn_decode(ag.a, ag.nblk, &d);
+		TG_HIP(set(pg.attn[(size_t)l]));
+		if (ag.needs_merge != (pg.merge[(size_t)l] != nullptr)) return tg_fail(TG_ERR_STATE, "graph replay: the step's launches differ from the captured ones");
+		if (ag.needs_merge) {
+			tg_desc_attn_merge(ag.a, ag.nblk, s->merged_acc, s->merged_ml, &d);
+			TG_HIP(set(pg.merge[(size_t)l]));
+		}
+		tg_desc_gemv(oproj_gemv(s, l, ag), TG_ROLE_OPROJ, &d);
+		TG_HIP(set(pg.oproj[(size_t)l]));
+	}
+	return TG_OK;
+}
+
+static int enqueue_patched_graph_step(tg_session *s, bool chained) {
+	const tg_config &c = s->m->cfg;
+	if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
+	if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
+	const uint64_t key = patched_graph_key(s, chained);
+	auto it = s->pgraphs.find(key);
+	if (it == s->pgraphs.end()) {
+		tg_session::PatchedGraph pg;
+		const int rc = patched_graph_capture(s, &pg, chained);  // the captured step holds this position's parameters
+		if (rc != TG_OK) {
+			if (pg.exec) (void)hipGraphExecDestroy(pg.exec);
+			if (pg.graph) (void)hipGraphDestroy(pg.graph);
+			return rc;
+		}
+		s->pgraphs[key] = pg;
+		TG_HIP(hipGraphLaunch(pg.exec, g_stream));
+		return TG_OK;
+	}
+	if (int rc = patched_graph_update(s, it->second)) return rc;
+	TG_HIP(hipGraphLaunch(it->second.exec, g_stream));
+	s->pos += 1;
+	s->bp_local += 1;
+	s->bp_global += 1;
+	s->steps += 1;
+	return TG_OK;
+}
+
+static bool profiler_attached();
+// The mode a session's greedy steps take.  Left to the library (-1), a model whose decode step streams less than 5 MB of
+// weights per launch replays updated graphs: the device then needs less time per launch (3.6 us for the 270m shape's
+// 3 MB) than a host core that is slow or shared needs to issue one (2.5 us at best, 4.2-4.4 us on other cores of the same
+// machine), and the step would follow the host.  The 1B shape (7.7 MB, 4.6 us per launch) stays ahead of the host either
+// way and keeps its stream launches, which are 0.7 % faster there.  Never graphs under a profiler.
+static int decode_graph_mode(const tg_session *s) {
+	if (g_use_graphs >= 0) return g_use_graphs;
+	if (profiler_attached()) return 0;
+	const tg_config &c = s->m->cfg;
+	const double h = c.hidden_size, qo = (double)c.n_head * c.head_dim, kv = (double)c.n_kv * c.head_dim, f = c.intermediate_size;
+	const double bytes = c.n_layers * (h * (qo + 2 * kv) + qo * h + 3 * h * f) + h * c.n_vocab;
+	return bytes / (5.0 * c.n_layers + 1.0) < 5e6 ? 2 : 0;
 }
 
 int tg_decode_enqueue(tg_session *s, int n_steps) {
 	if (!s || n_steps < 0) return tg_fail(TG_ERR_BAD_ARG, "bad argument");
 	if (int rc = session_usable(s)) return rc;
 	const tg_config &c = s->m->cfg;
-	if (g_use_graphs && s->graph_epoch != g_knob_epoch) {
+	const int graph_mode = decode_graph_mode(s);
+	if (graph_mode && s->graph_epoch != g_knob_epoch) {
 		// the graphs captured so far hold the launch parameters of other knob settings
 		TG_HIP(hipStreamSynchronize(g_stream));
 		session_drop_graphs(s);
 		s->graph_epoch = g_knob_epoch;
 	}
 	for (int i = 0; i < n_steps; i++) {
-		if (!g_use_graphs) {
+		if (!graph_mode || (graph_mode == 2 && g_fused)) {
 			if (int rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks)) {
+				flush_pick(s);
+				return rc;
+			}
+			continue;
+		}
+		if (graph_mode == 2) {
+			// With chained picks the first step of a batch is a plain one (its first launch has no pick to finish); the
+			// steps behind it replay the chained form, whose pick stays pending for the next step or the flush below.
+			int rc;
+			if (g_chain_picks && !s->pick_pending) rc = enqueue_decode_step(s, nullptr, false, nullptr, true);
+			else rc = enqueue_patched_graph_step(s, g_chain_picks);
+			if (rc != TG_OK) {
 				flush_pick(s);
 				return rc;
 			}
@@ -1658,7 +1829,7 @@ int tg_reset_knobs() {
 	g_prefetch_plan = 0;
 	g_prefetch_blocks = 128;
 	g_gemv_max_blocks = 2048;
-	g_use_graphs = false;
+	g_use_graphs = -1;
 	g_gemm_split = true;
 	g_gemm_lds = 2;
 	g_gemm_lds_ksplit = 1;
@@ -1673,9 +1844,11 @@ int tg_reset_knobs() {
 }
 
 int tg_set_graphs(int enable) {
-	if (enable && profiler_attached())
+	if (enable > 0 && profiler_attached())
 		return tg_fail(TG_ERR_STATE, "graph replay is not available under a profiler (a kernel trace of replayed graphs ended the process); use plain launches");
-	g_use_graphs = enable != 0;
+	if (enable < -1 || enable > 2) return tg_fail(TG_ERR_BAD_ARG, "mode: -1, 0, 1 or 2");
+	g_use_graphs = enable;
+	g_knob_epoch++;  // graphs of the other mode are dropped
 	return TG_OK;
 }
 

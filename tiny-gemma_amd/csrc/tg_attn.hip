@@ -124,20 +124,61 @@ __global__ __launch_bounds__(ANT) void qk_norm_rope_rows_kernel(float *q, float 
 
 }  // namespace
 
-void tg_launch_attn_decode(const TgAttnDecode &a_in, int max_blocks, hipStream_t s) {
-	TgAttnDecode a = a_in;
+void tg_desc_attn_decode(const TgAttnDecode &a_in, int max_blocks, TgLaunchDesc *d) {
+	TgAttnDecode &a = d->a;
+	a = a_in;
 	a.nblocks = max_blocks;
 	if (a.pf.ptr == nullptr) a.pf.nblocks = 0;
 	if (a.pf2.ptr == nullptr) a.pf2.nblocks = 0;
-	hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)(max_blocks + a.pf.nblocks + a.pf2.nblocks)), dim3(ANT), 0, s, a.qkv, a.rms_q,
-	                   a.rms_k, a.cos_t, a.sin_t, a.host_pos, a.host_bp, a.nblocks, a.chunk, a);
+	d->func = reinterpret_cast<const void *>(&attn_decode_kernel);
+	d->grid = dim3((unsigned)(max_blocks + a.pf.nblocks + a.pf2.nblocks));
+	d->block = dim3(ANT);
+	// qkv, rms_q, rms_k, cos_t, sin_t, host_pos, host_bp, nblocks, chunk, a
+	d->p[0] = a.qkv;
+	d->p[1] = a.rms_q;
+	d->p[2] = a.rms_k;
+	d->p[3] = a.cos_t;
+	d->p[4] = a.sin_t;
+	d->i[0] = a.host_pos;
+	d->i[1] = a.host_bp;
+	d->i[2] = a.nblocks;
+	d->i[3] = a.chunk;
+	for (int k = 0; k < 5; k++) d->args[k] = &d->p[k];
+	for (int k = 0; k < 4; k++) d->args[5 + k] = &d->i[k];
+	d->args[9] = &d->a;
 }
 
 // nblk: workgroups of the attention launch whose partials are folded
-void tg_launch_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, hipStream_t s) {
+void tg_desc_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, TgLaunchDesc *d) {
 	static_assert(TG_ATTN_FOLD == 64 && TG_ATTN_MAX_BLOCKS == TG_ATTN_FOLD * TG_ATTN_MERGE_MAX, "one partial per lane; the consumer merges the rest");
-	hipLaunchKernelGGL(attn_merge_kernel, dim3(NH, HD / 64, (unsigned)((nblk + TG_ATTN_FOLD - 1) / TG_ATTN_FOLD)), dim3(ANT), 0, s, a,
-	                   merged_acc, merged_ml);
+	d->a = a;
+	d->func = reinterpret_cast<const void *>(&attn_merge_kernel);
+	d->grid = dim3(NH, HD / 64, (unsigned)((nblk + TG_ATTN_FOLD - 1) / TG_ATTN_FOLD));
+	d->block = dim3(ANT);
+	d->p[0] = merged_acc;
+	d->p[1] = merged_ml;
+	d->args[0] = &d->a;
+	d->args[1] = &d->p[0];
+	d->args[2] = &d->p[1];
+}
+
+bool tg_gemv_is_oproj(const void *func);  // tg_gemv.hip
+int tg_decode_node_kind(const void *func) {
+	if (func == reinterpret_cast<const void *>(&attn_decode_kernel)) return 1;
+	if (func == reinterpret_cast<const void *>(&attn_merge_kernel)) return 2;
+	return tg_gemv_is_oproj(func) ? 3 : 0;
+}
+
+void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s) {
+	TgLaunchDesc d;
+	tg_desc_attn_decode(a, max_blocks, &d);
+	tg_launch_desc(d, s);
+}
+
+void tg_launch_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, hipStream_t s) {
+	TgLaunchDesc d;
+	tg_desc_attn_merge(a, nblk, merged_acc, merged_ml, &d);
+	tg_launch_desc(d, s);
 }
 
 void tg_launch_qk_norm_rope_rows(float *q, float *k, const float *v, const float *rms_q, const float *rms_k, const float *cos_t,

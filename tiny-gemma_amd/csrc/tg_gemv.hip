@@ -388,17 +388,23 @@ int tg_gemv_depth(int K, int C) {
 	return best;
 }
 
-void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
+void tg_desc_gemv(const TgGemv &g_in, int role, TgLaunchDesc *d) {
 	// more than max_blocks tiles: workgroups loop over tiles, so the prologue is paid once per workgroup
-	TgGemv g = g_in;
+	TgGemv &g = d->g;
+	g = g_in;
 	g.nmain = (g.max_blocks > 0 && g.ntiles > g.max_blocks) ? g.max_blocks : g.ntiles;
 	if (g.pf.ptr == nullptr) g.pf.nblocks = 0;
 	if (g.pf2.ptr == nullptr) g.pf2.nblocks = 0;
-	dim3 grid((unsigned)(g.nmain + g.pf.nblocks + g.pf2.nblocks)), block(NT);
+	d->grid = dim3((unsigned)(g.nmain + g.pf.nblocks + g.pf2.nblocks));
+	d->block = dim3(NT);
 	// hot arguments in the order with_hot_args expects for the role's prologue
-	const void *a0 = g.pend, *a1 = g.x, *a2 = g.w_post, *a3 = g.w_pre;
-	if (role == TG_ROLE_OPROJ) { a0 = g.part_acc; a1 = g.part_ml; a2 = a3 = nullptr; }
-	if (role == TG_ROLE_QKV_EMBED) { a0 = g.wte; a1 = g.wte_scales; a2 = g.tok; a3 = g.w_pre; }
+	d->p[0] = g.pend;
+	d->p[1] = g.x;
+	d->p[2] = g.w_post;
+	d->p[3] = g.w_pre;
+	if (role == TG_ROLE_OPROJ) { d->p[0] = g.part_acc; d->p[1] = g.part_ml; d->p[2] = d->p[3] = nullptr; }
+	if (role == TG_ROLE_QKV_EMBED) { d->p[0] = g.wte; d->p[1] = g.wte_scales; d->p[2] = g.tok; d->p[3] = g.w_pre; }
+	d->p[4] = g.W;
 	int hot_hidden = g.hidden;
 	if (role == TG_ROLE_OPROJ) {  // the number of attention partials to merge rides in the slot of `hidden`
 		hot_hidden = -1;
@@ -407,31 +413,50 @@ void tg_launch_gemv(const TgGemv &g_in, int role, hipStream_t s) {
 			hot_hidden = (valid + g.attn_chunk - 1) / g.attn_chunk;
 		}
 	}
-#define TG_LAUNCH(KERNEL) hipLaunchKernelGGL(KERNEL, grid, block, 0, s, a0, a1, a2, a3, g.W, hot_hidden, g.K, g.nmain, g.C, g)
-#define TG_LAUNCH_D(KERNEL)                          \
-	switch (depth) {                                 \
-		case 2: TG_LAUNCH(KERNEL<2>); break;         \
-		case 3: TG_LAUNCH(KERNEL<3>); break;         \
-		case 4: TG_LAUNCH(KERNEL<4>); break;         \
-		default: TG_LAUNCH(KERNEL<8>); break;        \
+	d->i[0] = hot_hidden;
+	d->i[1] = g.K;
+	d->i[2] = g.nmain;
+	d->i[3] = g.C;
+	// TG_GEMV_ARGS: a0, a1, a2, a3, W, hidden, K, nmain, aux, g
+	for (int k = 0; k < 5; k++) d->args[k] = &d->p[k];
+	for (int k = 0; k < 4; k++) d->args[5 + k] = &d->i[k];
+	d->args[9] = &d->g;
+#define TG_FUNC(KERNEL) d->func = reinterpret_cast<const void *>(&KERNEL)
+#define TG_FUNC_D(KERNEL)                          \
+	switch (depth) {                               \
+		case 2: TG_FUNC(KERNEL<2>); break;         \
+		case 3: TG_FUNC(KERNEL<3>); break;         \
+		case 4: TG_FUNC(KERNEL<4>); break;         \
+		default: TG_FUNC(KERNEL<8>); break;        \
 	}
 	const int depth = tg_gemv_depth(g.K, g.C);
 	switch (role) {
-		case TG_ROLE_QKV_EMBED: TG_LAUNCH_D(tg_gemv_qkv_embed); break;
-		case TG_ROLE_QKV: TG_LAUNCH_D(tg_gemv_qkv); break;
-		case TG_ROLE_OPROJ: TG_LAUNCH_D(tg_gemv_oproj); break;
-		case TG_ROLE_UPGATE: TG_LAUNCH_D(tg_gemv_upgate_geglu); break;
-		case TG_ROLE_DOWN: TG_LAUNCH_D(tg_gemv_down); break;
-		case TG_ROLE_LMHEAD: TG_LAUNCH(tg_gemv_lmhead_argmax); break;
-		case TG_ROLE_LMHEAD_PLAIN: TG_LAUNCH(tg_gemv_lmhead_plain); break;
+		case TG_ROLE_QKV_EMBED: TG_FUNC_D(tg_gemv_qkv_embed); break;
+		case TG_ROLE_QKV: TG_FUNC_D(tg_gemv_qkv); break;
+		case TG_ROLE_OPROJ: TG_FUNC_D(tg_gemv_oproj); break;
+		case TG_ROLE_UPGATE: TG_FUNC_D(tg_gemv_upgate_geglu); break;
+		case TG_ROLE_DOWN: TG_FUNC_D(tg_gemv_down); break;
+		case TG_ROLE_LMHEAD: TG_FUNC(tg_gemv_lmhead_argmax); break;
+		case TG_ROLE_LMHEAD_PLAIN: TG_FUNC(tg_gemv_lmhead_plain); break;
 		default:
 			// a matrix of a quarter of the 256 MB memory-side cache or more is streamed as read-once data
-			if ((size_t)g.K * g.C * g.ntiles >= ((size_t)64 << 20)) TG_LAUNCH(tg_gemv_plain_stream);
-			else TG_LAUNCH_D(tg_gemv_plain);
+			if ((size_t)g.K * g.C * g.ntiles >= ((size_t)64 << 20)) TG_FUNC(tg_gemv_plain_stream);
+			else TG_FUNC_D(tg_gemv_plain);
 			break;
 	}
-#undef TG_LAUNCH_D
-#undef TG_LAUNCH
+#undef TG_FUNC_D
+#undef TG_FUNC
+}
+
+bool tg_gemv_is_oproj(const void *func) {
+	return func == reinterpret_cast<const void *>(&tg_gemv_oproj<2>) || func == reinterpret_cast<const void *>(&tg_gemv_oproj<3>) ||
+	       func == reinterpret_cast<const void *>(&tg_gemv_oproj<4>) || func == reinterpret_cast<const void *>(&tg_gemv_oproj<8>);
+}
+
+void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s) {
+	TgLaunchDesc d;
+	tg_desc_gemv(g, role, &d);
+	tg_launch_desc(d, s);
 }
 
 void tg_launch_argmax_finish(const float *blk_val, const int *blk_idx, int n, int *ctr, int *tok_log, int advance, hipStream_t s) {

@@ -151,6 +151,28 @@ struct TgAttnDecode {
 
 enum { TG_ROLE_PLAIN = 0, TG_ROLE_QKV_EMBED, TG_ROLE_QKV, TG_ROLE_OPROJ, TG_ROLE_UPGATE, TG_ROLE_DOWN, TG_ROLE_LMHEAD,
        TG_ROLE_LMHEAD_PLAIN };
+// A launch spelled out: kernel, geometry and the argument list in the form hipLaunchKernel and a graph's kernel node
+// take it.  The tg_desc_* functions fill one in place (`args` points into the descriptor itself: it is not copied
+// afterwards); tg_launch_* = describe + launch.  A replayed graph of a decode step has its position-dependent nodes
+// (attention, its merge, the output projection) re-described before every replay.
+struct TgLaunchDesc {
+	const void *func;
+	dim3 grid, block;
+	void *args[12];
+	const void *p[6];  // storage of pointer arguments
+	int i[6];          // ... of integer arguments
+	TgGemv g;          // ... of the descriptor a GEMV kernel takes by value
+	TgAttnDecode a;    // ... of the descriptor an attention kernel takes by value
+};
+void tg_desc_gemv(const TgGemv &g, int role, TgLaunchDesc *d);
+void tg_desc_attn_decode(const TgAttnDecode &a, int max_blocks, TgLaunchDesc *d);
+void tg_desc_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, TgLaunchDesc *d);
+// which of the position-dependent kernels of a decode step a kernel node's function is: 1 attention, 2 its merge, 3 the
+// output projection, 0 none of them
+int tg_decode_node_kind(const void *func);
+inline void tg_launch_desc(const TgLaunchDesc &d, hipStream_t s) {
+	(void)hipLaunchKernel(d.func, d.grid, d.block, const_cast<void **>(d.args), 0, s);
+}
 void tg_launch_gemv(const TgGemv &g, int role, hipStream_t s);
 void tg_launch_attn_decode(const TgAttnDecode &a, int max_blocks, hipStream_t s);
 void tg_launch_attn_merge(const TgAttnDecode &a, int nblk, float *merged_acc, float *merged_ml, hipStream_t s);
