@@ -615,7 +615,7 @@ def main():
             "prompt_tokens": n_prompt,
             "decode_position_start": n_prompt + args.warmup,
             "seed": args.seed,
-            "launch": "hipGraph replay" if args.graphs else "stream",
+            "launch": "hipGraph replay" if args.graphs else ("stream" if args.model == "1B" else "library default (updated hipGraph replay; stream launches under a profiler)"),
         },
         "roofline": {
             "kernel": "tg_gemv_lmhead_argmax",
