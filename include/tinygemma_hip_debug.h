@@ -16,12 +16,14 @@ extern "C" {
 /* device-to-device streaming copy kernel (bytes % 16 == 0), asynchronous: the known-size kernel
  * that hardware byte counters are calibrated against */
 int tg_dev_copy(void *dst_dev, const void *src_dev, size_t bytes);
-/* How tg_decode_enqueue issues greedy decode steps.  0 (default): plain stream launches.  1: replay of a captured step
+/* How tg_decode_enqueue issues greedy decode steps.  -1 (default): the library chooses, 2 for a model whose step
+ * streams under 5 MB of weights per launch (the 270m shape: the device would otherwise wait for the host's launches), 0
+ * for larger ones, and always 0 under a profiler.  0: plain stream launches.  1: replay of a captured step
  * whose kernels read the position from device memory and launch the largest grids their geometry can need.  2: replay
  * of a captured step of the stream path's own launches; the nodes that depend on the position (attention, its merge
  * launch, the output projection) get new parameters before every replay: one graph launch and 2-3 node updates per
  * layer on the host instead of 5-6 kernel launches.  Other values: TG_ERR_BAD_ARG.
- * Refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
+ * 1 and 2 are refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
  * replayed graphs ended the process.  Captured graphs are dropped whenever a tuning knob changes. */
 int tg_set_graphs(int enable);
 /* 1 (default): inside one tg_decode_enqueue call the first launch of a step also finishes the previous step's greedy
