@@ -323,6 +323,7 @@ struct tg_session {
 		std::vector<hipGraphNode_t> attn, merge, oproj;
 	};
 	std::map<uint64_t, PatchedGraph> pgraphs;
+	bool graphs_failed = false;  // the runtime refused a capture or a node update of mode 2: plain launches from then on
 	// min-p sampling (allocated on first use): scratch of the three sampler launches and the caller's uniform draws
 	float *probs = nullptr, *seg = nullptr, *bsum = nullptr, *bmax = nullptr, *randf = nullptr;
 	int randf_cap = 0;
@@ -1611,8 +1612,25 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 			// With chained picks the first step of a batch is a plain one (its first launch has no pick to finish); the
 			// steps behind it replay the chained form, whose pick stays pending for the next step or the flush below.
 			int rc;
-			if (g_chain_picks && !s->pick_pending) rc = enqueue_decode_step(s, nullptr, false, nullptr, true);
-			else rc = enqueue_patched_graph_step(s, g_chain_picks);
+			if (s->graphs_failed || (g_chain_picks && !s->pick_pending)) {
+				rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks);
+			} else {
+				// a capture or a node update the runtime refuses leaves nothing enqueued: the session's counters go back
+				// and this and all later steps of the session are plain launches
+				const int pos = s->pos, bpl = s->bp_local, bpg = s->bp_global, steps = s->steps;
+				const bool pending = s->pick_pending;
+				rc = enqueue_patched_graph_step(s, g_chain_picks);
+				if (rc == TG_ERR_HIP || (rc == TG_ERR_STATE && s->pos < c.n_pos && s->steps < s->tok_log_cap)) {
+					(void)hipGetLastError();
+					s->pos = pos;
+					s->bp_local = bpl;
+					s->bp_global = bpg;
+					s->steps = steps;
+					s->pick_pending = pending;
+					s->graphs_failed = true;
+					rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks);
+				}
+			}
 			if (rc != TG_OK) {
 				flush_pick(s);
 				return rc;
