@@ -162,6 +162,9 @@ int tg_debug_gemm_clock(float *C_dev, const float *A_dev, const tg_qweight *w, i
 int tg_plan_attention_prefill(int n_tokens, int n_cu, int window, int *query_tile, int32_t *items, int max_items, int *n_items,
                               int *n_split);
 int tg_plan_gemm_k_parts(int m, int in_dim, int out_dim, int n_cu);
+/* the form tg_decode_enqueue's greedy steps take for a model of this configuration under the current tg_set_graphs
+ * setting and environment: 0 stream launches, 1 or 2 the graph replays described there; -1: bad argument */
+int tg_plan_decode_launch_mode(const tg_config *cfg);
 
 
 

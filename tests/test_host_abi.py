@@ -190,6 +190,30 @@ def test_attention_work_list_covers_every_visible_key_exactly_once(pkg, S, windo
             assert span(lengths) <= 0.85 * span(plain)   # 527 items of up to 23 key tiles -> 492 of up to 25
 
 
+def test_decode_launch_mode_rule(pkg, monkeypatch):
+    """Left to the library, greedy steps of a model that streams under 5 MB of weights per launch (the 270m shape: 3.0 MB)
+    replay updated graphs, larger ones (the 1B shape: 7.7 MB) are stream launches; an explicit setting wins; under a
+    profiler the library's own choice is stream launches and graph replay is refused."""
+    lib = pkg.lib()
+    f = lib.tg_plan_decode_launch_mode
+    f.argtypes = [C.c_void_p]
+    small, big = pkg.named_config("270m"), pkg.named_config("1B")
+    assert lib.tg_set_graphs(-1) == 0
+    assert f(C.byref(small)) == 2 and f(C.byref(big)) == 0 and f(None) == -1
+    try:
+        for mode in (0, 1, 2):
+            assert lib.tg_set_graphs(mode) == 0
+            assert f(C.byref(small)) == mode and f(C.byref(big)) == mode
+        assert lib.tg_set_graphs(3) != 0 and lib.tg_set_graphs(-2) != 0
+        assert lib.tg_set_graphs(-1) == 0
+        monkeypatch.setenv("ROCP_TOOL_LIBRARIES", "librocprofiler-sdk-tool.so")
+        assert f(C.byref(small)) == 0 and f(C.byref(big)) == 0
+        assert lib.tg_set_graphs(2) != 0 and lib.tg_set_graphs(1) != 0 and lib.tg_set_graphs(0) == 0
+    finally:
+        monkeypatch.delenv("ROCP_TOOL_LIBRARIES", raising=False)
+        assert lib.tg_set_graphs(-1) == 0
+
+
 def test_gemm_k_parts_rule(pkg):
     f = pkg.lib().tg_plan_gemm_k_parts
     f.argtypes = [C.c_int] * 4

@@ -1580,13 +1580,18 @@ static bool profiler_attached();
 // 3 MB) than a host core that is slow or shared needs to issue one (2.5 us at best, 4.2-4.4 us on other cores of the same
 // machine), and the step would follow the host.  The 1B shape (7.7 MB, 4.6 us per launch) stays ahead of the host either
 // way and keeps its stream launches, which are 0.7 % faster there.  Never graphs under a profiler.
-static int decode_graph_mode(const tg_session *s) {
+static int decode_graph_mode_of(const tg_config &c) {
 	if (g_use_graphs >= 0) return g_use_graphs;
 	if (profiler_attached()) return 0;
-	const tg_config &c = s->m->cfg;
 	const double h = c.hidden_size, qo = (double)c.n_head * c.head_dim, kv = (double)c.n_kv * c.head_dim, f = c.intermediate_size;
 	const double bytes = c.n_layers * (h * (qo + 2 * kv) + qo * h + 3 * h * f) + h * c.n_vocab;
 	return bytes / (5.0 * c.n_layers + 1.0) < 5e6 ? 2 : 0;
+}
+static int decode_graph_mode(const tg_session *s) { return decode_graph_mode_of(s->m->cfg); }
+
+int tg_plan_decode_launch_mode(const tg_config *cfg) {
+	if (!cfg || cfg->n_layers < 1) return -1;
+	return decode_graph_mode_of(*cfg);
 }
 
 int tg_decode_enqueue(tg_session *s, int n_steps) {
