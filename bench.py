@@ -148,6 +148,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1024)
     ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--stream-launches", action="store_true", help="plain stream launches for the decode steps, whatever the library would choose for the model")
     ap.add_argument("--model", default="1B", choices=sorted(MODELS))
     ap.add_argument("--seed", type=int, default=20251)
     ap.add_argument("--cpu-steps", type=int, default=128, help="decode steps of the CPU baseline sample (0 = skip)")
@@ -176,7 +177,7 @@ def main():
     dev = tg.init(0)
     # the headline model's steps: stream launches unless --graphs; the library's own choice (-1) would be the same for the
     # 1B shape and updated-graph replay for the 270m shape (its section below runs both)
-    if tg.lib().tg_set_graphs(1 if args.graphs else (0 if args.model == "1B" else -1)) != 0:
+    if tg.lib().tg_set_graphs(1 if args.graphs else (0 if (args.model == "1B" or args.stream_launches) else -1)) != 0:
         print("bench.py: " + tg.lib().tg_last_error().decode(), file=sys.stderr)
         sys.exit(2)
     if args.prefetch_blocks is not None:
@@ -623,7 +624,7 @@ def main():
             "prompt_tokens": n_prompt,
             "decode_position_start": n_prompt + args.warmup,
             "seed": args.seed,
-            "launch": "hipGraph replay" if args.graphs else ("stream" if args.model == "1B" else "library default (updated hipGraph replay; stream launches under a profiler)"),
+            "launch": "hipGraph replay" if args.graphs else ("stream" if (args.model == "1B" or args.stream_launches) else "library default (updated hipGraph replay; stream launches under a profiler)"),
         },
         "roofline": {
             "kernel": "tg_gemv_lmhead_argmax",
