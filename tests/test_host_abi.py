@@ -190,6 +190,23 @@ def test_attention_work_list_covers_every_visible_key_exactly_once(pkg, S, windo
             assert span(lengths) <= 0.85 * span(plain)   # 527 items of up to 23 key tiles -> 492 of up to 25
 
 
+@pytest.mark.parametrize("S,n_cu", [(100, 1), (178, 2), (600, 3), (2100, 8), (4096, 16), (5000, 40)])
+def test_attention_work_list_on_few_compute_units(pkg, S, n_cu):
+    """The planner with far fewer compute units than query tiles (several rounds even for short prompts, chunks longer
+    than any key range): every key tile of every query tile still lies in exactly one item."""
+    tq, items, nsplit = attention_plan(pkg.lib(), S, n_cu, -1)
+    nq = (S + tq - 1) // tq
+    covered = {}
+    for qt, tb, te, slot in items:
+        covered.setdefault(int(qt), []).append((int(tb), int(te)))
+    if len(items) == 0:
+        return   # one workgroup per query tile over its whole range
+    for qt in range(nq):
+        chunks = sorted(covered[qt])
+        assert chunks[0][0] == 0 and all(a[1] == b[0] for a, b in zip(chunks, chunks[1:]))
+        assert chunks[-1][1] == (min(qt * tq + tq, S) + 31) // 32
+
+
 def test_decode_launch_mode_rule(pkg, monkeypatch):
     """Left to the library, greedy steps of a model that streams under 5 MB of weights per launch (the 270m shape: 3.0 MB)
     replay updated graphs, larger ones (the 1B shape: 7.7 MB) are stream launches; an explicit setting wins; under a

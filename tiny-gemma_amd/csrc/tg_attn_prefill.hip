@@ -1413,7 +1413,7 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 				for (int qt = 0; qt < nq; qt++) n += chunks_of(end_tile(qt) - first_tile(qt), c);
 				return n;
 			};
-			std::vector<int> count((size_t)longest + 1);  // items by length
+			std::vector<int> count((size_t)std::max(longest, chunk) + 1);  // items by length (a chunk may be longer than any key range)
 			auto span = [&](int c) {
 				std::fill(count.begin(), count.end(), 0);
 				long n = 0;
@@ -1426,7 +1426,7 @@ bool tg_attn_prefill_plan(int S, int n_cu, int tq, int window, std::vector<int4>
 				std::priority_queue<long, std::vector<long>, std::greater<long>> free_at;
 				for (int i = 0; i < n_cu; i++) free_at.push(0);
 				long end = 0;
-				for (int l = longest; l >= 1; l--)
+				for (int l = (int)count.size() - 1; l >= 1; l--)
 					for (int k = 0; k < count[(size_t)l]; k++) {
 						const long t = free_at.top() + 4 + l;
 						free_at.pop();
