@@ -19,6 +19,10 @@ Reported beside it: `gemv_lmhead_shape` (the plain GEMV entry point tg_qgemv_dev
 launched back to back in rotation over three copies of the matrix so that none is served from cache), `gemv_640x2048` (the bare matvec of the first benchmark configuration, warm and
 rotating over 512 MB of distinct copies) and `prefill.long_prompt` (a 4096-token prefill of the same
 model: the matrix-matrix path on the int8 matrix cores).
+`settle_ms` is the pause between the warm-up's synchronisation and the timed region (the host's first launches right
+behind a long wait are slow), `host_pace` the time the host needs to issue 32 steps against the time the device needs to
+run them, and `gemma3_270m` the 270m shape in the launch form the library chooses for it (a replayed graph whose
+position-dependent nodes are updated every step) with the same steps as stream launches beside it.
 `cpu_baseline` times the reference's single-threaded AVX2 path (oracle/_ref, built from the
 reference's own sources) — or, where that library is absent, the scalar C restatement — on
 this machine's host cores over a bounded sample of the same workload.
