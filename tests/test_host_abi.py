@@ -251,3 +251,13 @@ def test_gemm_k_parts_rule(pkg):
         assert f(1000, 6912, 1152, 256) == 2
     finally:
         assert pkg.lib().tg_set_gemm_lds(2) == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This path runs on one GPU: `bench.py --gpus N` with N above 1 says so and exits (no GPU needed for that)."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr or "--gpus 1" in r.stderr, r.stderr[-500:]
+    assert r.stdout.strip() == ""
