@@ -21,8 +21,8 @@ int tg_dev_copy(void *dst_dev, const void *src_dev, size_t bytes);
  * for larger ones, and always 0 under a profiler.  0: plain stream launches.  1: replay of a captured step
  * whose kernels read the position from device memory and launch the largest grids their geometry can need.  2: replay
  * of a captured step of the stream path's own launches; the nodes that depend on the position (attention, its merge
- * launch, the output projection) get new parameters before every replay: one graph launch and 2-3 node updates per
- * layer on the host instead of 5-6 kernel launches.  Other values: TG_ERR_BAD_ARG.
+ * launch, the output projection) get new parameters before every replay: 2-3 node updates per layer and step and one
+ * graph launch per four steps on the host instead of 5-6 kernel launches per layer and step.  Other values: TG_ERR_BAD_ARG.
  * 1 and 2 are refused with TG_ERR_STATE while a profiler's tool library is loaded (rocprofv3's environment): a kernel trace of
  * replayed graphs ended the process.  Captured graphs are dropped whenever a tuning knob changes. */
 int tg_set_graphs(int enable);

@@ -320,6 +320,7 @@ struct tg_session {
 	struct PatchedGraph {
 		hipGraph_t graph = nullptr;
 		hipGraphExec_t exec = nullptr;
+		int steps = 1;  // decode steps in the graph; the node lists are indexed step * layers + layer
 		std::vector<hipGraphNode_t> attn, merge, oproj;
 	};
 	std::map<uint64_t, PatchedGraph> pgraphs;
@@ -1462,20 +1463,29 @@ static void session_drop_graphs(tg_session *s) {
 // layer instead of 5-6 kernel launches: a decode step of the 270m shape, 91 launches of 3.6 us on the device, is bound
 // by the host's launch rate whenever the launching thread sits on a slow core (2.5 or 4.2 us per launch: 3,070 or
 // 2,500-2,600 tok/s from process to process).
-static uint64_t patched_graph_key(const tg_session *s, bool chained) {
+constexpr int TG_GRAPH_STEPS = 4;  // decode steps per replayed graph where a batch has that many left (a graph launch costs the device 5-6 us)
+
+// which layer kinds have a merge launch at the session's position + ahead
+static uint64_t patched_graph_topology(const tg_session *s, int ahead) {
 	const tg_config &c = s->m->cfg;
 	bool ml = false, mg = false;
-	(void)attn_chunk_for(std::min(s->pos + 1, c.n_pos_local), &ml);
-	(void)attn_chunk_for(std::min(s->pos + 1, c.n_pos), &mg);
-	return (uint64_t)ml | ((uint64_t)mg << 1) | ((uint64_t)chained << 2);
+	(void)attn_chunk_for(std::min(s->pos + ahead + 1, c.n_pos_local), &ml);
+	(void)attn_chunk_for(std::min(s->pos + ahead + 1, c.n_pos), &mg);
+	return (uint64_t)ml | ((uint64_t)mg << 1);
+}
+static uint64_t patched_graph_key(const tg_session *s, bool chained, int nsteps) {
+	return patched_graph_topology(s, 0) | ((uint64_t)chained << 2) | ((uint64_t)nsteps << 3);
 }
 
-// chained: the step's first launch finishes the previous step's greedy pick and its own pick stays pending (the caller
-// has a pick pending on entry and flushes after its last step); else the step ends with the finishing launch.
-static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bool chained) {
-	const int L = s->m->cfg.n_layers;
+// Captures nsteps consecutive steps.  chained: a step's first launch finishes the previous step's greedy pick and its
+// own pick stays pending (the caller has a pick pending on entry and flushes after its last step); else every step ends
+// with the finishing launch.
+static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bool chained, int nsteps) {
+	const int L = s->m->cfg.n_layers, pos0 = s->pos;
+	pg->steps = nsteps;
 	TG_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal));
-	const int rc = enqueue_decode_step(s, nullptr, false, nullptr, chained);  // advances the host mirrors once
+	int rc = TG_OK;
+	for (int k = 0; k < nsteps && rc == TG_OK; k++) rc = enqueue_decode_step(s, nullptr, false, nullptr, chained);  // advances the host mirrors
 	const hipError_t e = hipStreamEndCapture(g_stream, &pg->graph);
 	if (rc != TG_OK) return rc;
 	if (e != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipStreamEndCapture: ") + hipGetErrorString(e));
@@ -1483,9 +1493,9 @@ static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bo
 	TG_HIP(hipGraphGetNodes(pg->graph, nullptr, &n));
 	std::vector<hipGraphNode_t> nodes(n);
 	TG_HIP(hipGraphGetNodes(pg->graph, nodes.data(), &n));
-	pg->attn.assign((size_t)L, nullptr);
-	pg->merge.assign((size_t)L, nullptr);
-	pg->oproj.assign((size_t)L, nullptr);
+	pg->attn.assign((size_t)(nsteps * L), nullptr);
+	pg->merge.assign((size_t)(nsteps * L), nullptr);
+	pg->oproj.assign((size_t)(nsteps * L), nullptr);
 	for (hipGraphNode_t node : nodes) {
 		hipGraphNodeType type;
 		TG_HIP(hipGraphNodeGetType(node, &type));
@@ -1494,30 +1504,34 @@ static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bo
 		TG_HIP(hipGraphKernelNodeGetParams(node, &kp));
 		const int kind = tg_decode_node_kind(kp.func);
 		if (kind == 0 || kp.kernelParams == nullptr) continue;
-		// which layer: by the cache (attention, merge) or the weights (projection) the node's descriptor names
-		int layer = -1;
+		// which layer: by the cache (attention, merge) or the weights (projection) the node's descriptor names; which
+		// step: by the position it was captured with
+		int layer = -1, step = -1;
 		if (kind == 3) {
 			const TgGemv *g = static_cast<const TgGemv *>(kp.kernelParams[9]);
 			for (int l = 0; l < L; l++)
 				if (g->W == s->m->L[(size_t)l].o.W) layer = l;
+			step = g->host_pos - pos0;
 		} else {
 			const TgAttnDecode *a = static_cast<const TgAttnDecode *>(kp.kernelParams[kind == 1 ? 9 : 0]);
 			for (int l = 0; l < L; l++)
 				if (a->kc == s->kc[(size_t)l]) layer = l;
+			step = a->host_pos - pos0;
 		}
-		if (layer < 0) return tg_fail(TG_ERR_STATE, "graph replay: a captured node names no layer of this session");
+		if (layer < 0 || step < 0 || step >= nsteps) return tg_fail(TG_ERR_STATE, "graph replay: a captured node names no layer or step of this capture");
 		std::vector<hipGraphNode_t> &slot = kind == 1 ? pg->attn : (kind == 2 ? pg->merge : pg->oproj);
-		if (slot[(size_t)layer] != nullptr) return tg_fail(TG_ERR_STATE, "graph replay: two captured nodes for one launch");
-		slot[(size_t)layer] = node;
+		if (slot[(size_t)(step * L + layer)] != nullptr) return tg_fail(TG_ERR_STATE, "graph replay: two captured nodes for one launch");
+		slot[(size_t)(step * L + layer)] = node;
 	}
-	for (int l = 0; l < L; l++)
-		if (pg->attn[(size_t)l] == nullptr || pg->oproj[(size_t)l] == nullptr)
-			return tg_fail(TG_ERR_STATE, "graph replay: the captured step lacks a layer's attention or projection node");
+	for (int i = 0; i < nsteps * L; i++)
+		if (pg->attn[(size_t)i] == nullptr || pg->oproj[(size_t)i] == nullptr)
+			return tg_fail(TG_ERR_STATE, "graph replay: the captured steps lack a layer's attention or projection node");
 	const hipError_t e2 = hipGraphInstantiate(&pg->exec, pg->graph, nullptr, nullptr, 0);
 	if (e2 != hipSuccess) return tg_fail(TG_ERR_HIP, std::string("hipGraphInstantiate: ") + hipGetErrorString(e2));
 	return TG_OK;
 }
 
+// New parameters for the position-dependent nodes of every step of the graph; advances the host mirrors by its steps.
 static int patched_graph_update(tg_session *s, const tg_session::PatchedGraph &pg) {
 	const int L = s->m->cfg.n_layers;
 	TgLaunchDesc d;
@@ -1532,30 +1546,36 @@ static int patched_graph_update(tg_session *s, const tg_session::PatchedGraph &p
 		kp.extra = nullptr;
 		return hipGraphExecKernelNodeSetParams(pg.exec, node, &kp);
 	};
-	for (int l = 0; l < L; l++) {
-		const AttnGeom ag = attn_geometry(s, l, false);
-		tg_desc_attn_decode(ag.a, ag.nblk, &d);
-		TG_HIP(set(pg.attn[(size_t)l]));
-		if (ag.needs_merge != (pg.merge[(size_t)l] != nullptr)) return tg_fail(TG_ERR_STATE, "graph replay: the step's launches differ from the captured ones");
-		if (ag.needs_merge) {
-			tg_desc_attn_merge(ag.a, ag.nblk, s->merged_acc, s->merged_ml, &d);
-			TG_HIP(set(pg.merge[(size_t)l]));
+	for (int k = 0; k < pg.steps; k++) {
+		for (int l = 0; l < L; l++) {
+			const size_t at = (size_t)(k * L + l);
+			const AttnGeom ag = attn_geometry(s, l, false);
+			tg_desc_attn_decode(ag.a, ag.nblk, &d);
+			TG_HIP(set(pg.attn[at]));
+			if (ag.needs_merge != (pg.merge[at] != nullptr)) return tg_fail(TG_ERR_STATE, "graph replay: the step's launches differ from the captured ones");
+			if (ag.needs_merge) {
+				tg_desc_attn_merge(ag.a, ag.nblk, s->merged_acc, s->merged_ml, &d);
+				TG_HIP(set(pg.merge[at]));
+			}
+			tg_desc_gemv(oproj_gemv(s, l, ag), TG_ROLE_OPROJ, &d);
+			TG_HIP(set(pg.oproj[at]));
 		}
-		tg_desc_gemv(oproj_gemv(s, l, ag), TG_ROLE_OPROJ, &d);
-		TG_HIP(set(pg.oproj[(size_t)l]));
+		s->pos += 1;
+		s->bp_local += 1;
+		s->bp_global += 1;
+		s->steps += 1;
 	}
 	return TG_OK;
 }
 
-static int enqueue_patched_graph_step(tg_session *s, bool chained) {
-	const tg_config &c = s->m->cfg;
-	if (s->pos >= c.n_pos) return tg_fail(TG_ERR_STATE, "context is full (n_pos)");
-	if (s->steps >= s->tok_log_cap) return tg_fail(TG_ERR_STATE, "token log is full");
-	const uint64_t key = patched_graph_key(s, chained);
+// nsteps steps from one graph launch; the caller has checked that they fit the context and the token log and that all of
+// them have the launches of the first
+static int enqueue_patched_graph_steps(tg_session *s, bool chained, int nsteps) {
+	const uint64_t key = patched_graph_key(s, chained, nsteps);
 	auto it = s->pgraphs.find(key);
 	if (it == s->pgraphs.end()) {
 		tg_session::PatchedGraph pg;
-		const int rc = patched_graph_capture(s, &pg, chained);  // the captured step holds this position's parameters
+		const int rc = patched_graph_capture(s, &pg, chained, nsteps);  // the captured steps hold these positions' parameters
 		if (rc != TG_OK) {
 			if (pg.exec) (void)hipGraphExecDestroy(pg.exec);
 			if (pg.graph) (void)hipGraphDestroy(pg.graph);
@@ -1567,10 +1587,6 @@ static int enqueue_patched_graph_step(tg_session *s, bool chained) {
 	}
 	if (int rc = patched_graph_update(s, it->second)) return rc;
 	TG_HIP(hipGraphLaunch(it->second.exec, g_stream));
-	s->pos += 1;
-	s->bp_local += 1;
-	s->bp_global += 1;
-	s->steps += 1;
 	return TG_OK;
 }
 
@@ -1579,7 +1595,7 @@ static bool profiler_attached();
 // weights per launch replays updated graphs: the device then needs less time per launch (3.6 us for the 270m shape's
 // 3 MB) than a host core that is slow or shared needs to issue one (2.5 us at best, 4.2-4.4 us on other cores of the same
 // machine), and the step would follow the host.  The 1B shape (7.7 MB, 4.6 us per launch) stays ahead of the host either
-// way and keeps its stream launches, which are 0.7 % faster there.  Never graphs under a profiler.
+// way and keeps its stream launches (as fast there as the replay).  Never graphs under a profiler.
 static int decode_graph_mode_of(const tg_config &c) {
 	if (g_use_graphs >= 0) return g_use_graphs;
 	if (profiler_attached()) return 0;
@@ -1622,18 +1638,32 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 			} else {
 				// a capture or a node update the runtime refuses leaves nothing enqueued: the session's counters go back
 				// and this and all later steps of the session are plain launches
-				const int pos = s->pos, bpl = s->bp_local, bpg = s->bp_global, steps = s->steps;
-				const bool pending = s->pick_pending;
-				rc = enqueue_patched_graph_step(s, g_chain_picks);
-				if (rc == TG_ERR_HIP || (rc == TG_ERR_STATE && s->pos < c.n_pos && s->steps < s->tok_log_cap)) {
-					(void)hipGetLastError();
-					s->pos = pos;
-					s->bp_local = bpl;
-					s->bp_global = bpg;
-					s->steps = steps;
-					s->pick_pending = pending;
-					s->graphs_failed = true;
-					rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks);
+				if (s->pos >= c.n_pos) rc = tg_fail(TG_ERR_STATE, "context is full (n_pos)");
+				else if (s->steps >= s->tok_log_cap) rc = tg_fail(TG_ERR_STATE, "token log is full");
+				else {
+					// several steps per graph launch where the batch, the context and the token log have room for them and
+					// none of them changes which layers have a merge launch
+					int ns = 1;
+					if (n_steps - i >= TG_GRAPH_STEPS && s->pos + TG_GRAPH_STEPS <= c.n_pos && s->steps + TG_GRAPH_STEPS <= s->tok_log_cap) {
+						ns = TG_GRAPH_STEPS;
+						for (int k = 1; k < TG_GRAPH_STEPS; k++)
+							if (patched_graph_topology(s, k) != patched_graph_topology(s, 0)) ns = 1;
+					}
+					const int pos = s->pos, bpl = s->bp_local, bpg = s->bp_global, steps = s->steps;
+					const bool pending = s->pick_pending;
+					rc = enqueue_patched_graph_steps(s, g_chain_picks, ns);
+					if (rc == TG_OK) {
+						i += ns - 1;
+					} else if (rc == TG_ERR_HIP || rc == TG_ERR_STATE) {
+						(void)hipGetLastError();
+						s->pos = pos;
+						s->bp_local = bpl;
+						s->bp_global = bpg;
+						s->steps = steps;
+						s->pick_pending = pending;
+						s->graphs_failed = true;
+						rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks);
+					}
 				}
 			}
 			if (rc != TG_OK) {
