@@ -1463,7 +1463,8 @@ static void session_drop_graphs(tg_session *s) {
 // layer instead of 5-6 kernel launches: a decode step of the 270m shape, 91 launches of 3.6 us on the device, is bound
 // by the host's launch rate whenever the launching thread sits on a slow core (2.5 or 4.2 us per launch: 3,070 or
 // 2,500-2,600 tok/s from process to process).
-constexpr int TG_GRAPH_STEPS = 4;  // decode steps per replayed graph where a batch has that many left (a graph launch costs the device 5-6 us)
+constexpr int TG_GRAPH_STEPS = 4;  // decode steps per replayed graph where a batch has that many left (a graph launch costs the device 5-6 us;
+                                   // graphs of two and three steps for the tails would be further kinds to capture on first use)
 
 // which layer kinds have a merge launch at the session's position + ahead
 static uint64_t patched_graph_topology(const tg_session *s, int ahead) {
@@ -1473,13 +1474,15 @@ static uint64_t patched_graph_topology(const tg_session *s, int ahead) {
 	(void)attn_chunk_for(std::min(s->pos + ahead + 1, c.n_pos), &mg);
 	return (uint64_t)ml | ((uint64_t)mg << 1);
 }
+// A graph is one of: which layers merge, whether picks are chained, whether a pick is pending when its first step starts
+// (that step's first launch then finishes it; the first step of a batch has none), how many steps it holds.
 static uint64_t patched_graph_key(const tg_session *s, bool chained, int nsteps) {
-	return patched_graph_topology(s, 0) | ((uint64_t)chained << 2) | ((uint64_t)nsteps << 3);
+	return patched_graph_topology(s, 0) | ((uint64_t)chained << 2) | ((uint64_t)s->pick_pending << 3) | ((uint64_t)nsteps << 4);
 }
 
-// Captures nsteps consecutive steps.  chained: a step's first launch finishes the previous step's greedy pick and its
-// own pick stays pending (the caller has a pick pending on entry and flushes after its last step); else every step ends
-// with the finishing launch.
+// Captures nsteps consecutive steps.  chained: a step's first launch finishes the greedy pick that is pending when it
+// starts, if any, and its own pick stays pending (the caller flushes after its last step); else every step ends with
+// the finishing launch.
 static int patched_graph_capture(tg_session *s, tg_session::PatchedGraph *pg, bool chained, int nsteps) {
 	const int L = s->m->cfg.n_layers, pos0 = s->pos;
 	pg->steps = nsteps;
@@ -1587,6 +1590,7 @@ static int enqueue_patched_graph_steps(tg_session *s, bool chained, int nsteps) 
 	}
 	if (int rc = patched_graph_update(s, it->second)) return rc;
 	TG_HIP(hipGraphLaunch(it->second.exec, g_stream));
+	if (chained) s->pick_pending = true;  // as the captured steps left it: the last step's pick waits for the next step or the flush
 	return TG_OK;
 }
 
@@ -1630,10 +1634,10 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 			continue;
 		}
 		if (graph_mode == 2) {
-			// With chained picks the first step of a batch is a plain one (its first launch has no pick to finish); the
-			// steps behind it replay the chained form, whose pick stays pending for the next step or the flush below.
+			// With chained picks a step's pick stays pending for the next step or the flush below; the first step of a
+			// batch, which has no pick to finish, is a graph of its own kind.
 			int rc;
-			if (s->graphs_failed || (g_chain_picks && !s->pick_pending)) {
+			if (s->graphs_failed) {
 				rc = enqueue_decode_step(s, nullptr, false, nullptr, g_chain_picks);
 			} else {
 				// a capture or a node update the runtime refuses leaves nothing enqueued: the session's counters go back
@@ -1643,8 +1647,10 @@ int tg_decode_enqueue(tg_session *s, int n_steps) {
 				else {
 					// several steps per graph launch where the batch, the context and the token log have room for them and
 					// none of them changes which layers have a merge launch
+					// (the first step of a batch goes out alone: the device would otherwise wait until the host has updated the
+					// nodes of four steps, 0.4 ms, before it sees the first launch)
 					int ns = 1;
-					if (n_steps - i >= TG_GRAPH_STEPS && s->pos + TG_GRAPH_STEPS <= c.n_pos && s->steps + TG_GRAPH_STEPS <= s->tok_log_cap) {
+					if (i > 0 && n_steps - i >= TG_GRAPH_STEPS && s->pos + TG_GRAPH_STEPS <= c.n_pos && s->steps + TG_GRAPH_STEPS <= s->tok_log_cap) {
 						ns = TG_GRAPH_STEPS;
 						for (int k = 1; k < TG_GRAPH_STEPS; k++)
 							if (patched_graph_topology(s, k) != patched_graph_topology(s, 0)) ns = 1;
